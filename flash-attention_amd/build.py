@@ -1,0 +1,62 @@
+"""Builds libflash_attn_gfx950.so (the C-ABI attention library) with hipcc for gfx950.
+
+Usage:  python flash-attention_amd/build.py [-j JOBS]
+The translation units under csrc/ compile in parallel; objects go to build/ (git-ignored) and the
+shared library next to the Python package that loads it.
+"""
+import argparse
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ_DIR = os.path.join(HERE, "build")
+LIB_PATH = os.path.join(HERE, "flash_attn", "libflash_attn_gfx950.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    # packed fp32 VALU forms are switched off on purpose (build flags)
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-munsafe-fp-atomics",  # hardware global_atomic_add_f32 for the dQ accumulator
+    "-Wno-unused-result",
+]
+
+
+def sources():
+    return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
+
+
+def _compile(src):
+    obj = os.path.join(OBJ_DIR, src[:-4] + ".o")
+    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in r.stdout.splitlines() if "not a recognized feature" not in l)
+    return src, obj, r.returncode, out
+
+
+def build(jobs=8, verbose=False):
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    objs = []
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        for src, obj, rc, out in ex.map(_compile, sources()):
+            if rc != 0:
+                raise RuntimeError("hipcc failed on %s:\n%s" % (src, out))
+            if verbose and out.strip():
+                print(out)
+            objs.append(obj)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("link failed:\n" + r.stdout)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("-j", type=int, default=8)
+    ap.add_argument("-v", action="store_true")
+    a = ap.parse_args()
+    print(build(a.j, a.v))

@@ -1,0 +1,298 @@
+// C-ABI front end: argument validation, seqlen rounding, workspace layout and kernel dispatch.
+// Host-side counterpart of mha_fwd / mha_bwd / mha_fwd_block / mha_bwd_block
+// (csrc/flash_attn/fmha_api.cpp:173-718).  Every failed check returns a negative status and leaves a
+// message for fa_last_error(); nothing here synchronises the device or terminates the process.
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/flash_attn_gfx950.h"
+#include "fa_params.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define FA_REQUIRE(cond, ...) \
+  do {                        \
+    if (!(cond)) return fail(FA_ERR_INVALID_ARGUMENT, __VA_ARGS__); \
+  } while (0)
+
+#define FA_LAUNCH(expr)                                                                              \
+  do {                                                                                               \
+    hipError_t e_ = (expr);                                                                          \
+    if (e_ != hipSuccess) return fail(FA_ERR_LAUNCH, "%s failed: %s", #expr, hipGetErrorString(e_)); \
+  } while (0)
+
+inline size_t align16(size_t x) { return (x + 15) & ~(size_t)15; }
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+inline bool stride_ok(int64_t s) { return s % 8 == 0; }
+
+struct Rounded {
+  int sq_r, sk_r;
+};
+
+// fmha_api.cpp:232-241 (dense; blocksize_c taken for a device that is not sm80) and :509-514 (block-sparse)
+Rounded round_seqlens(int head_dim, int max_sq, int max_sk, bool blocksparse) {
+  Rounded r;
+  if (blocksparse) {
+    r.sk_r = ((max_sk + 255) / 256) * 256;
+    if (r.sk_r <= 256) r.sk_r = 256;
+  } else {
+    const int blocksize_c = head_dim == 128 ? 128 : 256;
+    r.sk_r = ((max_sk + blocksize_c - 1) / blocksize_c) * blocksize_c;
+    if (max_sk <= 128) r.sk_r = 128;
+    else if (max_sk <= 256) r.sk_r = 256;
+  }
+  r.sq_r = ((max_sq + 15) / 16) * 16;
+  return r;
+}
+
+struct SparseLayout {
+  int nrb, ncb, nqt, nqt2;
+  size_t off16, offq, offk, bytes;
+};
+
+SparseLayout sparse_layout(const Rounded& r) {
+  SparseLayout s;
+  s.nrb = r.sq_r / 16;
+  s.ncb = r.sk_r / 256;
+  s.nqt = (r.sq_r + fa::kFwdBM - 1) / fa::kFwdBM;
+  s.nqt2 = (r.sq_r + fa::kBwdBM - 1) / fa::kBwdBM;
+  s.off16 = 0;
+  s.offq = s.off16 + align16((size_t)s.nrb * s.ncb);
+  s.offk = s.offq + align16((size_t)s.nqt * s.ncb);
+  s.bytes = s.offk + align16((size_t)s.ncb * s.nqt2);
+  return s;
+}
+
+int build_maps(const int32_t* blockmask, unsigned char* ws, const SparseLayout& sl, fa::SparseMaps* out,
+               hipStream_t stream) {
+  FA_LAUNCH(fa::launch_fill_f32(reinterpret_cast<float*>(ws), sl.bytes / 4, 0.f, stream));
+  FA_LAUNCH(fa::launch_build_sparse_maps(blockmask, ws + sl.off16, ws + sl.offq, ws + sl.offk, sl.nrb, sl.ncb,
+                                         fa::kFwdBM, sl.nqt, fa::kBwdBM, sl.nqt2, stream));
+  out->act16 = ws + sl.off16;
+  out->actq = ws + sl.offq;
+  out->actk = ws + sl.offk;
+  out->nrb = sl.nrb;
+  out->ncb = sl.ncb;
+  out->nqt = sl.nqt;
+  out->nqt2 = sl.nqt2;
+  return FA_OK;
+}
+
+fa::PhiloxKey make_key(uint64_t seed, uint64_t offset) {
+  fa::PhiloxKey k;
+  k.k0 = (uint32_t)seed;
+  k.k1 = (uint32_t)(seed >> 32) ^ (uint32_t)(offset >> 32);
+  k.c3 = (uint32_t)offset;
+  return k;
+}
+
+int check_common(uint32_t struct_bytes, size_t expect, int dtype, int batch, int nheads, int head_dim, int total_q,
+                 int total_k, int max_sq, int max_sk, float p_dropout, float scale) {
+  FA_REQUIRE(struct_bytes == expect, "struct_bytes is %u, this library expects %zu (ABI mismatch)", struct_bytes, expect);
+  FA_REQUIRE(dtype == FA_FP16 || dtype == FA_BF16, "dtype must be fp16 or bf16");                  // fmha_api.cpp:198
+  FA_REQUIRE(batch > 0, "batch_size must be positive");                                            // :223
+  FA_REQUIRE(nheads > 0, "nheads must be positive");
+  FA_REQUIRE(head_dim == 16 || head_dim == 32 || head_dim == 64 || head_dim == 128,
+             "head_size must be 16, 32, 64 or 128 (got %d)", head_dim);                            // :224
+  FA_REQUIRE(total_q >= 0 && total_k >= 0, "negative token count");
+  FA_REQUIRE(max_sq > 0 && max_sk > 0, "max_seqlen must be positive");
+  FA_REQUIRE(p_dropout >= 0.f && p_dropout < 1.f, "p_dropout must be in [0, 1) (got %g)", p_dropout);  // :113
+  FA_REQUIRE(std::isfinite(scale) && scale > 0.f, "softmax_scale must be finite and positive (got %g)", scale);
+  return FA_OK;
+}
+
+int fwd_impl(const fa_fwd_args* a, bool want_block) {
+  if (!a) return fail(FA_ERR_INVALID_ARGUMENT, "args is NULL");
+  int rc = check_common(a->struct_bytes, sizeof(fa_fwd_args), a->dtype, a->batch, a->nheads, a->head_dim, a->total_q,
+                        a->total_k, a->max_seqlen_q, a->max_seqlen_k, a->p_dropout, a->softmax_scale);
+  if (rc) return rc;
+  const bool sparse = a->blockmask != nullptr;
+  FA_REQUIRE(sparse == want_block, want_block ? "fa_fwd_block needs a blockmask" : "fa_fwd takes no blockmask; call fa_fwd_block");
+  FA_REQUIRE(a->q && a->k && a->v && a->o && a->softmax_lse && a->cu_seqlens_q && a->cu_seqlens_k, "NULL tensor pointer");
+  FA_REQUIRE(aligned16(a->q) && aligned16(a->k) && aligned16(a->v) && aligned16(a->o),
+             "q, k, v, o must be 16-byte aligned");
+  FA_REQUIRE(stride_ok(a->q_row_stride) && stride_ok(a->q_head_stride) && stride_ok(a->k_row_stride) &&
+                 stride_ok(a->k_head_stride) && stride_ok(a->v_row_stride) && stride_ok(a->v_head_stride) &&
+                 stride_ok(a->o_row_stride) && stride_ok(a->o_head_stride),
+             "row and head strides must be multiples of 8 elements");
+  FA_REQUIRE(!(sparse && a->is_causal), "block-sparse attention does not support causal");  // interface.py:21
+
+  const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, sparse);
+  hipStream_t stream = reinterpret_cast<hipStream_t>(a->stream);
+  const bool dropout = a->p_dropout > 0.f;
+  const float p_keep = 1.f - a->p_dropout;
+
+  fa::FwdParams p;
+  memset(&p, 0, sizeof(p));
+  if (sparse) {
+    const SparseLayout sl = sparse_layout(r);
+    if (!a->workspace || a->workspace_bytes < sl.bytes)
+      return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", sl.bytes, a->workspace_bytes);
+    FA_REQUIRE(aligned16(a->workspace), "workspace must be 16-byte aligned");
+    rc = build_maps(a->blockmask, reinterpret_cast<unsigned char*>(a->workspace), sl, &p.sp, stream);
+    if (rc) return rc;
+  }
+  if (a->zero_tensors) {  // fmha_api.cpp:256-260
+    FA_LAUNCH(fa::launch_zero_rows(a->o, a->o_row_stride, a->o_head_stride, a->total_q, a->nheads, a->head_dim, stream));
+    FA_LAUNCH(fa::launch_fill_f32(a->softmax_lse, (size_t)a->batch * a->nheads * r.sq_r, -INFINITY, stream));
+  }
+
+  p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o; p.lse = a->softmax_lse;
+  p.cu_q = a->cu_seqlens_q; p.cu_k = a->cu_seqlens_k;
+  p.q_rs = a->q_row_stride; p.q_hs = a->q_head_stride;
+  p.k_rs = a->k_row_stride; p.k_hs = a->k_head_stride;
+  p.v_rs = a->v_row_stride; p.v_hs = a->v_head_stride;
+  p.o_rs = a->o_row_stride; p.o_hs = a->o_head_stride;
+  p.B = a->batch; p.H = a->nheads;
+  p.total_q = a->total_q; p.total_k = a->total_k;
+  p.max_sq = a->max_seqlen_q; p.max_sk = a->max_seqlen_k;
+  p.sq_r = r.sq_r;
+  p.nq_tiles = (a->max_seqlen_q + fa::kFwdBM - 1) / fa::kFwdBM;
+  p.total_tiles = p.nq_tiles * a->nheads * a->batch;
+  p.scale = a->softmax_scale;
+  p.scale_log2 = a->softmax_scale * fa::kLog2e;
+  p.rp_keep = 1.f / p_keep;
+  p.keep_thr = (uint32_t)std::floor(p_keep * 65535.0);  // fmha_api.cpp:110
+  p.pk = make_key(a->philox_seed, a->philox_offset);
+  FA_LAUNCH(fa::launch_fwd(p, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));
+
+  if (a->s_dmask) {
+    fa::DumpParams d;
+    memset(&d, 0, sizeof(d));
+    d.q = a->q; d.k = a->k; d.lse = a->softmax_lse; d.s = a->s_dmask;
+    d.cu_q = a->cu_seqlens_q; d.cu_k = a->cu_seqlens_k;
+    d.q_rs = a->q_row_stride; d.q_hs = a->q_head_stride; d.k_rs = a->k_row_stride; d.k_hs = a->k_head_stride;
+    d.B = a->batch; d.H = a->nheads; d.D = a->head_dim;
+    d.total_q = a->total_q; d.total_k = a->total_k;
+    d.max_sq = a->max_seqlen_q; d.max_sk = a->max_seqlen_k;
+    d.sq_r = r.sq_r; d.sk_r = r.sk_r;
+    d.scale = a->softmax_scale;
+    d.causal = a->is_causal != 0; d.dropout = dropout; d.sparse = sparse;
+    d.keep_thr = p.keep_thr; d.pk = p.pk; d.sp = p.sp;
+    FA_LAUNCH(fa::launch_dump_probs(d, a->dtype, stream));
+  }
+  return FA_OK;
+}
+
+int bwd_impl(const fa_bwd_args* a, bool want_block) {
+  if (!a) return fail(FA_ERR_INVALID_ARGUMENT, "args is NULL");
+  int rc = check_common(a->struct_bytes, sizeof(fa_bwd_args), a->dtype, a->batch, a->nheads, a->head_dim, a->total_q,
+                        a->total_k, a->max_seqlen_q, a->max_seqlen_k, a->p_dropout, a->softmax_scale);
+  if (rc) return rc;
+  const bool sparse = a->blockmask != nullptr;
+  FA_REQUIRE(sparse == want_block, want_block ? "fa_bwd_block needs a blockmask" : "fa_bwd takes no blockmask; call fa_bwd_block");
+  FA_REQUIRE(a->dout && a->q && a->k && a->v && a->out && a->softmax_lse && a->dq && a->dk && a->dv && a->softmax_d &&
+                 a->cu_seqlens_q && a->cu_seqlens_k, "NULL tensor pointer");
+  FA_REQUIRE(aligned16(a->dout) && aligned16(a->q) && aligned16(a->k) && aligned16(a->v) && aligned16(a->out) &&
+                 aligned16(a->dq) && aligned16(a->dk) && aligned16(a->dv), "tensors must be 16-byte aligned");
+  const int64_t strides[] = {a->do_row_stride, a->do_head_stride, a->q_row_stride,  a->q_head_stride,  a->k_row_stride,
+                             a->k_head_stride, a->v_row_stride,  a->v_head_stride, a->o_row_stride,  a->o_head_stride,
+                             a->dq_row_stride, a->dq_head_stride, a->dk_row_stride, a->dk_head_stride, a->dv_row_stride,
+                             a->dv_head_stride};
+  for (int64_t s : strides) FA_REQUIRE(stride_ok(s), "row and head strides must be multiples of 8 elements");
+  FA_REQUIRE(!(sparse && a->is_causal), "block-sparse attention does not support causal");
+
+  const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, sparse);
+  FA_REQUIRE(a->lse_seq_stride >= a->max_seqlen_q, "softmax_lse is shorter than max_seqlen_q");
+  hipStream_t stream = reinterpret_cast<hipStream_t>(a->stream);
+  const bool dropout = a->p_dropout > 0.f;
+  const float p_keep = 1.f - a->p_dropout;
+
+  const size_t dq_bytes = align16((size_t)a->total_q * a->nheads * a->head_dim * sizeof(float));
+  const SparseLayout sl = sparse_layout(r);
+  const size_t need = dq_bytes + (sparse ? sl.bytes : 0);
+  if (need > 0 && (!a->workspace || a->workspace_bytes < need))
+    return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, a->workspace_bytes);
+  FA_REQUIRE(need == 0 || aligned16(a->workspace), "workspace must be 16-byte aligned");
+  unsigned char* ws = reinterpret_cast<unsigned char*>(a->workspace);
+
+  fa::BwdParams p;
+  memset(&p, 0, sizeof(p));
+  if (sparse) {
+    rc = build_maps(a->blockmask, ws + dq_bytes, sl, &p.sp, stream);
+    if (rc) return rc;
+  }
+  if (a->zero_tensors) {  // fmha_api.cpp:406-411
+    FA_LAUNCH(fa::launch_zero_rows(a->dq, a->dq_row_stride, a->dq_head_stride, a->total_q, a->nheads, a->head_dim, stream));
+    FA_LAUNCH(fa::launch_zero_rows(a->dk, a->dk_row_stride, a->dk_head_stride, a->total_k, a->nheads, a->head_dim, stream));
+    FA_LAUNCH(fa::launch_zero_rows(a->dv, a->dv_row_stride, a->dv_head_stride, a->total_k, a->nheads, a->head_dim, stream));
+    FA_LAUNCH(fa::launch_fill_f32(a->softmax_d, (size_t)a->batch * a->nheads * r.sq_r, 0.f, stream));
+  }
+  p.dout = a->dout; p.q = a->q; p.k = a->k; p.v = a->v; p.out = a->out; p.lse = a->softmax_lse;
+  p.dsoftmax = a->softmax_d; p.dq_acc = reinterpret_cast<float*>(ws);
+  p.dq = a->dq; p.dk = a->dk; p.dv = a->dv;
+  p.cu_q = a->cu_seqlens_q; p.cu_k = a->cu_seqlens_k;
+  p.do_rs = a->do_row_stride; p.do_hs = a->do_head_stride;
+  p.q_rs = a->q_row_stride; p.q_hs = a->q_head_stride;
+  p.k_rs = a->k_row_stride; p.k_hs = a->k_head_stride;
+  p.v_rs = a->v_row_stride; p.v_hs = a->v_head_stride;
+  p.o_rs = a->o_row_stride; p.o_hs = a->o_head_stride;
+  p.dq_rs = a->dq_row_stride; p.dq_hs = a->dq_head_stride;
+  p.dk_rs = a->dk_row_stride; p.dk_hs = a->dk_head_stride;
+  p.dv_rs = a->dv_row_stride; p.dv_hs = a->dv_head_stride;
+  p.B = a->batch; p.H = a->nheads;
+  p.total_q = a->total_q; p.total_k = a->total_k;
+  p.max_sq = a->max_seqlen_q; p.max_sk = a->max_seqlen_k;
+  p.sq_r = r.sq_r; p.lse_stride = a->lse_seq_stride;
+  const int bn = fa::bwd_block_n(a->head_dim);
+  p.nk_tiles = (a->max_seqlen_k + bn - 1) / bn;
+  p.total_tiles = p.nk_tiles * a->nheads * a->batch;
+  p.scale = a->softmax_scale;
+  p.scale_log2 = a->softmax_scale * fa::kLog2e;
+  p.p_keep = p_keep;
+  p.rp_keep = 1.f / p_keep;
+  p.keep_thr = (uint32_t)std::floor(p_keep * 65535.0);
+  p.pk = make_key(a->philox_seed, a->philox_offset);
+
+  FA_LAUNCH(fa::launch_bwd_preprocess(p, a->dtype, a->head_dim, stream));
+  FA_LAUNCH(fa::launch_bwd(p, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));
+  FA_LAUNCH(fa::launch_bwd_postprocess(p, a->dtype, a->head_dim, stream));
+  return FA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int fa_fwd(const fa_fwd_args* args) { return fwd_impl(args, false); }
+int fa_fwd_block(const fa_fwd_args* args) { return fwd_impl(args, true); }
+int fa_bwd(const fa_bwd_args* args) { return bwd_impl(args, false); }
+int fa_bwd_block(const fa_bwd_args* args) { return bwd_impl(args, true); }
+
+size_t fa_fwd_workspace_bytes(const fa_fwd_args* a) {
+  if (!a || !a->blockmask) return 0;
+  return sparse_layout(round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, true)).bytes;
+}
+
+size_t fa_bwd_workspace_bytes(const fa_bwd_args* a) {
+  if (!a) return 0;
+  size_t n = align16((size_t)a->total_q * a->nheads * a->head_dim * sizeof(float));
+  if (a->blockmask) n += sparse_layout(round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, true)).bytes;
+  return n;
+}
+
+void fa_round_seqlens(int32_t head_dim, int32_t max_seqlen_q, int32_t max_seqlen_k, int32_t blocksparse,
+                      int32_t* max_seqlen_q_rounded, int32_t* max_seqlen_k_rounded) {
+  const Rounded r = round_seqlens(head_dim, max_seqlen_q, max_seqlen_k, blocksparse != 0);
+  if (max_seqlen_q_rounded) *max_seqlen_q_rounded = r.sq_r;
+  if (max_seqlen_k_rounded) *max_seqlen_k_rounded = r.sk_r;
+}
+
+uint64_t fa_philox_offset_increment(void) { return 4; }
+
+const char* fa_last_error(void) { return g_err; }
+int fa_abi_version(void) { return FA_ABI_VERSION; }
+
+}  // extern "C"

@@ -1,0 +1,207 @@
+// Small HBM-bound helper kernels around the two attention kernels: fills, the block-sparse activity
+// maps, the backward's rowsum(dO o O) pre-pass and dQ conversion post-pass, and the probability dump
+// behind return_softmax.
+#include "fa_params.h"
+
+namespace fa {
+
+namespace {
+
+__global__ void fill_f32_kernel(float* p, size_t n, float value) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) p[i] = value;
+}
+
+__global__ void zero_rows_kernel(uint16_t* base, int64_t rs, int64_t hs, int total, int H, int D) {
+  const int64_t n = (int64_t)total * H * (D / 8);
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) {
+    const int ch = (int)(i % (D / 8));
+    const int64_t rh = i / (D / 8);
+    const int h = (int)(rh % H);
+    const int64_t row = rh / H;
+    st_global16(base + row * rs + h * hs + ch * 8, u32x4{0, 0, 0, 0});
+  }
+}
+
+// blockmask: [ncb][nrb] int32, entries 4*rowblock + flags for the active 16-row blocks of each 256-key
+// column block, -1 padded (flash_blocksparse_attn_interface.py:8-40; read as fmha_blockmask.h:41-53 does).
+__global__ void sparse_maps_kernel(const int32_t* blockmask, uint8_t* act16, uint8_t* actq, uint8_t* actk, int nrb,
+                                   int ncb, int rpq, int nqt, int rpq2, int nqt2) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= nrb * ncb) return;
+  const int cb = i / nrb;
+  const int e = blockmask[i];
+  if (e < 0) return;
+  const int rb = e >> 2;
+  if (rb >= nrb) return;
+  act16[rb * ncb + cb] = 1;
+  if (rb / rpq < nqt) actq[(rb / rpq) * ncb + cb] = 1;
+  if (rb / rpq2 < nqt2) actk[cb * nqt2 + rb / rpq2] = 1;
+}
+
+template <typename T, int D>
+__global__ void __launch_bounds__(256) bwd_preprocess_kernel(const BwdParams p) {
+  constexpr int TPR = D / 8;         // threads per (row, head)
+  constexpr int RPB = 256 / TPR;     // (row, head) pairs per block
+  const int sub = threadIdx.x % TPR;
+  const int64_t rh = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
+  const int64_t n = (int64_t)p.total_q * p.H;
+  if (rh >= n) return;
+  const int h = (int)(rh % p.H);
+  const int64_t row = rh / p.H;
+  const T* dop = reinterpret_cast<const T*>(p.dout) + row * p.do_rs + (int64_t)h * p.do_hs + sub * 8;
+  const T* op = reinterpret_cast<const T*>(p.out) + row * p.o_rs + (int64_t)h * p.o_hs + sub * 8;
+  typedef typename Elem<T>::vec8 vec8;
+  const vec8 a = bitcast<vec8>(ld_global16(dop)), b = bitcast<vec8>(ld_global16(op));
+  float acc = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) acc += (float)a[i] * (float)b[i];
+#pragma unroll
+  for (int off = TPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+  float* dqa = p.dq_acc + rh * D + sub * 8;
+  *reinterpret_cast<f32x4*>(dqa) = f32x4{0.f, 0.f, 0.f, 0.f};
+  *reinterpret_cast<f32x4*>(dqa + 4) = f32x4{0.f, 0.f, 0.f, 0.f};
+  if (sub == 0) {
+    // locate (batch, position) of this row: binary search in cu_seqlens_q
+    int lo = 0, hi = p.B;
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (p.cu_q[mid] <= row) lo = mid; else hi = mid;
+    }
+    const int pos = (int)(row - p.cu_q[lo]);
+    if (pos >= 0 && pos < p.sq_r) p.dsoftmax[((int64_t)lo * p.H + h) * p.sq_r + pos] = acc * p.p_keep;
+  }
+}
+
+template <typename T, int D>
+__global__ void __launch_bounds__(256) bwd_postprocess_kernel(const BwdParams p) {
+  constexpr int TPR = D / 8;
+  constexpr int RPB = 256 / TPR;
+  const int sub = threadIdx.x % TPR;
+  const int64_t rh = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
+  const int64_t n = (int64_t)p.total_q * p.H;
+  if (rh >= n) return;
+  const int h = (int)(rh % p.H);
+  const int64_t row = rh / p.H;
+  const float* src = p.dq_acc + rh * D + sub * 8;
+  const f32x4 x0 = *reinterpret_cast<const f32x4*>(src), x1 = *reinterpret_cast<const f32x4*>(src + 4);
+  const float f = p.scale * p.rp_keep;
+  f32x8 y = {x0[0] * f, x0[1] * f, x0[2] * f, x0[3] * f, x1[0] * f, x1[1] * f, x1[2] * f, x1[3] * f};
+  T* dst = reinterpret_cast<T*>(p.dq) + row * p.dq_rs + (int64_t)h * p.dq_hs + sub * 8;
+  st_global16(dst, bitcast<u32x4>(cvt8<T>(y)));
+}
+
+// One thread per (query row, key) element of S_dmask.  Slow scalar dot products: this path exists for tests
+// (flash_attn_interface.py:163-173).  The value is the normalised probability exp(scale*s - lse); its sign
+// bit is set when dropout dropped the element.
+template <typename T>
+__global__ void __launch_bounds__(256) dump_probs_kernel(const DumpParams p) {
+  const int key = blockIdx.x * 256 + threadIdx.x;
+  const int qrow = blockIdx.y;
+  const int bh = blockIdx.z;
+  const int b = bh / p.H, h = bh % p.H;
+  int q_begin = 0, Lq = 0, k_begin = 0, Lk = 0;
+  if (!seq_extent(p.cu_q, b, p.total_q, p.max_sq, &q_begin, &Lq)) Lq = 0;
+  if (!seq_extent(p.cu_k, b, p.total_k, p.max_sk, &k_begin, &Lk)) Lk = 0;
+  if (key >= p.sk_r) return;
+  float val = 0.f;
+  bool dropped = false;
+  bool live = qrow < Lq && key < Lk;
+  if (p.causal && key > qrow) live = false;
+  if (live && p.sparse) {
+    const int rb = qrow >> 4, cb = key >> 8;
+    live = rb < p.sp.nrb && cb < p.sp.ncb && p.sp.act16[rb * p.sp.ncb + cb] != 0;
+  }
+  if (live) {
+    const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)(q_begin + qrow) * p.q_rs + (int64_t)h * p.q_hs;
+    const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)(k_begin + key) * p.k_rs + (int64_t)h * p.k_hs;
+    float s = 0.f;
+    for (int d = 0; d < p.D; d++) s += (float)qp[d] * (float)kp[d];
+    const float lse = p.lse[((int64_t)b * p.H + h) * p.sq_r + qrow];
+    val = __expf(s * p.scale - lse);
+    if (p.dropout) {
+      const uint32_t bits = dropout_keep_bits16(p.pk, (uint32_t)bh, (uint32_t)qrow >> 2, (uint32_t)key >> 2, p.keep_thr);
+      dropped = !((bits >> (4 * (qrow & 3) + (key & 3))) & 1u);
+    }
+  }
+  T out = (T)val;
+  if (dropped) out = -out;
+  reinterpret_cast<T*>(p.s)[(((int64_t)b * p.H + h) * p.sq_r + qrow) * p.sk_r + key] = out;
+}
+
+}  // namespace
+
+hipError_t launch_fill_f32(float* p, size_t n, float value, hipStream_t stream) {
+  if (n == 0) return hipSuccess;
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 65535) blocks = 65535;
+  hipLaunchKernelGGL(fill_f32_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, p, n, value);
+  return hipGetLastError();
+}
+
+hipError_t launch_zero_rows(void* base, int64_t row_stride, int64_t head_stride, int total, int H, int D,
+                            hipStream_t stream) {
+  const int64_t n = (int64_t)total * H * (D / 8);
+  if (n == 0) return hipSuccess;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 65535) blocks = 65535;
+  hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, stream,
+                     reinterpret_cast<uint16_t*>(base), row_stride, head_stride, total, H, D);
+  return hipGetLastError();
+}
+
+hipError_t launch_build_sparse_maps(const int32_t* blockmask, uint8_t* act16, uint8_t* actq, uint8_t* actk, int nrb,
+                                    int ncb, int rows_per_qt, int nqt, int rows_per_qt2, int nqt2,
+                                    hipStream_t stream) {
+  const int n = nrb * ncb;
+  hipLaunchKernelGGL(sparse_maps_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, blockmask, act16, actq, actk,
+                     nrb, ncb, rows_per_qt / 16, nqt, rows_per_qt2 / 16, nqt2);
+  return hipGetLastError();
+}
+
+namespace {
+template <typename T, int D>
+hipError_t pre_one(const BwdParams& p, hipStream_t stream) {
+  const int64_t n = (int64_t)p.total_q * p.H;
+  constexpr int RPB = 256 / (D / 8);
+  hipLaunchKernelGGL((bwd_preprocess_kernel<T, D>), dim3((unsigned)((n + RPB - 1) / RPB)), dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+template <typename T, int D>
+hipError_t post_one(const BwdParams& p, hipStream_t stream) {
+  const int64_t n = (int64_t)p.total_q * p.H;
+  constexpr int RPB = 256 / (D / 8);
+  hipLaunchKernelGGL((bwd_postprocess_kernel<T, D>), dim3((unsigned)((n + RPB - 1) / RPB)), dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+}  // namespace
+
+#define FA_DISPATCH_TD(fn)                                                          \
+  switch (head_dim) {                                                               \
+    case 16: return dtype == 0 ? fn<_Float16, 16>(p, stream) : fn<__bf16, 16>(p, stream);   \
+    case 32: return dtype == 0 ? fn<_Float16, 32>(p, stream) : fn<__bf16, 32>(p, stream);   \
+    case 64: return dtype == 0 ? fn<_Float16, 64>(p, stream) : fn<__bf16, 64>(p, stream);   \
+    case 128: return dtype == 0 ? fn<_Float16, 128>(p, stream) : fn<__bf16, 128>(p, stream); \
+    default: return hipErrorInvalidValue;                                           \
+  }
+
+hipError_t launch_bwd_preprocess(const BwdParams& p, int dtype, int head_dim, hipStream_t stream) {
+  if ((int64_t)p.total_q * p.H == 0) return hipSuccess;
+  FA_DISPATCH_TD(pre_one)
+}
+hipError_t launch_bwd_postprocess(const BwdParams& p, int dtype, int head_dim, hipStream_t stream) {
+  if ((int64_t)p.total_q * p.H == 0) return hipSuccess;
+  FA_DISPATCH_TD(post_one)
+}
+
+hipError_t launch_dump_probs(const DumpParams& p, int dtype, hipStream_t stream) {
+  dim3 grid((p.sk_r + 255) / 256, p.sq_r, p.B * p.H);
+  if (dtype == 0) hipLaunchKernelGGL(dump_probs_kernel<_Float16>, grid, dim3(256), 0, stream, p);
+  else hipLaunchKernelGGL(dump_probs_kernel<__bf16>, grid, dim3(256), 0, stream, p);
+  return hipGetLastError();
+}
+
+}  // namespace fa

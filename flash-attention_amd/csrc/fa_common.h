@@ -1,0 +1,160 @@
+// Shared device-side building blocks of the gfx950 attention kernels: vector types, MFMA wrappers,
+// LDS transposed reads, half-wave exchange, Philox dropout bits.
+//
+// MFMA register layouts used throughout (wave64, v_mfma_f32_32x32x16_{f16,bf16}):
+//   A operand: lane l holds row (l % 32), contraction indices 8*(l / 32) .. +7
+//   B operand: lane l holds column (l % 32), contraction indices 8*(l / 32) .. +7
+//   C/D:       lane l holds column (l % 32); register r (0..15) holds row 8*(r/4) + 4*(l/32) + r%4
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fa {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+
+#define FA_DEVICE __device__ __forceinline__
+#define FA_LDS __attribute__((address_space(3)))
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+template <typename T>
+struct Elem;
+
+template <>
+struct Elem<_Float16> {
+  typedef f16x8 vec8;
+  typedef f16x4 vec4;
+  static FA_DEVICE f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  static FA_DEVICE f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <>
+struct Elem<__bf16> {
+  typedef bf16x8 vec8;
+  typedef bf16x4 vec4;
+  static FA_DEVICE f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static FA_DEVICE f32x4 mfma16(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <typename To, typename From>
+FA_DEVICE To bitcast(const From& x) {
+  static_assert(sizeof(To) == sizeof(From), "bitcast size");
+  return __builtin_bit_cast(To, x);
+}
+
+// Round 8 floats to the 16-bit element type (round-to-nearest-even, v_cvt_pk_*).
+template <typename T>
+FA_DEVICE typename Elem<T>::vec8 cvt8(f32x8 x) {
+  return __builtin_convertvector(x, typename Elem<T>::vec8);
+}
+template <typename T>
+FA_DEVICE typename Elem<T>::vec4 cvt4(f32x4 x) {
+  return __builtin_convertvector(x, typename Elem<T>::vec4);
+}
+
+FA_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+FA_DEVICE float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+FA_DEVICE float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// Values of the two lanes l and l^32 (the two halves of a wave that share an MFMA column).
+// v_permlane32_swap with both operands equal returns (lower half's value, upper half's value) in
+// every lane, so symmetric reductions need no lane select.
+FA_DEVICE float half_max(float x) {
+  uint32_t u = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+FA_DEVICE float half_sum(float x) {
+  uint32_t u = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// 16-byte global load/store helpers.
+FA_DEVICE u32x4 ld_global16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+FA_DEVICE void st_global16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
+
+// ds_read_b64_tr_b16: within each group of 16 lanes, lane j supplies the address of 4 consecutive
+// 16-bit elements M[j][0..3]; lane i receives { M[4e + i/4][i%4] : e = 0..3 }.  With lane j pointing
+// at row (j/4), columns 4*(j%4).. of a row-major [k][n] tile, lane i ends up with column i of rows
+// 0..3, i.e. a k-contiguous MFMA operand fragment read from an n-contiguous tile.
+FA_DEVICE u32x2 lds_read_tr16(const void* lds_ptr) {
+  i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((FA_LDS i16x4*)(lds_ptr));
+  return bitcast<u32x2>(v);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Dropout.  The keep/drop decision of score element (b, h, q, key) is a pure function of
+// (seed, offset, b*H+h, q, key), so forward, backward and the probability dump agree whatever
+// their tiling.  Philox-4x32 with 7 rounds (the round function and count of the reference's
+// philox.cuh:35-42,121-135).  One 4x4 micro-block of the score matrix (rows 4*Q4.., keys 4*K4..)
+// draws two Philox outputs (call 0: rows 0,1; call 1: rows 2,3 of the micro-block); element
+// (q%4, key%4) uses 16-bit field  hw = 4*(q%4) + key%4  of the 16 fields, field f being bits
+// 16*(f%2).. of word (f/2)%4 of call f/8.  keep  <=>  field <= keep_threshold
+// (threshold = floor(keep_prob * 65535), fmha_api.cpp:110).
+// ---------------------------------------------------------------------------------------------
+struct PhiloxKey {
+  uint32_t k0, k1;  // seed_lo, seed_hi ^ offset_hi
+  uint32_t c3;      // offset_lo
+};
+
+FA_DEVICE u32x4 philox4x32_7(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int i = 0; i < 7; i++) {
+    uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+    uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    uint32_t n1 = (uint32_t)p1;
+    uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    uint32_t n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  u32x4 r = {c0, c1, c2, c3};
+  return r;
+}
+
+// 16 keep bits of micro-block (Q4, K4): bit (4*(q%4) + key%4) set <=> keep.
+FA_DEVICE uint32_t dropout_keep_bits16(const PhiloxKey& pk, uint32_t bh, uint32_t Q4, uint32_t K4, uint32_t thr) {
+  uint32_t bits = 0;
+#pragma unroll
+  for (int call = 0; call < 2; call++) {
+    u32x4 r = philox4x32_7((K4 << 1) | call, Q4, bh, pk.c3, pk.k0, pk.k1);
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+      uint32_t lo = r[w] & 0xffffu, hi = r[w] >> 16;
+      bits |= (lo <= thr ? 1u : 0u) << (call * 8 + w * 2);
+      bits |= (hi <= thr ? 1u : 0u) << (call * 8 + w * 2 + 1);
+    }
+  }
+  return bits;
+}
+
+// Broadcast lane (4*(lane/4) + j)'s value to the 4 lanes of its quad.
+template <int J>
+FA_DEVICE uint32_t quad_bcast(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_mov_dpp((int)x, J | (J << 2) | (J << 4) | (J << 6), 0xf, 0xf, true);
+}
+
+}  // namespace fa

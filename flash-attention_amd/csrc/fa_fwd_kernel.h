@@ -1,0 +1,304 @@
+// Forward attention kernel for gfx950.
+//
+// Computes what the reference's device_1xN_loop does (csrc/flash_attn/src/fmha_fprop_kernel_1xN.h:199-671):
+// O = dropout(softmax(scale * Q K^T + mask)) V and lse = logsumexp(scale * Q K^T + mask), but organised
+// query-tile-outer: one workgroup owns 128 query rows of one (batch, head), keeps the output accumulator
+// and the running (max, sum) in registers, streams K/V tiles through LDS, and writes o and lse once.
+// There is no fp32 o_tmp round trip through global memory.
+//
+// Everything is computed transposed so that one lane owns one query row:
+//   S^T = K Q^T   (A = K tile from LDS, B = Q fragment held in registers), C layout: lane -> query
+//                 column l%32, registers -> 16 keys.  Row max / row sum are in-lane plus ONE exchange with lane l^32.
+//   O^T = V^T P^T (A = V^T read from the row-major V tile with ds_read_b64_tr_b16, B = P^T taken straight from the
+//                 S^T accumulator registers, rounded to fp16/bf16).  The contraction runs over keys in the order the
+//                 accumulator registers hold them; the V^T fragment is fetched in the same order.
+#pragma once
+
+#include "fa_common.h"
+#include "fa_params.h"
+
+namespace fa {
+
+template <typename T, int D, int BN>
+struct FwdCfg {
+  static constexpr int BM = kFwdBM;
+  static constexpr int NW = 4;                 // waves per workgroup, 32 query rows each
+  static constexpr int DV = D < 32 ? 32 : D;   // V tile width in LDS (zero padded for D = 16)
+  static constexpr int KS = D + 8;             // K row stride in LDS, elements
+  static constexpr int VS = DV + 8;            // V row stride in LDS, elements
+  static constexpr int OS = D + 8;             // epilogue staging row stride
+  static constexpr int kTileBytes = BN * (KS + VS) * 2;
+  static constexpr int kEpiBytes = BM * OS * 2;
+  static constexpr int kLdsBytes = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
+  static constexpr int CH = D / 8;                              // 16-byte chunks per row
+  static constexpr int CPT = (BN * CH + 255) / 256;             // chunks per thread per tile
+};
+
+template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse>
+__global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
+  using Cfg = FwdCfg<T, D, BN>;
+  using E = Elem<T>;
+  using vec8 = typename E::vec8;
+  constexpr int BM = Cfg::BM, DV = Cfg::DV, KS = Cfg::KS, VS = Cfg::VS, CH = Cfg::CH, CPT = Cfg::CPT;
+
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
+  T* Ks = reinterpret_cast<T*>(lds_raw);
+  T* Vs = Ks + BN * KS;
+
+  // Workgroup -> (batch, head, query tile).  Consecutive workgroup ids go to different XCDs, so the
+  // id is re-mapped to give every XCD a contiguous range of tiles: all query tiles of one (batch, head)
+  // then share that XCD's L2 copy of K and V.
+  const int per_xcd = (p.total_tiles + 7) >> 3;
+  const int vid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (vid >= p.total_tiles) return;
+  const int bh = vid / p.nq_tiles;
+  // heaviest (last) query tiles first under a causal mask
+  const int qt = kCausal ? (p.nq_tiles - 1 - vid % p.nq_tiles) : (vid % p.nq_tiles);
+  const int b = bh / p.H, h = bh % p.H;
+
+  int q_begin, Lq, k_begin = 0, Lk = 0;
+  if (!seq_extent(p.cu_q, b, p.total_q, p.max_sq, &q_begin, &Lq)) return;
+  if (!seq_extent(p.cu_k, b, p.total_k, p.max_sk, &k_begin, &Lk)) Lk = 0;  // no keys: o = 0, lse = -inf
+  const int m0 = qt * BM;
+  if (m0 >= Lq) return;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 31, hf = lane >> 5;
+  const int mw = m0 + wave * 32;  // first query row of this wave
+  const int qrow = mw + c;        // this lane's query row (sequence-local)
+
+  // ---- Q fragment (B operand of S^T = K Q^T), held in registers for the whole kernel
+  vec8 qreg[D / 16];
+  {
+    const int qr = qrow < Lq ? qrow : Lq - 1;
+    const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)(q_begin + qr) * p.q_rs + (int64_t)h * p.q_hs + hf * 8;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ks++) {
+      u32x4 raw = ld_global16(qp + ks * 16);
+      if (qrow >= Lq) raw = u32x4{0, 0, 0, 0};
+      qreg[ks] = bitcast<vec8>(raw);
+    }
+  }
+
+  if (D < 32) {  // zero the padding columns of the V tile once
+    for (int i = tid; i < BN * (DV - D); i += 256) Vs[(i / (DV - D)) * VS + D + i % (DV - D)] = (T)0.f;
+  }
+
+  int n_end = Lk;
+  if (kCausal) n_end = n_end < m0 + BM ? n_end : m0 + BM;
+  const int ntiles = (n_end + BN - 1) / BN;
+
+  const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)k_begin * p.k_rs + (int64_t)h * p.k_hs;
+  const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)k_begin * p.v_rs + (int64_t)h * p.v_hs;
+
+  u32x4 kpre[CPT], vpre[CPT];
+  auto prefetch = [&](int it) {
+    const int n0 = it * BN;
+#pragma unroll
+    for (int i = 0; i < CPT; i++) {
+      const int ch = tid + i * 256;
+      const int row = ch / CH, col = (ch % CH) * 8;
+      const int key = n0 + row;
+      if ((BN * CH % 256 == 0 || ch < BN * CH) && key < Lk) {
+        kpre[i] = ld_global16(kbase + (int64_t)key * p.k_rs + col);
+        vpre[i] = ld_global16(vbase + (int64_t)key * p.v_rs + col);
+      } else {
+        kpre[i] = u32x4{0, 0, 0, 0};
+        vpre[i] = u32x4{0, 0, 0, 0};
+      }
+    }
+  };
+  auto commit = [&]() {
+#pragma unroll
+    for (int i = 0; i < CPT; i++) {
+      const int ch = tid + i * 256;
+      const int row = ch / CH, col = (ch % CH) * 8;
+      if (BN * CH % 256 == 0 || ch < BN * CH) {
+        *reinterpret_cast<u32x4*>(Ks + row * KS + col) = kpre[i];
+        *reinterpret_cast<u32x4*>(Vs + row * VS + col) = vpre[i];
+      }
+    }
+  };
+
+  // Sparse: tile `it` is computed iff its 256-key block is active for any 16-row block of this query tile.
+  auto tile_active = [&](int it) -> bool {
+    if (!kSparse) return true;
+    const int cb = (it * BN) >> 8;
+    return p.sp.actq[qt * p.sp.ncb + cb] != 0;
+  };
+  auto next_active = [&](int it) -> int {
+    while (it < ntiles && !tile_active(it)) it++;
+    return it;
+  };
+
+  f32x16 o_acc[DV / 32];
+#pragma unroll
+  for (int i = 0; i < DV / 32; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) o_acc[i][r] = 0.f;
+  float m_i = -INFINITY;  // running row max of raw scores (before scaling)
+  float l_i = 0.f;        // this lane's share of the running row sum (other share in lane^32)
+
+  const float cs = p.scale_log2;
+  // operand addressing of the transposed V reads (see lds_read_tr16)
+  const int j16 = lane & 15, g16 = lane >> 4;
+  const int vtr_off = (4 * hf + (j16 >> 2)) * VS + 16 * (g16 & 1) + 4 * (j16 & 3);
+
+  int it = next_active(0);
+  if (it < ntiles) prefetch(it);
+  while (it < ntiles) {
+    const int n0 = it * BN;
+    __syncthreads();  // everyone is done reading the previous tile
+    commit();
+    __syncthreads();
+    const int it_next = next_active(it + 1);
+    if (it_next < ntiles) prefetch(it_next);
+
+    bool wave_work = true;
+    if (kCausal && n0 > mw + 31) wave_work = false;  // every key of this tile is above the wave's diagonal
+    bool row_on = true;
+    if (kSparse) {
+      const int rb = (qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1;
+      row_on = p.sp.act16[rb * p.sp.ncb + (n0 >> 8)] != 0;
+      if (__ballot(row_on) == 0) wave_work = false;
+    }
+
+    if (wave_work) {
+      // ---- S^T = K Q^T
+      f32x16 s[BN / 32];
+#pragma unroll
+      for (int kb = 0; kb < BN / 32; kb++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[kb][r] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ks++) {
+          vec8 a = *reinterpret_cast<const vec8*>(Ks + (kb * 32 + c) * KS + ks * 16 + hf * 8);
+          s[kb] = E::mfma32(a, qreg[ks], s[kb]);
+        }
+      }
+      // ---- mask (only tiles that straddle the key length, the diagonal, or an inactive row block)
+      const bool need_mask = (n0 + BN > Lk) || (kCausal && (n0 + BN - 1 > mw)) || (kSparse && !row_on);
+      if (need_mask) {
+#pragma unroll
+        for (int kb = 0; kb < BN / 32; kb++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int key = n0 + kb * 32 + (r >> 2) * 8 + hf * 4 + (r & 3);
+            bool dead = key >= Lk;
+            if (kCausal) dead = dead || key > qrow;
+            if (kSparse) dead = dead || !row_on;
+            if (dead) s[kb][r] = -INFINITY;
+          }
+      }
+      // ---- online softmax (fmha_fprop_kernel_1xN.h:408-454,560-611 restated for a register-resident row)
+      float mt = s[0][0];
+#pragma unroll
+      for (int kb = 0; kb < BN / 32; kb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) mt = fmaxf(mt, s[kb][r]);
+      mt = half_max(mt);
+      const float m_new = fmaxf(m_i, mt);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float mc = m_use * cs;
+      const float alpha = fast_exp2(m_i * cs - mc);
+      m_i = m_new;
+      float rs = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < BN / 32; kb++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const float pe = fast_exp2(__builtin_fmaf(s[kb][r], cs, -mc));
+          s[kb][r] = pe;
+          rs += pe;
+        }
+      l_i = l_i * alpha + rs;  // the sum uses P before dropout (fmha_fprop_kernel_1xN.h:454 vs :471)
+#pragma unroll
+      for (int i = 0; i < DV / 32; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o_acc[i][r] *= alpha;
+
+      if (kDropout) {
+        const uint32_t bhu = (uint32_t)bh;
+        const uint32_t Q4 = (uint32_t)qrow >> 2;
+        const int t = c & 3;
+#pragma unroll
+        for (int kb = 0; kb < BN / 32; kb++) {
+          const uint32_t K4 = ((uint32_t)(n0 + kb * 32) >> 2) + 2 * t + hf;
+          const uint32_t mine = dropout_keep_bits16(p.pk, bhu, Q4, K4, p.keep_thr);
+          uint32_t bj[4];
+          bj[0] = quad_bcast<0>(mine);
+          bj[1] = quad_bcast<1>(mine);
+          bj[2] = quad_bcast<2>(mine);
+          bj[3] = quad_bcast<3>(mine);
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            const uint32_t rowbits = bj[j] >> (4 * t);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+              if (!((rowbits >> i) & 1u)) s[kb][4 * j + i] = 0.f;
+          }
+        }
+      }
+
+      // ---- O^T += V^T P^T
+#pragma unroll
+      for (int kb = 0; kb < BN / 32; kb++) {
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+          f32x8 pf;
+#pragma unroll
+          for (int i = 0; i < 8; i++) pf[i] = s[kb][8 * t + i];
+          const vec8 pb = cvt8<T>(pf);
+#pragma unroll
+          for (int db = 0; db < DV / 32; db++) {
+            const T* vp = Vs + (kb * 32 + 16 * t) * VS + db * 32 + vtr_off;
+            u32x2 lo = lds_read_tr16(vp);
+            u32x2 hi = lds_read_tr16(vp + 8 * VS);
+            u32x4 av = {lo[0], lo[1], hi[0], hi[1]};
+            o_acc[db] = E::mfma32(bitcast<vec8>(av), pb, o_acc[db]);
+          }
+        }
+      }
+    }
+    it = it_next;
+  }
+
+  // ---- epilogue: normalise, write lse, transpose O^T through LDS for coalesced 16-byte stores
+  const float l_tot = half_sum(l_i);
+  const bool empty = !(l_tot > 0.f);  // also catches NaN (fmha_fprop_kernel_1xN.h:575,606)
+  float inv = empty ? 1.f : fast_rcp(l_tot);
+  if (kDropout) inv *= p.rp_keep;
+  if (hf == 0 && qrow < Lq) {
+    const float lse = empty ? -INFINITY : (m_i * cs + fast_log2(l_tot)) * kLn2;
+    p.lse[((int64_t)b * p.H + h) * p.sq_r + qrow] = lse;
+  }
+  __syncthreads();
+  constexpr int OS = Cfg::OS;
+  T* Os = reinterpret_cast<T*>(lds_raw) + wave * 32 * OS;
+#pragma unroll
+  for (int db = 0; db < DV / 32; db++)
+#pragma unroll
+    for (int g4 = 0; g4 < 4; g4++) {
+      const int d0 = db * 32 + g4 * 8 + hf * 4;
+      if (d0 < D) {
+        f32x4 x;
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] = o_acc[db][g4 * 4 + i] * inv;
+        *reinterpret_cast<typename E::vec4*>(Os + c * OS + d0) = cvt4<T>(x);
+      }
+    }
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's LDS writes have landed
+  __builtin_amdgcn_wave_barrier();
+  T* obase = reinterpret_cast<T*>(p.o) + (int64_t)q_begin * p.o_rs + (int64_t)h * p.o_hs;
+#pragma unroll
+  for (int i = 0; i < (32 * CH + 63) / 64; i++) {
+    const int ch = lane + i * 64;
+    const int row = ch / CH, col = (ch % CH) * 8;
+    if ((32 * CH % 64 == 0 || ch < 32 * CH) && mw + row < Lq) {
+      u32x4 val = *reinterpret_cast<const u32x4*>(Os + row * OS + col);
+      st_global16(obase + (int64_t)(mw + row) * p.o_rs + col, val);
+    }
+  }
+}
+
+}  // namespace fa

@@ -1,0 +1,134 @@
+// Kernel parameter blocks (passed by value to the kernels) and launcher entry points shared
+// between the C-ABI front end and the kernel translation units.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fa_common.h"
+
+namespace fa {
+
+// Block-sparse activity maps, built on the device from the reference's converted block list
+// (flash_blocksparse_attn_interface.py:8-40) by build_sparse_maps():
+//   act16[rb * ncb + cb]  != 0  <=> the 16-row x 256-key block (rb, cb) is computed
+//   actq [qt * ncb + cb]  != 0  <=> any 16-row block of forward query tile qt is active in cb
+//   actk [cb * nqt2 + qt2] != 0 <=> any 16-row block of backward query tile qt2 is active in cb
+struct SparseMaps {
+  const uint8_t* act16;
+  const uint8_t* actq;
+  const uint8_t* actk;
+  int nrb;   // 16-row blocks  (= max_seqlen_q_rounded / 16)
+  int ncb;   // 256-key blocks (= max_seqlen_k_rounded / 256)
+  int nqt;   // forward query tiles
+  int nqt2;  // backward query tiles
+};
+
+struct FwdParams {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* o;
+  float* lse;
+  const int32_t* cu_q;
+  const int32_t* cu_k;
+  int64_t q_rs, q_hs, k_rs, k_hs, v_rs, v_hs, o_rs, o_hs;  // strides in elements
+  int B, H;
+  int total_q, total_k;
+  int max_sq, max_sk;  // caller's bounds on the sequence lengths; longer sequences are truncated to them
+  int sq_r;  // rounded max_seqlen_q = innermost extent of lse
+  int nq_tiles;
+  int total_tiles;  // nq_tiles * H * B
+  float scale;       // softmax_scale
+  float scale_log2;  // softmax_scale * log2(e)
+  float rp_keep;     // 1 / keep probability
+  uint32_t keep_thr; // floor(keep * 65535)
+  PhiloxKey pk;
+  SparseMaps sp;
+};
+
+struct DumpParams {  // return_softmax path
+  const void* q;
+  const void* k;
+  const float* lse;
+  void* s;  // [B, H, sq_r, sk_r]
+  const int32_t* cu_q;
+  const int32_t* cu_k;
+  int64_t q_rs, q_hs, k_rs, k_hs;
+  int B, H, D;
+  int total_q, total_k;
+  int max_sq, max_sk;
+  int sq_r, sk_r;
+  float scale;
+  int causal, dropout, sparse;
+  uint32_t keep_thr;
+  PhiloxKey pk;
+  SparseMaps sp;
+};
+
+struct BwdParams {
+  const void* dout;
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* out;
+  const float* lse;
+  float* dsoftmax;  // softmax_d [B, H, sq_r]
+  float* dq_acc;    // fp32 [total_q, H, D] accumulator (workspace)
+  void* dq;
+  void* dk;
+  void* dv;
+  const int32_t* cu_q;
+  const int32_t* cu_k;
+  int64_t do_rs, do_hs, q_rs, q_hs, k_rs, k_hs, v_rs, v_hs, o_rs, o_hs;
+  int64_t dq_rs, dq_hs, dk_rs, dk_hs, dv_rs, dv_hs;
+  int B, H;
+  int total_q, total_k;
+  int max_sq, max_sk;
+  int sq_r;        // innermost extent of dsoftmax
+  int lse_stride;  // innermost extent of lse
+  int nk_tiles;
+  int total_tiles;
+  float scale;
+  float scale_log2;
+  float p_keep;
+  float rp_keep;
+  uint32_t keep_thr;
+  PhiloxKey pk;
+  SparseMaps sp;
+};
+
+// Sequence extent of batch entry b, clamped so that a cu_seqlens array that disagrees with the declared
+// totals or maxima can never index outside the tensors: returns false if the entry must be skipped.
+FA_DEVICE bool seq_extent(const int32_t* cu, int b, int total, int max_len, int* begin, int* len) {
+  const int s = cu[b], e = cu[b + 1];
+  int n = e - s;
+  if (s < 0 || n <= 0 || e > total) return false;
+  *begin = s;
+  *len = n < max_len ? n : max_len;
+  return true;
+}
+
+// Launchers (defined in fa_fwd.hip / fa_bwd.hip / fa_aux.hip).  Return hipError_t of the launch.
+hipError_t launch_fwd(const FwdParams& p, int dtype, int head_dim, bool causal, bool dropout, bool sparse,
+                      hipStream_t stream);
+hipError_t launch_dump_probs(const DumpParams& p, int dtype, hipStream_t stream);
+hipError_t launch_bwd(const BwdParams& p, int dtype, int head_dim, bool causal, bool dropout, bool sparse,
+                      hipStream_t stream);
+hipError_t launch_build_sparse_maps(const int32_t* blockmask, uint8_t* act16, uint8_t* actq, uint8_t* actk, int nrb,
+                                    int ncb, int rows_per_qt, int nqt, int rows_per_qt2, int nqt2, hipStream_t stream);
+hipError_t launch_fill_f32(float* p, size_t n, float value, hipStream_t stream);
+// Zero a strided [total, H, D] tensor of 16-bit elements.
+hipError_t launch_zero_rows(void* base, int64_t row_stride, int64_t head_stride, int total, int H, int D,
+                            hipStream_t stream);
+// softmax_d = keep * rowsum(dO o O) and dq_acc = 0 (fmha_dgrad_kernel_1xN_loop.h:15-30).
+hipError_t launch_bwd_preprocess(const BwdParams& p, int dtype, int head_dim, hipStream_t stream);
+// dq = dq_acc * scale / keep, rounded to the element type (fmha_dgrad_kernel_1xN_loop.h:571-592).
+hipError_t launch_bwd_postprocess(const BwdParams& p, int dtype, int head_dim, hipStream_t stream);
+
+// Tile shapes, needed by the front end for grid sizes and workspace layout.
+constexpr int kFwdBM = 128;   // query rows per forward workgroup
+int bwd_block_n(int head_dim);  // keys per backward workgroup
+constexpr int kBwdBM = 64;    // query rows per backward inner step
+
+}  // namespace fa

@@ -1,0 +1,334 @@
+"""Binding of libflash_attn_gfx950.so: the module that stands where the reference's pybind11 extension
+``flash_attn_cuda`` stood (csrc/flash_attn/fmha_api.cpp:721-727).
+
+``fwd``, ``bwd``, ``fwd_block`` and ``bwd_block`` take the same arguments, in the same order, as
+mha_fwd / mha_bwd / mha_fwd_block / mha_bwd_block (fmha_api.cpp:173-186, 302-321, 451-464, 575-594) and return the
+same lists of tensors.  Torch is used only to own device memory, the current stream and the Philox
+(seed, offset) of the device's default generator; all computation happens behind the C ABI declared in
+include/flash_attn_gfx950.h.  There is no fallback: if the shared library is missing, importing the
+functions works but the first call raises.
+"""
+import ctypes
+import os
+import threading
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_NAME = "libflash_attn_gfx950.so"
+LIB_PATH = os.path.join(_HERE, LIB_NAME)
+
+FA_FP16, FA_BF16 = 0, 1
+FA_ABI_VERSION = 1
+
+_c_i32p = ctypes.c_void_p
+
+
+class FwdArgs(ctypes.Structure):
+    """struct fa_fwd_args of include/flash_attn_gfx950.h"""
+    _fields_ = [
+        ("struct_bytes", ctypes.c_uint32), ("dtype", ctypes.c_int32),
+        ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p), ("o", ctypes.c_void_p),
+        ("softmax_lse", ctypes.c_void_p), ("s_dmask", ctypes.c_void_p),
+        ("cu_seqlens_q", _c_i32p), ("cu_seqlens_k", _c_i32p), ("blockmask", _c_i32p),
+        ("q_row_stride", ctypes.c_int64), ("q_head_stride", ctypes.c_int64),
+        ("k_row_stride", ctypes.c_int64), ("k_head_stride", ctypes.c_int64),
+        ("v_row_stride", ctypes.c_int64), ("v_head_stride", ctypes.c_int64),
+        ("o_row_stride", ctypes.c_int64), ("o_head_stride", ctypes.c_int64),
+        ("batch", ctypes.c_int32), ("nheads", ctypes.c_int32), ("head_dim", ctypes.c_int32),
+        ("total_q", ctypes.c_int32), ("total_k", ctypes.c_int32),
+        ("max_seqlen_q", ctypes.c_int32), ("max_seqlen_k", ctypes.c_int32),
+        ("p_dropout", ctypes.c_float), ("softmax_scale", ctypes.c_float),
+        ("zero_tensors", ctypes.c_int32), ("is_causal", ctypes.c_int32),
+        ("philox_seed", ctypes.c_uint64), ("philox_offset", ctypes.c_uint64),
+        ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
+class BwdArgs(ctypes.Structure):
+    """struct fa_bwd_args of include/flash_attn_gfx950.h"""
+    _fields_ = [
+        ("struct_bytes", ctypes.c_uint32), ("dtype", ctypes.c_int32),
+        ("dout", ctypes.c_void_p), ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
+        ("out", ctypes.c_void_p), ("softmax_lse", ctypes.c_void_p),
+        ("dq", ctypes.c_void_p), ("dk", ctypes.c_void_p), ("dv", ctypes.c_void_p), ("softmax_d", ctypes.c_void_p),
+        ("cu_seqlens_q", _c_i32p), ("cu_seqlens_k", _c_i32p), ("blockmask", _c_i32p),
+        ("do_row_stride", ctypes.c_int64), ("do_head_stride", ctypes.c_int64),
+        ("q_row_stride", ctypes.c_int64), ("q_head_stride", ctypes.c_int64),
+        ("k_row_stride", ctypes.c_int64), ("k_head_stride", ctypes.c_int64),
+        ("v_row_stride", ctypes.c_int64), ("v_head_stride", ctypes.c_int64),
+        ("o_row_stride", ctypes.c_int64), ("o_head_stride", ctypes.c_int64),
+        ("dq_row_stride", ctypes.c_int64), ("dq_head_stride", ctypes.c_int64),
+        ("dk_row_stride", ctypes.c_int64), ("dk_head_stride", ctypes.c_int64),
+        ("dv_row_stride", ctypes.c_int64), ("dv_head_stride", ctypes.c_int64),
+        ("lse_seq_stride", ctypes.c_int32),
+        ("batch", ctypes.c_int32), ("nheads", ctypes.c_int32), ("head_dim", ctypes.c_int32),
+        ("total_q", ctypes.c_int32), ("total_k", ctypes.c_int32),
+        ("max_seqlen_q", ctypes.c_int32), ("max_seqlen_k", ctypes.c_int32),
+        ("p_dropout", ctypes.c_float), ("softmax_scale", ctypes.c_float),
+        ("zero_tensors", ctypes.c_int32), ("is_causal", ctypes.c_int32),
+        ("philox_seed", ctypes.c_uint64), ("philox_offset", ctypes.c_uint64),
+        ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
+EXPORTED_SYMBOLS = (
+    "fa_fwd", "fa_bwd", "fa_fwd_block", "fa_bwd_block", "fa_fwd_workspace_bytes", "fa_bwd_workspace_bytes",
+    "fa_round_seqlens", "fa_philox_offset_increment", "fa_last_error", "fa_abi_version",
+)
+
+_lib = None
+_lib_lock = threading.Lock()
+
+
+def load_library():
+    """dlopen the shared library once and declare the prototypes.  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lib_lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "%s is not built (expected at %s); run `python flash-attention_amd/build.py`. "
+                "There is no non-HIP fallback." % (LIB_NAME, LIB_PATH))
+        lib = ctypes.CDLL(LIB_PATH)
+        for name in ("fa_fwd", "fa_fwd_block"):
+            fn = getattr(lib, name)
+            fn.argtypes = [ctypes.POINTER(FwdArgs)]
+            fn.restype = ctypes.c_int
+        for name in ("fa_bwd", "fa_bwd_block"):
+            fn = getattr(lib, name)
+            fn.argtypes = [ctypes.POINTER(BwdArgs)]
+            fn.restype = ctypes.c_int
+        lib.fa_fwd_workspace_bytes.argtypes = [ctypes.POINTER(FwdArgs)]
+        lib.fa_fwd_workspace_bytes.restype = ctypes.c_size_t
+        lib.fa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdArgs)]
+        lib.fa_bwd_workspace_bytes.restype = ctypes.c_size_t
+        lib.fa_round_seqlens.argtypes = [ctypes.c_int32] * 4 + [ctypes.POINTER(ctypes.c_int32)] * 2
+        lib.fa_round_seqlens.restype = None
+        lib.fa_philox_offset_increment.argtypes = []
+        lib.fa_philox_offset_increment.restype = ctypes.c_uint64
+        lib.fa_last_error.argtypes = []
+        lib.fa_last_error.restype = ctypes.c_char_p
+        lib.fa_abi_version.argtypes = []
+        lib.fa_abi_version.restype = ctypes.c_int
+        if lib.fa_abi_version() != FA_ABI_VERSION:
+            raise RuntimeError("%s has ABI version %d, binding expects %d" % (LIB_NAME, lib.fa_abi_version(), FA_ABI_VERSION))
+        _lib = lib
+    return _lib
+
+
+def round_seqlens(head_dim, max_seqlen_q, max_seqlen_k, blocksparse=False):
+    """(max_seqlen_q_rounded, max_seqlen_k_rounded) as the library shapes softmax_lse / S_dmask
+    (fmha_api.cpp:232-241 and :509-514)."""
+    sq, sk = ctypes.c_int32(), ctypes.c_int32()
+    load_library().fa_round_seqlens(head_dim, max_seqlen_q, max_seqlen_k, int(blocksparse), ctypes.byref(sq), ctypes.byref(sk))
+    return sq.value, sk.value
+
+
+def _check(cond, msg):
+    # the reference's TORCH_CHECK failures surface in Python as RuntimeError
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _dtype_code(t):
+    _check(t.dtype in (torch.float16, torch.bfloat16), "q, k, v must be fp16 or bf16")  # fmha_api.cpp:198
+    return FA_FP16 if t.dtype == torch.float16 else FA_BF16
+
+
+def _check_qkv(name, t, dtype, total, nheads, head_dim):
+    _check(t.is_cuda, "%s must be on the GPU" % name)                                    # fmha_api.cpp:204-208
+    _check(t.dtype == dtype, "%s has dtype %s, expected %s" % (name, t.dtype, dtype))    # :199-200
+    _check(t.dim() == 3 and tuple(t.shape) == (total, nheads, head_dim),
+           "%s has shape %s, expected %s" % (name, tuple(t.shape), (total, nheads, head_dim)))  # CHECK_SHAPE :226-228
+    _check(t.stride(-1) == 1, "%s must have a contiguous last dimension" % name)         # :210-212
+
+
+def _check_cu(name, t, batch):
+    _check(t.is_cuda, "%s must be on the GPU" % name)
+    _check(t.dtype == torch.int32, "%s must be int32" % name)                            # :201-202
+    _check(t.is_contiguous(), "%s must be contiguous" % name)                            # :213-214
+    _check(t.dim() == 1 and t.numel() == batch + 1, "%s must have shape (batch + 1,)" % name)  # :229-230
+
+
+def _philox_state(device, p_dropout, gen):
+    """(seed, offset) of the device's generator, advanced the way philox_cuda_state(counter_offset) does
+    (fmha_api.cpp:288-292).  Restoring the generator state reproduces the pair, which is how the backward
+    regenerates the forward's mask (flash_attn_interface.py:43,61-63)."""
+    if not p_dropout > 0.0:
+        return 0, 0
+    if gen is None:
+        idx = device.index if device.index is not None else torch.cuda.current_device()
+        gen = torch.cuda.default_generators[idx]
+    seed = gen.initial_seed()
+    offset = gen.get_offset()
+    gen.set_offset(offset + int(load_library().fa_philox_offset_increment()))
+    return seed & 0xFFFFFFFFFFFFFFFF, offset & 0xFFFFFFFFFFFFFFFF
+
+
+def _stream_handle(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _raise(rc, lib):
+    msg = lib.fa_last_error().decode("utf-8", "replace")
+    raise RuntimeError("flash_attn_gfx950 error %d: %s" % (rc, msg))
+
+
+def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
+              zero_tensors, is_causal, return_softmax, gen):
+    lib = load_library()
+    code = _dtype_code(q)
+    _check(q.dim() == 3, "q must be (total_q, nheads, head_size)")
+    total_q, nheads, head_dim = q.shape
+    total_k = k.shape[0]
+    batch = cu_seqlens_q.numel() - 1
+    _check(batch > 0, "batch size must be positive")                                     # :223
+    _check(head_dim in (16, 32, 64, 128), "head_size must be 16, 32, 64 or 128")         # :224
+    _check_qkv("q", q, q.dtype, total_q, nheads, head_dim)
+    _check_qkv("k", k, q.dtype, total_k, nheads, head_dim)
+    _check_qkv("v", v, q.dtype, total_k, nheads, head_dim)
+    _check_cu("cu_seqlens_q", cu_seqlens_q, batch)
+    _check_cu("cu_seqlens_k", cu_seqlens_k, batch)
+    sparse = blockmask is not None
+    sq_r, sk_r = round_seqlens(head_dim, max_seqlen_q, max_seqlen_k, sparse)
+    if sparse:
+        _check(blockmask.is_cuda and blockmask.dtype == torch.int32 and blockmask.is_contiguous(),
+               "blockmask must be a contiguous int32 GPU tensor")                         # :477,484,491
+        _check(tuple(blockmask.shape) == (sk_r // 256, sq_r // 16),
+               "blockmask has shape %s, expected %s" % (tuple(blockmask.shape), (sk_r // 256, sq_r // 16)))  # :515
+
+    dev = q.device
+    with torch.cuda.device(dev):
+        o = torch.empty((total_q, nheads, head_dim), dtype=q.dtype, device=dev)
+        lse = torch.empty((batch, nheads, sq_r), dtype=torch.float32, device=dev)
+        s = torch.empty((batch, nheads, sq_r, sk_r), dtype=q.dtype, device=dev) if return_softmax else None
+        seed, offset = _philox_state(dev, p_dropout, gen)
+        a = FwdArgs()
+        a.struct_bytes = ctypes.sizeof(FwdArgs)
+        a.dtype = code
+        a.q, a.k, a.v, a.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
+        a.softmax_lse = lse.data_ptr()
+        a.s_dmask = s.data_ptr() if s is not None else None
+        a.cu_seqlens_q, a.cu_seqlens_k = cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr()
+        a.blockmask = blockmask.data_ptr() if sparse else None
+        a.q_row_stride, a.q_head_stride = q.stride(0), q.stride(1)
+        a.k_row_stride, a.k_head_stride = k.stride(0), k.stride(1)
+        a.v_row_stride, a.v_head_stride = v.stride(0), v.stride(1)
+        a.o_row_stride, a.o_head_stride = o.stride(0), o.stride(1)
+        a.batch, a.nheads, a.head_dim = batch, nheads, head_dim
+        a.total_q, a.total_k = total_q, total_k
+        a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
+        a.p_dropout, a.softmax_scale = float(p_dropout), float(softmax_scale)
+        a.zero_tensors, a.is_causal = int(bool(zero_tensors)), int(bool(is_causal))
+        a.philox_seed, a.philox_offset = seed, offset
+        ws_bytes = lib.fa_fwd_workspace_bytes(ctypes.byref(a))
+        ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev) if ws_bytes else None
+        a.workspace = ws.data_ptr() if ws is not None else None
+        a.workspace_bytes = ws_bytes
+        a.stream = _stream_handle(dev)
+        rc = (lib.fa_fwd_block if sparse else lib.fa_fwd)(ctypes.byref(a))
+        if rc != 0:
+            _raise(rc, lib)
+    return [o, lse, s] if return_softmax else [o, lse]
+
+
+def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q,
+              max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen):
+    lib = load_library()
+    code = _dtype_code(q)
+    _check(q.dim() == 3, "q must be (total_q, nheads, head_size)")
+    total_q, nheads, head_dim = q.shape
+    total_k = k.shape[0]
+    batch = cu_seqlens_q.numel() - 1
+    _check(batch > 0, "batch size must be positive")                                     # :371
+    _check(head_dim in (16, 32, 64, 128), "head_size must be 16, 32, 64 or 128")         # :372
+    for name, t, tot in (("q", q, total_q), ("k", k, total_k), ("v", v, total_k), ("out", out, total_q),
+                         ("dout", dout, total_q), ("dq", dq, total_q), ("dk", dk, total_k), ("dv", dv, total_k)):
+        _check_qkv(name, t, q.dtype, tot, nheads, head_dim)                              # :332-386
+    _check(out.is_contiguous() and dout.is_contiguous(), "out and dout must be contiguous")  # :355-356
+    _check_cu("cu_seqlens_q", cu_seqlens_q, batch)
+    _check_cu("cu_seqlens_k", cu_seqlens_k, batch)
+    _check(softmax_lse.is_cuda and softmax_lse.dtype == torch.float32 and softmax_lse.dim() == 3 and
+           softmax_lse.shape[0] == batch and softmax_lse.shape[1] == nheads, "softmax_lse must be fp32 (batch, nheads, seqlen)")
+    sparse = blockmask is not None
+    sq_r, sk_r = round_seqlens(head_dim, max_seqlen_q, max_seqlen_k, sparse)
+    if sparse:
+        _check(blockmask.is_cuda and blockmask.dtype == torch.int32 and blockmask.is_contiguous(),
+               "blockmask must be a contiguous int32 GPU tensor")
+        _check(tuple(blockmask.shape) == (sk_r // 256, sq_r // 16),
+               "blockmask has shape %s, expected %s" % (tuple(blockmask.shape), (sk_r // 256, sq_r // 16)))
+    softmax_lse = softmax_lse.contiguous()
+
+    dev = q.device
+    with torch.cuda.device(dev):
+        softmax_d = torch.empty((batch, nheads, sq_r), dtype=torch.float32, device=dev)
+        seed, offset = _philox_state(dev, p_dropout, gen)
+        a = BwdArgs()
+        a.struct_bytes = ctypes.sizeof(BwdArgs)
+        a.dtype = code
+        a.dout, a.q, a.k, a.v, a.out = dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+        a.softmax_lse = softmax_lse.data_ptr()
+        a.dq, a.dk, a.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+        a.softmax_d = softmax_d.data_ptr()
+        a.cu_seqlens_q, a.cu_seqlens_k = cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr()
+        a.blockmask = blockmask.data_ptr() if sparse else None
+        a.do_row_stride, a.do_head_stride = dout.stride(0), dout.stride(1)
+        a.q_row_stride, a.q_head_stride = q.stride(0), q.stride(1)
+        a.k_row_stride, a.k_head_stride = k.stride(0), k.stride(1)
+        a.v_row_stride, a.v_head_stride = v.stride(0), v.stride(1)
+        a.o_row_stride, a.o_head_stride = out.stride(0), out.stride(1)
+        a.dq_row_stride, a.dq_head_stride = dq.stride(0), dq.stride(1)
+        a.dk_row_stride, a.dk_head_stride = dk.stride(0), dk.stride(1)
+        a.dv_row_stride, a.dv_head_stride = dv.stride(0), dv.stride(1)
+        a.lse_seq_stride = softmax_lse.shape[2]
+        a.batch, a.nheads, a.head_dim = batch, nheads, head_dim
+        a.total_q, a.total_k = total_q, total_k
+        a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
+        a.p_dropout, a.softmax_scale = float(p_dropout), float(softmax_scale)
+        a.zero_tensors, a.is_causal = int(bool(zero_tensors)), int(bool(is_causal))
+        a.philox_seed, a.philox_offset = seed, offset
+        ws_bytes = lib.fa_bwd_workspace_bytes(ctypes.byref(a))
+        ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device=dev)
+        a.workspace = ws.data_ptr()
+        a.workspace_bytes = ws_bytes
+        a.stream = _stream_handle(dev)
+        rc = (lib.fa_bwd_block if sparse else lib.fa_bwd)(ctypes.byref(a))
+        if rc != 0:
+            _raise(rc, lib)
+    return [dq, dk, dv, softmax_d]
+
+
+def fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors,
+        is_causal, return_softmax, gen=None):
+    """mha_fwd (fmha_api.cpp:173-299): returns [o, softmax_lse] or [o, softmax_lse, s]."""
+    return _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, None, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
+                     zero_tensors, is_causal, return_softmax, gen)
+
+
+def bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+        p_dropout, softmax_scale, zero_tensors, is_causal, gen=None):
+    """mha_bwd (fmha_api.cpp:302-449): fills dq, dk, dv in place, returns [dq, dk, dv, softmax_d]."""
+    return _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, None, max_seqlen_q,
+                     max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen)
+
+
+def fwd_block(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
+              is_causal, return_softmax, gen=None):
+    """mha_fwd_block (fmha_api.cpp:451-573)."""
+    _check(blockmask is not None, "blockmask is required")
+    return _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout,
+                     softmax_scale, False, is_causal, return_softmax, gen)
+
+
+def bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q,
+              max_seqlen_k, p_dropout, softmax_scale, is_causal, gen=None):
+    """mha_bwd_block (fmha_api.cpp:575-718)."""
+    _check(blockmask is not None, "blockmask is required")
+    return _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q,
+                     max_seqlen_k, p_dropout, softmax_scale, False, is_causal, gen)

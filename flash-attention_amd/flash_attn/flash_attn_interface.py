@@ -1,0 +1,173 @@
+"""Functional API of the fused attention path, signature-compatible with the reference's
+flash_attn/flash_attn_interface.py (:151-252).  All three packings (qkv packed, kv packed, separate q/k/v) share one
+implementation; the packed variants hand strided views of the packed tensor to the kernels and let the backward write
+straight into views of one packed gradient buffer, as the reference does (:58-72, :96-111).
+"""
+import torch
+
+from . import flash_attn_gfx950 as _backend
+
+
+def _get_block_size(device, head_dim, is_dropout):
+    """Width of the key blocks that fix the rounded length of S_dmask (the reference keeps the same helper, :7-14;
+    on this device the answer follows fmha_api.cpp:232 for a non-sm80 part)."""
+    assert head_dim in [16, 32, 64, 128]
+    return 128 if head_dim == 128 else 256
+
+
+def _flash_attn_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
+                        softmax_scale, causal, return_softmax):
+    res = _backend.fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale,
+                       False, causal, return_softmax, None)
+    return res[0], res[1], (res[2] if return_softmax else None)
+
+
+def _flash_attn_backward(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
+                         max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal):
+    _, _, _, softmax_d = _backend.bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
+                                      max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, False, causal, None)
+    return dq, dk, dv, softmax_d
+
+
+def _split(packing, tensors):
+    """q, k, v views of the user's tensors for a given packing."""
+    if packing == "qkv":
+        (qkv,) = tensors
+        return qkv[:, 0], qkv[:, 1], qkv[:, 2]
+    if packing == "kv":
+        q, kv = tensors
+        return q, kv[:, 0], kv[:, 1]
+    return tensors
+
+
+def _forward(ctx, packing, tensors, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
+             softmax_scale, causal, return_softmax):
+    q, k, v = _split(packing, tensors)
+    # the dropout mask is a function of the generator state at this point; the backward rewinds to it
+    rng_state = torch.cuda.get_rng_state(q.device) if dropout_p > 0 else None
+    if softmax_scale is None:
+        softmax_scale = q.shape[-1] ** (-0.5)
+    out, softmax_lse, S_dmask = _flash_attn_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                                                    dropout_p, softmax_scale, causal, return_softmax)
+    ctx.save_for_backward(*tensors, out, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state)
+    ctx.packing = packing
+    ctx.n_in = len(tensors)
+    ctx.dropout_p = dropout_p
+    ctx.max_seqlen_q, ctx.max_seqlen_k = max_seqlen_q, max_seqlen_k
+    ctx.softmax_scale = softmax_scale
+    ctx.causal = causal
+    return out if not return_softmax else (out, softmax_lse, S_dmask)
+
+
+def _backward(ctx, dout):
+    saved = ctx.saved_tensors
+    tensors = saved[:ctx.n_in]
+    out, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state = saved[ctx.n_in:]
+    q, k, v = _split(ctx.packing, tensors)
+    grads = tuple(torch.empty_like(t) for t in tensors)
+    dq, dk, dv = _split(ctx.packing, grads)
+    dev = q.device
+    if rng_state is not None:
+        cur_rng_state = torch.cuda.get_rng_state(dev)
+        torch.cuda.set_rng_state(rng_state, dev)
+    _flash_attn_backward(dout.contiguous(), q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
+                         ctx.max_seqlen_q, ctx.max_seqlen_k, ctx.dropout_p, ctx.softmax_scale, ctx.causal)
+    if rng_state is not None:
+        torch.cuda.set_rng_state(cur_rng_state, dev)
+    return grads
+
+
+class FlashAttnQKVPackedFunc(torch.autograd.Function):
+    """apply(qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal, return_softmax)"""
+
+    @staticmethod
+    def forward(ctx, qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal, return_softmax):
+        return _forward(ctx, "qkv", (qkv,), cu_seqlens, cu_seqlens, max_seqlen, max_seqlen, dropout_p, softmax_scale,
+                        causal, return_softmax)
+
+    @staticmethod
+    def backward(ctx, dout, *args):
+        return _backward(ctx, dout) + (None,) * 6
+
+
+class FlashAttnKVPackedFunc(torch.autograd.Function):
+    """apply(q, kv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal,
+    return_softmax)"""
+
+    @staticmethod
+    def forward(ctx, q, kv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal,
+                return_softmax):
+        return _forward(ctx, "kv", (q, kv), cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
+                        softmax_scale, causal, return_softmax)
+
+    @staticmethod
+    def backward(ctx, dout, *args):
+        return _backward(ctx, dout) + (None,) * 8
+
+
+class FlashAttnFunc(torch.autograd.Function):
+    """apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal,
+    return_softmax)"""
+
+    @staticmethod
+    def forward(ctx, q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal,
+                return_softmax):
+        return _forward(ctx, "sep", (q, k, v), cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
+                        softmax_scale, causal, return_softmax)
+
+    @staticmethod
+    def backward(ctx, dout, *args):
+        return _backward(ctx, dout) + (None,) * 8
+
+
+_COMMON_DOC = """
+    dropout_p must be 0.0 at evaluation time.
+
+    Common arguments
+        cu_seqlens*: (batch_size + 1,) int32, cumulative sequence lengths; sequence b occupies rows
+            cu_seqlens[b]:cu_seqlens[b+1] of the packed token dimension.
+        max_seqlen*: int, an upper bound on the longest sequence in the batch.
+        dropout_p: float, probability of dropping an attention weight.
+        softmax_scale: float, multiplies Q K^T before the softmax; defaults to headdim ** -0.5.
+        causal: bool, query i of a sequence attends only to keys j <= i of that sequence.
+        return_attn_probs: bool, testing aid.
+    Returns
+        out: (total_q, nheads, headdim).
+        With return_attn_probs=True additionally
+        softmax_lse: (batch_size, nheads, seqlen_q rounded up to 16), fp32 log-sum-exp of each scaled score row.
+        S_dmask: (batch_size, nheads, seqlen_q rounded, seqlen_k rounded), softmax probabilities in the input dtype
+            with the dropout pattern in the sign bit: sign set = dropped, clear = kept.
+"""
+
+
+def flash_attn_unpadded_qkvpacked_func(qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale=None,
+                                       causal=False, return_attn_probs=False):
+    """Self-attention on a packed (total, 3, nheads, headdim) tensor of variable-length sequences."""
+    return FlashAttnQKVPackedFunc.apply(qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal,
+                                        return_attn_probs)
+
+
+def flash_attn_unpadded_kvpacked_func(q, kv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                                      dropout_p, softmax_scale=None, causal=False,
+                                      return_attn_probs=False):
+    """Attention of q (total_q, nheads, headdim) over packed keys/values kv (total_k, 2, nheads, headdim)."""
+    return FlashAttnKVPackedFunc.apply(q, kv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
+                                       softmax_scale, causal, return_attn_probs)
+
+
+def flash_attn_unpadded_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                             dropout_p, softmax_scale=None, causal=False, return_attn_probs=False):
+    """Attention of q (total_q, nheads, headdim) over k, v (total_k, nheads, headdim)."""
+    return FlashAttnFunc.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
+                               softmax_scale, causal, return_attn_probs)
+
+
+def flash_attn_func(qkv, cu_seqlens, dropout_p, max_s, softmax_scale=None, causal=False,
+                    return_attn_probs=False):
+    """Older argument order of flash_attn_unpadded_qkvpacked_func, kept for callers that still use it."""
+    return flash_attn_unpadded_qkvpacked_func(qkv, cu_seqlens, max_s, dropout_p, softmax_scale, causal,
+                                              return_attn_probs)
+
+
+for _f in (flash_attn_unpadded_qkvpacked_func, flash_attn_unpadded_kvpacked_func, flash_attn_unpadded_func):
+    _f.__doc__ += _COMMON_DOC

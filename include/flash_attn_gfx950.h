@@ -1,0 +1,147 @@
+/*
+ * flash_attn_gfx950.h -- C ABI of the MI355X (gfx950) FlashAttention engine.
+ *
+ * This shared library replaces the reference's pybind11 module `flash_attn_cuda`
+ * (csrc/flash_attn/fmha_api.cpp:721-727).  Each entry point below is what a binding for one of
+ * that module's four functions calls.  Differences from the reference boundary, by design:
+ *   - plain pointers, sizes and strides only (no ATen types);
+ *   - every buffer is owned by the caller, including outputs and scratch (`workspace`);
+ *   - the Philox (seed, offset) pair is passed in instead of being drawn from a generator;
+ *   - errors are returned as negative codes with a message in fa_last_error(); nothing here
+ *     exits the process (the reference's FMHA_CHECK_CUDA does, fmha_utils.h:39-50);
+ *   - work is enqueued on `stream` and never synchronised.
+ *
+ * Tensor conventions (as fmha_api.cpp:173-186): q is [total_q, nheads, head_dim], k and v are
+ * [total_k, nheads, head_dim], element type fp16 or bf16, innermost stride 1, row and head strides
+ * given in ELEMENTS (a packed qkv[total,3,H,d] view has row stride 3*H*d).  cu_seqlens_* are int32
+ * [batch+1] device arrays of cumulative sequence lengths.
+ */
+#ifndef FLASH_ATTN_GFX950_H_
+#define FLASH_ATTN_GFX950_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FA_ABI_VERSION 1
+
+enum fa_dtype { FA_FP16 = 0, FA_BF16 = 1 };
+
+enum fa_status {
+  FA_OK = 0,
+  FA_ERR_INVALID_ARGUMENT = -1, /* a TORCH_CHECK of fmha_api.cpp would have thrown */
+  FA_ERR_WORKSPACE = -2,        /* workspace missing or smaller than fa_*_workspace_bytes() */
+  FA_ERR_LAUNCH = -3,           /* HIP reported a launch error */
+  FA_ERR_UNSUPPORTED = -4
+};
+
+/* Arguments of the forward pass.  Mirrors mha_fwd (fmha_api.cpp:173-186) and, when `blockmask`
+ * is non-NULL, mha_fwd_block (fmha_api.cpp:451-464). */
+typedef struct fa_fwd_args {
+  uint32_t struct_bytes; /* sizeof(fa_fwd_args), checked */
+  int32_t dtype;         /* enum fa_dtype */
+  const void* q;
+  const void* k;
+  const void* v;
+  void* o;            /* [total_q, nheads, head_dim], same dtype; written for rows < seqlen_q */
+  float* softmax_lse; /* [batch, nheads, max_seqlen_q_rounded] fp32 */
+  void* s_dmask;      /* NULL, or [batch, nheads, max_seqlen_q_rounded, max_seqlen_k_rounded] in `dtype`:
+                         row-major softmax probabilities, negative sign = dropped (return_softmax) */
+  const int32_t* cu_seqlens_q;
+  const int32_t* cu_seqlens_k;
+  const int32_t* blockmask; /* NULL = dense.  Else the converted block list of
+                               flash_blocksparse_attn_interface.py:8-40: int32
+                               [max_seqlen_k_rounded/256, max_seqlen_q_rounded/16] */
+  int64_t q_row_stride, q_head_stride;
+  int64_t k_row_stride, k_head_stride;
+  int64_t v_row_stride, v_head_stride;
+  int64_t o_row_stride, o_head_stride;
+  int32_t batch, nheads, head_dim;
+  int32_t total_q, total_k;
+  int32_t max_seqlen_q, max_seqlen_k; /* as given by the caller, before rounding */
+  float p_dropout;                    /* probability of DROPPING, in [0,1) (fmha_api.cpp:113) */
+  float softmax_scale;
+  int32_t zero_tensors; /* pre-fill o=0, lse=-inf, s_dmask=0 (fmha_api.cpp:256-260) */
+  int32_t is_causal;
+  uint64_t philox_seed, philox_offset;
+  void* workspace; /* device scratch of >= fa_fwd_workspace_bytes() bytes (may be NULL if that is 0) */
+  size_t workspace_bytes;
+  void* stream; /* hipStream_t */
+} fa_fwd_args;
+
+/* Arguments of the backward pass.  Mirrors mha_bwd (fmha_api.cpp:302-321) and, when `blockmask`
+ * is non-NULL, mha_bwd_block (fmha_api.cpp:575-594).  dq, dk, dv are caller-allocated, possibly
+ * strided views written in place. */
+typedef struct fa_bwd_args {
+  uint32_t struct_bytes;
+  int32_t dtype;
+  const void* dout; /* [total_q, nheads, head_dim] */
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* out;
+  const float* softmax_lse; /* [batch, nheads, lse_seq_stride] as written by the forward */
+  void* dq;
+  void* dk;
+  void* dv;
+  float* softmax_d; /* [batch, nheads, max_seqlen_q_rounded] fp32: rowsum(dout * out) */
+  const int32_t* cu_seqlens_q;
+  const int32_t* cu_seqlens_k;
+  const int32_t* blockmask;
+  int64_t do_row_stride, do_head_stride;
+  int64_t q_row_stride, q_head_stride;
+  int64_t k_row_stride, k_head_stride;
+  int64_t v_row_stride, v_head_stride;
+  int64_t o_row_stride, o_head_stride;
+  int64_t dq_row_stride, dq_head_stride;
+  int64_t dk_row_stride, dk_head_stride;
+  int64_t dv_row_stride, dv_head_stride;
+  int32_t lse_seq_stride; /* innermost extent of softmax_lse (the forward's max_seqlen_q_rounded) */
+  int32_t batch, nheads, head_dim;
+  int32_t total_q, total_k;
+  int32_t max_seqlen_q, max_seqlen_k;
+  float p_dropout;
+  float softmax_scale;
+  int32_t zero_tensors; /* pre-fill dq=dk=dv=0, softmax_d=0 (fmha_api.cpp:406-411) */
+  int32_t is_causal;
+  uint64_t philox_seed, philox_offset; /* the pair the forward was given */
+  void* workspace;
+  size_t workspace_bytes;
+  void* stream;
+} fa_bwd_args;
+
+/* replaces flash_attn_cuda.fwd -> mha_fwd, csrc/flash_attn/fmha_api.cpp:173-299 */
+int fa_fwd(const fa_fwd_args* args);
+/* replaces flash_attn_cuda.bwd -> mha_bwd, csrc/flash_attn/fmha_api.cpp:302-449 */
+int fa_bwd(const fa_bwd_args* args);
+/* replaces flash_attn_cuda.fwd_block -> mha_fwd_block, csrc/flash_attn/fmha_api.cpp:451-573
+ * (args->blockmask must be non-NULL) */
+int fa_fwd_block(const fa_fwd_args* args);
+/* replaces flash_attn_cuda.bwd_block -> mha_bwd_block, csrc/flash_attn/fmha_api.cpp:575-718 */
+int fa_bwd_block(const fa_bwd_args* args);
+
+/* Scratch the caller must provide; stands in for the o_tmp / dq_tmp / softmax_d allocations of
+ * fmha_api.cpp:243-254,401-404.  Only shapes, dtype and blockmask!=NULL are read. */
+size_t fa_fwd_workspace_bytes(const fa_fwd_args* args);
+size_t fa_bwd_workspace_bytes(const fa_bwd_args* args);
+
+/* Seqlen rounding used for the shapes of softmax_lse / s_dmask / softmax_d / blockmask
+ * (fmha_api.cpp:232-241 dense, :509-514 block-sparse).  Writes the rounded values. */
+void fa_round_seqlens(int32_t head_dim, int32_t max_seqlen_q, int32_t max_seqlen_k, int32_t blocksparse,
+                      int32_t* max_seqlen_q_rounded, int32_t* max_seqlen_k_rounded);
+
+/* Number of 64-bit Philox offsets one forward call consumes; the caller advances its generator
+ * by this much (the role of launch_params.elts_per_thread, fmha_api.cpp:282-292). */
+uint64_t fa_philox_offset_increment(void);
+
+/* Message for the last non-zero status returned on the calling thread. */
+const char* fa_last_error(void);
+int fa_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASH_ATTN_GFX950_H_ */
