@@ -1,0 +1,90 @@
+"""nn.Module front ends of the fused attention path, interface-compatible with the reference's
+flash_attn/flash_attention.py (:12-118)."""
+import torch
+import torch.nn as nn
+
+from .bert_padding import pad_input, unpad_input
+from .flash_attn_interface import flash_attn_unpadded_qkvpacked_func
+
+
+class FlashAttention(nn.Module):
+    """Scaled dot-product softmax attention on packed qkv.
+
+    Arguments
+    ---------
+        softmax_scale: temperature of the softmax (default: 1/sqrt(head_dim), taken at run time)
+        attention_dropout: dropout probability applied to the attention weights while training (default 0.0)
+    """
+
+    def __init__(self, softmax_scale=None, attention_dropout=0.0, device=None, dtype=None):
+        super().__init__()
+        self.softmax_scale = softmax_scale
+        self.dropout_p = attention_dropout
+
+    def forward(self, qkv, attn_mask=None, key_padding_mask=None, causal=False, cu_seqlens=None, max_s=None,
+                need_weights=False):
+        """qkv is (B, S, 3, H, D) when cu_seqlens is None, else already packed (nnz, 3, H, D) with cu_seqlens / max_s.
+        key_padding_mask, if given, is an object whose `.bool_matrix` is a (B, S) bool tensor, True = keep.
+        Returns (output, None); output has the layout of the input's token dimensions."""
+        assert not need_weights
+        assert attn_mask is None
+        assert qkv.dtype == torch.float16  # the reference's module restriction (:41); the functional API takes bf16 too
+        assert qkv.is_cuda
+        p = self.dropout_p if self.training else 0.0
+
+        if cu_seqlens is not None:
+            assert max_s is not None
+            out = flash_attn_unpadded_qkvpacked_func(qkv, cu_seqlens, max_s, p, softmax_scale=self.softmax_scale,
+                                                     causal=causal)
+            return out, None
+
+        batch, seqlen = qkv.shape[0], qkv.shape[1]
+        if key_padding_mask is None:
+            packed = qkv.reshape(batch * seqlen, *qkv.shape[2:])
+            cu = torch.arange(0, (batch + 1) * seqlen, step=seqlen, dtype=torch.int32, device=qkv.device)
+            out = flash_attn_unpadded_qkvpacked_func(packed, cu, seqlen, p, softmax_scale=self.softmax_scale,
+                                                     causal=causal)
+            return out.reshape(batch, seqlen, *out.shape[1:]), None
+
+        nheads, headdim = qkv.shape[-2], qkv.shape[-1]
+        x = qkv.reshape(batch, seqlen, 3 * nheads * headdim)
+        x_unpad, indices, cu, max_len = unpad_input(x, key_padding_mask.bool_matrix)
+        out_unpad = flash_attn_unpadded_qkvpacked_func(x_unpad.reshape(-1, 3, nheads, headdim), cu, max_len, p,
+                                                       softmax_scale=self.softmax_scale, causal=causal)
+        out = pad_input(out_unpad.reshape(-1, nheads * headdim), indices, batch, seqlen)
+        return out.reshape(batch, seqlen, nheads, headdim), None
+
+
+class FlashMHA(nn.Module):
+    """Multi-head self-attention block: fused QKV projection, FlashAttention, output projection."""
+
+    def __init__(self, embed_dim, num_heads, bias=True, batch_first=True, attention_dropout=0.0, causal=False,
+                 use_rotary_emb=None, device=None, dtype=None, **kwargs) -> None:
+        assert batch_first
+        factory_kwargs = {"device": device, "dtype": dtype}
+        super().__init__()
+        self.embed_dim = embed_dim
+        self.causal = causal
+        self.num_heads = num_heads
+        assert self.embed_dim % num_heads == 0, "self.kdim must be divisible by num_heads"
+        self.head_dim = self.embed_dim // num_heads
+        assert self.head_dim in [16, 32, 64], "Only support head_dim == 16, 32, or 64"
+        assert use_rotary_emb in [None, "1d", "2d"]
+        self.use_rotary_emb = use_rotary_emb
+        if use_rotary_emb is not None:
+            from .rotary import RotaryEmbedding, RotaryEmbedding2D
+            self.rotary_emb = RotaryEmbedding(self.head_dim) if use_rotary_emb == "1d" else RotaryEmbedding2D(self.head_dim)
+        self.Wqkv = nn.Linear(embed_dim, 3 * embed_dim, bias=bias, **factory_kwargs)
+        self.inner_attn = FlashAttention(attention_dropout=attention_dropout, **factory_kwargs)
+        self.out_proj = nn.Linear(embed_dim, embed_dim, bias=bias, **factory_kwargs)
+
+    def forward(self, x, x_ignored_, x_ignored_1_, attn_mask=None, key_padding_mask=None, need_weights=False):
+        b, s = x.shape[0], x.shape[1]
+        qkv = self.Wqkv(x).reshape(b, s, 3, self.num_heads, self.head_dim)
+        if self.use_rotary_emb:
+            query, key, value = qkv.unbind(dim=2)
+            query, key = self.rotary_emb(query, key, seq_dimension=-3)
+            qkv = torch.stack([query, key, value], dim=2)
+        context, attn_weights = self.inner_attn(qkv, key_padding_mask=key_padding_mask, need_weights=need_weights,
+                                                causal=self.causal)
+        return self.out_proj(context.reshape(b, s, self.embed_dim)), attn_weights

@@ -1,0 +1,113 @@
+"""Block-sparse attention, signature-compatible with the reference's flash_attn/flash_blocksparse_attn_interface.py.
+
+The sparsity layout has one entry per 16-row x 256-key block of the score matrix.  `convert_blockmask` turns a 0/1
+layout into the per-column block lists the native entry points take (the reference's own format, :8-40).  The
+reference's Python at this commit calls its extension with an argument list its C++ no longer accepts
+(:45-47,56-58 vs fmha_api.cpp:451-464,575-594); here the public signature is kept and the native call uses the
+C++ argument order.
+"""
+import torch
+
+from . import flash_attn_gfx950 as _backend
+
+
+def convert_blockmask(blockmask, causal):
+    """0/1 layout (row, col) -> int32 (col, row).  Row c of the result lists the nonzero row-block indices of column
+    c in ascending order, padded with -1.  Each index is multiplied by 4; bit 0 marks the first nonzero of its
+    layout row, bit 1 the last nonzero of its layout row."""
+    assert not causal
+    nz = blockmask != 0
+    nrow, ncol = nz.shape
+    dev = nz.device
+    cols = torch.arange(ncol, device=dev)
+    big = ncol + 1
+    first_col = torch.where(nz, cols, torch.full_like(cols, big)).min(dim=1).values   # (nrow,)
+    last_col = torch.where(nz, cols, torch.full_like(cols, -1)).max(dim=1).values
+    rows = torch.arange(nrow, device=dev)[:, None]
+    code = 4 * rows + (cols[None, :] == first_col[:, None]).long() + 2 * (cols[None, :] == last_col[:, None]).long()
+    code = torch.where(nz, code, torch.full_like(code, -1))                           # (nrow, ncol)
+    # per column: active rows first (ascending), then the -1 padding
+    order = torch.sort((~nz).to(torch.int64) * (nrow + 1) + rows, dim=0).indices      # (nrow, ncol)
+    return torch.gather(code, 0, order).T.contiguous().to(torch.int32)
+
+
+def _flash_blocksparse_attn_forward(qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal,
+                                    return_softmax):
+    res = _backend.fwd_block(qkv[:, 0], qkv[:, 1], qkv[:, 2], cu_seqlens, cu_seqlens, blockmask, max_s, max_s,
+                             dropout_p, softmax_scale, causal, return_softmax, None)
+    return res[0], res[1], (res[2] if return_softmax else None)
+
+
+def _flash_blocksparse_attn_backward(dout, qkv, out, S_dmask, softmax_lse, cu_seqlens, blockmask, dropout_p, max_s,
+                                     softmax_scale, causal):
+    dqkv = torch.empty_like(qkv)
+    _backend.bwd_block(dout.contiguous(), qkv[:, 0], qkv[:, 1], qkv[:, 2], out, softmax_lse, dqkv[:, 0], dqkv[:, 1],
+                       dqkv[:, 2], cu_seqlens, cu_seqlens, blockmask, max_s, max_s, dropout_p, softmax_scale, causal,
+                       None)
+    return dqkv
+
+
+def _fwd_common(ctx, qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal, return_softmax):
+    rng_state = torch.cuda.get_rng_state(qkv.device) if dropout_p > 0 else None
+    if softmax_scale is None:
+        softmax_scale = qkv.shape[-1] ** (-0.5)
+    context, softmax_lse, S_dmask = _flash_blocksparse_attn_forward(
+        qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal, return_softmax)
+    ctx.save_for_backward(qkv, context, softmax_lse, cu_seqlens, blockmask, rng_state)
+    ctx.dropout_p = dropout_p
+    ctx.max_s = max_s
+    ctx.softmax_scale = softmax_scale
+    ctx.causal = causal
+    return context, S_dmask, softmax_lse
+
+
+def _bwd_common(ctx, dout):
+    qkv, context, softmax_lse, cu_seqlens, blockmask, rng_state = ctx.saved_tensors
+    dev = qkv.device
+    if rng_state is not None:
+        cur_rng_state = torch.cuda.get_rng_state(dev)
+        torch.cuda.set_rng_state(rng_state, dev)
+    dqkv = _flash_blocksparse_attn_backward(dout, qkv, context, None, softmax_lse, cu_seqlens, blockmask,
+                                            ctx.dropout_p, ctx.max_s, ctx.softmax_scale, ctx.causal)
+    if rng_state is not None:
+        torch.cuda.set_rng_state(cur_rng_state, dev)
+    return dqkv
+
+
+class FlashBlocksparseAttnFun(torch.autograd.Function):
+    """apply(qkv, cu_seqlens, blockmask_converted, dropout_p, max_s, softmax_scale, causal) -> context"""
+
+    @staticmethod
+    def forward(ctx, qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal):
+        return _fwd_common(ctx, qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal, False)[0]
+
+    @staticmethod
+    def backward(ctx, dout):
+        return _bwd_common(ctx, dout), None, None, None, None, None, None
+
+
+class FlashBlocksparseAttnFunWithS(torch.autograd.Function):
+    """Same, returning (context, S_dmask, softmax_lse) for tests."""
+
+    @staticmethod
+    def forward(ctx, qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal):
+        context, S_dmask, softmax_lse = _fwd_common(ctx, qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale,
+                                                    causal, True)
+        ctx.mark_non_differentiable(S_dmask, softmax_lse)
+        return context, S_dmask, softmax_lse
+
+    @staticmethod
+    def backward(ctx, dout, _dS_dmask_ignored, _dsoftmax_sum_ignored):
+        return _bwd_common(ctx, dout), None, None, None, None, None, None
+
+
+def flash_blocksparse_attn_func(qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale=None,
+                                causal=False, return_attn_probs=False, convert_mask=True):
+    """Self-attention on packed qkv (total, 3, nheads, headdim) restricted to the active blocks of `blockmask`
+    ((seqlen rounded to 16) / 16 rows by (seqlen rounded to 256) / 256 columns of 0/1, or already converted when
+    convert_mask=False).  Query rows whose blocks are all inactive produce zeros.  dropout_p must be 0.0 at
+    evaluation time.  With return_attn_probs=True returns (context, S_dmask, softmax_lse)."""
+    func = FlashBlocksparseAttnFun if not return_attn_probs else FlashBlocksparseAttnFunWithS
+    if convert_mask:
+        blockmask = convert_blockmask(blockmask, causal=causal)
+    return func.apply(qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal)

@@ -1,0 +1,86 @@
+"""Rotary position embeddings used by FlashMHA(use_rotary_emb=...), interface-compatible with the reference's
+flash_attn/rotary.py (:22-135).  Pure PyTorch pre-processing of q and k ahead of the attention kernels.
+
+Convention (rotary.py:22-42,66-87): channel pairs are interleaved, (x[2i], x[2i+1]) is rotated by angle
+pos * 10000^(-2i/dim):   x'[2i] = x[2i] cos - x[2i+1] sin,   x'[2i+1] = x[2i+1] cos + x[2i] sin.
+The cos/sin tables are rounded to the input dtype before use, as the reference does.
+"""
+import math
+from typing import Tuple
+
+import torch
+
+
+def rotate_half(x):
+    """(x0, x1, x2, x3, ...) -> (-x1, x0, -x3, x2, ...)"""
+    pairs = x.reshape(*x.shape[:-1], -1, 2)
+    return torch.stack((-pairs[..., 1], pairs[..., 0]), dim=-1).reshape(x.shape)
+
+
+def apply_rotary_pos_emb(x, cos, sin, seq_dimension: int = -2):
+    """x: (..., s, d) if seq_dimension == -2, (..., s, h, d) if -3.  cos, sin: (>= s, d)."""
+    n = x.shape[seq_dimension]
+    cos, sin = cos[:n], sin[:n]
+    if seq_dimension == -3:
+        cos, sin = cos[:, None, :], sin[:, None, :]
+    return x * cos + rotate_half(x) * sin
+
+
+class RotaryEmbedding(torch.nn.Module):
+    """Rotary embedding of RoFormer (Su et al., arXiv:2104.09864) for queries and keys."""
+
+    def __init__(self, dim_model: int, *_, **__):
+        super().__init__()
+        exponent = torch.arange(0, dim_model, 2).float() / dim_model
+        self.register_buffer("inv_freq", 1.0 / (10000 ** exponent))
+        self._seq_len_cached = None
+        self._cos_cached = None
+        self._sin_cached = None
+
+    def _update_cos_sin_tables(self, x, seq_dimension=-2):
+        seq_len = x.shape[seq_dimension]
+        stale = (seq_len != self._seq_len_cached or self._cos_cached.device != x.device
+                 or self._cos_cached.dtype != x.dtype)
+        if stale:
+            self._seq_len_cached = seq_len
+            pos = torch.arange(seq_len, device=x.device, dtype=self.inv_freq.dtype)
+            angles = torch.outer(pos, self.inv_freq.to(x.device))  # fp32 (seq, dim/2)
+            self._cos_cached = torch.cos(angles).to(x.dtype).repeat_interleave(2, dim=-1)
+            self._sin_cached = torch.sin(angles).to(x.dtype).repeat_interleave(2, dim=-1)
+        return self._cos_cached, self._sin_cached
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, seq_dimension=-2) -> Tuple[torch.Tensor, torch.Tensor]:
+        assert seq_dimension in [-2, -3]  # (bs, h, s, d) or (bs, s, h, d)
+        cos, sin = self._update_cos_sin_tables(k, seq_dimension=seq_dimension)
+        return (apply_rotary_pos_emb(q, cos, sin, seq_dimension), apply_rotary_pos_emb(k, cos, sin, seq_dimension))
+
+
+class RotaryEmbedding2D(torch.nn.Module):
+    """Rotary embedding for a square grid of tokens (seqlen = side * side): the first half of the channels is
+    rotated by the column index, the second half by the row index."""
+
+    def __init__(self, dim: int):
+        super().__init__()
+        assert dim % 4 == 0
+        self.rotary_emb1d = RotaryEmbedding(dim // 2)
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, seq_dimension=-2):
+        assert seq_dimension in [-2, -3]
+        seqlen = q.shape[seq_dimension]
+        side = int(math.sqrt(seqlen))
+        assert seqlen == side * side
+        if seq_dimension == -3:  # (bs, s, h, d) -> (bs, h, s, d)
+            q, k = q.transpose(1, 2), k.transpose(1, 2)
+        half = q.shape[-1] // 2
+
+        def grid(t):  # (b, nheads, side*side, c) -> (b, nheads, side, side, c)
+            return t.reshape(t.shape[0], t.shape[1], side, side, t.shape[-1])
+
+        # first half: position = column (inner grid axis); second half: position = row (outer grid axis)
+        q0, k0 = self.rotary_emb1d(grid(q[..., :half]), grid(k[..., :half]), seq_dimension=-2)
+        q1, k1 = self.rotary_emb1d(grid(q[..., half:]), grid(k[..., half:]), seq_dimension=-3)
+        q_emb = torch.cat([q0.reshape(*q.shape[:-1], half), q1.reshape(*q.shape[:-1], half)], dim=-1)
+        k_emb = torch.cat([k0.reshape(*k.shape[:-1], half), k1.reshape(*k.shape[:-1], half)], dim=-1)
+        if seq_dimension == -3:
+            q_emb, k_emb = q_emb.transpose(1, 2), k_emb.transpose(1, 2)
+        return q_emb, k_emb

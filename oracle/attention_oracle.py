@@ -20,8 +20,8 @@ How each function is pinned (the reference has no tests, golden vectors or fixtu
       => mean of v) and against tiled_forward for several block widths;  lse: rows of exp(scale*S - lse) sum to 1.
   varlen_attention backward: autograd of the closed form, cross-checked with fp64 finite differences and with the
       explicit formulas dV = P^T dO, dS = P o (dP - D), dQ = scale dS K, dK = scale dS^T Q.
-  philox4x32: the published Random123 known-answer vectors for philox4x32-10; the 7-round variant the reference
-      uses has no published vector and is the same round function applied 7 times.
+  philox4x32: the published Random123 known-answer vectors for philox4x32 with 10 rounds and with the 7 rounds
+      the reference uses (tests/golden/philox_kat.json).
   dropout_keep_mask: it is the definition; tests compare the kernels' S_dmask signs to it bit for bit.
   convert_blockmask_ref: brute force over all small masks against an independent per-element definition.
 PARITY UNPINNED (only running the CUDA reference could pin them; nothing in this pipeline can): the reference's
@@ -60,19 +60,19 @@ def attention_ref(qkv, attn_mask, dropout_p, upcast=False, causal=False, keep_ma
 # --------------------------------------------------------------------------------------------------
 # Closed form on packed variable-length batches
 # --------------------------------------------------------------------------------------------------
-def expand_block_layout(layout, Lq, Lk):
+def expand_block_layout(layout, Lq, Lk, device="cpu"):
     """bool (Lq, Lk) mask from a 0/1 layout of 16-row x 256-key blocks (fmha_api.cpp:509-515)."""
-    m = torch.as_tensor(layout).bool()
+    m = torch.as_tensor(layout).bool().to(device)
     full = m.repeat_interleave(16, 0).repeat_interleave(256, 1)
     return full[:Lq, :Lk]
 
 
-def _score_mask(Lq, Lk, causal, layout):
-    valid = torch.ones(Lq, Lk, dtype=torch.bool)
+def _score_mask(Lq, Lk, causal, layout, device="cpu"):
+    valid = torch.ones(Lq, Lk, dtype=torch.bool, device=device)
     if causal:  # query i sees keys j <= i, both counted from the start of the sequence (mask.h:69)
-        valid &= torch.arange(Lk)[None, :] <= torch.arange(Lq)[:, None]
+        valid &= torch.arange(Lk, device=device)[None, :] <= torch.arange(Lq, device=device)[:, None]
     if layout is not None:
-        valid &= expand_block_layout(layout, Lq, Lk)
+        valid &= expand_block_layout(layout, Lq, Lk, device)
     return valid
 
 
@@ -102,14 +102,14 @@ def varlen_attention(q, k, v, cu_q, cu_k, softmax_scale=None, causal=False, p_dr
         vb = vf[cu_k[b]:cu_k[b + 1]].transpose(0, 1)
         Lq, Lk = qb.shape[1], kb.shape[1]
         s = torch.einsum("hqd,hkd->hqk", qb, kb) * scale
-        valid = _score_mask(Lq, Lk, causal, layout)
+        valid = _score_mask(Lq, Lk, causal, layout, qf.device)
         s = s.masked_fill(~valid[None], float("-inf"))
         lse = torch.logsumexp(s, dim=-1)  # -inf for empty rows
         p = torch.exp(s - torch.where(torch.isinf(lse), torch.zeros_like(lse), lse)[..., None])
         p = torch.where(valid[None], p, torch.zeros_like(p))
         pd = p
         if keep_mask is not None:
-            pd = p * keep_mask[b].to(dtype) / keep
+            pd = p * keep_mask[b].to(device=qf.device, dtype=dtype) / keep
         ob = torch.einsum("hqk,hkd->hqd", pd, vb)
         outs.append(ob.transpose(0, 1))
         lses.append(lse.detach())

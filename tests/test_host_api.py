@@ -1,0 +1,248 @@
+"""CPU-side tests: the C-ABI library loads and exports what include/flash_attn_gfx950.h declares, argument
+validation returns errors instead of aborting, the seqlen rounding follows fmha_api.cpp, and the pure-host helpers
+(bert_padding, convert_blockmask, rotary) match their specifications.  Nothing here launches a kernel."""
+import ctypes
+import inspect
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention_oracle as orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    header = open(os.path.join(ROOT, "include", "flash_attn_gfx950.h")).read()
+    declared = set(re.findall(r"^\s*(?:int|size_t|void|uint64_t|const char\*)\s+(fa_\w+)\s*\(", header, re.M))
+    from flash_attn import flash_attn_gfx950 as be
+    assert declared == set(be.EXPORTED_SYMBOLS)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.fa_abi_version() == 1
+
+
+def test_struct_layout_matches_library(lib):
+    """a wrong struct size is reported as an ABI mismatch; the right size passes that check"""
+    from flash_attn import flash_attn_gfx950 as be
+    a = be.FwdArgs()
+    a.struct_bytes = ctypes.sizeof(a) - 8
+    assert lib.fa_fwd(ctypes.byref(a)) == -1 and b"ABI mismatch" in lib.fa_last_error()
+    a.struct_bytes = ctypes.sizeof(a)
+    a.dtype = 7
+    assert lib.fa_fwd(ctypes.byref(a)) == -1 and b"dtype" in lib.fa_last_error()
+    g = be.BwdArgs()
+    g.struct_bytes = ctypes.sizeof(g)
+    g.dtype = 7
+    assert lib.fa_bwd(ctypes.byref(g)) == -1 and b"dtype" in lib.fa_last_error()
+
+
+def _valid_fwd_args(be):
+    a = be.FwdArgs()
+    a.struct_bytes = ctypes.sizeof(a)
+    a.dtype = be.FA_FP16
+    a.batch, a.nheads, a.head_dim = 1, 1, 64
+    a.total_q = a.total_k = 16
+    a.max_seqlen_q = a.max_seqlen_k = 16
+    a.p_dropout, a.softmax_scale = 0.0, 0.125
+    for f in ("q_row_stride", "k_row_stride", "v_row_stride", "o_row_stride"):
+        setattr(a, f, 64)
+    for f in ("q_head_stride", "k_head_stride", "v_head_stride", "o_head_stride"):
+        setattr(a, f, 64)
+    return a
+
+
+@pytest.mark.parametrize("field,value,needle", [
+    ("batch", 0, b"batch_size"),                 # fmha_api.cpp:223
+    ("head_dim", 48, b"head_size"),              # :224
+    ("p_dropout", 1.0, b"p_dropout"),            # :113
+    ("p_dropout", -0.1, b"p_dropout"),
+    ("softmax_scale", 0.0, b"softmax_scale"),
+    ("max_seqlen_q", 0, b"max_seqlen"),
+])
+def test_forward_argument_checks(lib, field, value, needle):
+    from flash_attn import flash_attn_gfx950 as be
+    a = _valid_fwd_args(be)
+    setattr(a, field, value)
+    rc = lib.fa_fwd(ctypes.byref(a))
+    assert rc == -1 and needle in lib.fa_last_error(), lib.fa_last_error()
+
+
+def test_null_pointers_and_alignment_are_errors_not_crashes(lib):
+    from flash_attn import flash_attn_gfx950 as be
+    a = _valid_fwd_args(be)
+    assert lib.fa_fwd(ctypes.byref(a)) == -1 and b"NULL" in lib.fa_last_error()
+    for f in ("q", "k", "v", "o", "softmax_lse", "cu_seqlens_q", "cu_seqlens_k"):
+        setattr(a, f, 0x1000)
+    a.q = 0x1008
+    assert lib.fa_fwd(ctypes.byref(a)) == -1 and b"aligned" in lib.fa_last_error()
+    a.q = 0x1000
+    a.k_row_stride = 70
+    assert lib.fa_fwd(ctypes.byref(a)) == -1 and b"strides" in lib.fa_last_error()
+    a.k_row_stride = 64
+    a.blockmask = 0x1000  # dense entry point refuses a blockmask, block entry point refuses its absence
+    assert lib.fa_fwd(ctypes.byref(a)) == -1 and b"blockmask" in lib.fa_last_error()
+    a.blockmask = None
+    assert lib.fa_fwd_block(ctypes.byref(a)) == -1 and b"blockmask" in lib.fa_last_error()
+    assert lib.fa_fwd(None) == -1
+
+
+def test_block_sparse_needs_workspace_and_rejects_causal(lib):
+    from flash_attn import flash_attn_gfx950 as be
+    a = _valid_fwd_args(be)
+    for f in ("q", "k", "v", "o", "softmax_lse", "cu_seqlens_q", "cu_seqlens_k", "blockmask"):
+        setattr(a, f, 0x1000)
+    assert lib.fa_fwd_workspace_bytes(ctypes.byref(a)) > 0
+    assert lib.fa_fwd_block(ctypes.byref(a)) == -2 and b"workspace" in lib.fa_last_error()
+    a.is_causal = 1
+    assert lib.fa_fwd_block(ctypes.byref(a)) == -1 and b"causal" in lib.fa_last_error()
+
+
+def test_workspace_sizes(lib):
+    from flash_attn import flash_attn_gfx950 as be
+    a = _valid_fwd_args(be)
+    assert lib.fa_fwd_workspace_bytes(ctypes.byref(a)) == 0  # the dense forward needs no scratch (no o_tmp)
+    g = be.BwdArgs()
+    g.struct_bytes = ctypes.sizeof(g)
+    g.batch, g.nheads, g.head_dim, g.total_q, g.total_k = 2, 3, 64, 100, 100
+    g.max_seqlen_q = g.max_seqlen_k = 64
+    assert lib.fa_bwd_workspace_bytes(ctypes.byref(g)) == 100 * 3 * 64 * 4  # the fp32 dq accumulator (dq_tmp)
+
+
+@pytest.mark.parametrize("d,sq,sk,sparse,want", [
+    (64, 1, 1, False, (16, 128)),          # fmha_api.cpp:235-236
+    (64, 128, 129, False, (128, 256)),     # :237-238
+    (64, 500, 500, False, (512, 512)),     # :234 with blocksize_c = 256
+    (64, 513, 513, False, (528, 768)),
+    (128, 300, 300, False, (304, 384)),    # blocksize_c = 128 for head_size 128 off sm80 (:232)
+    (32, 100, 100, True, (112, 256)),      # :509-513
+    (64, 4096, 4096, True, (4096, 4096)),
+    (64, 4097, 4097, True, (4112, 4352)),
+])
+def test_round_seqlens(lib, d, sq, sk, sparse, want):
+    from flash_attn import flash_attn_gfx950 as be
+    assert be.round_seqlens(d, sq, sk, sparse) == want
+
+
+def test_python_checks_raise_runtime_error():
+    """the binding's own checks mirror TORCH_CHECK -> RuntimeError before anything touches a GPU"""
+    from flash_attn import flash_attn_gfx950 as be
+    q = torch.zeros(16, 1, 64, dtype=torch.float32)
+    cu = torch.tensor([0, 16], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="fp16 or bf16"):
+        be.fwd(q, q, q, cu, cu, 16, 16, 0.0, 0.125, False, False, False, None)
+    h = q.half()
+    with pytest.raises(RuntimeError, match="GPU"):
+        be.fwd(h, h, h, cu, cu, 16, 16, 0.0, 0.125, False, False, False, None)
+    with pytest.raises(RuntimeError, match="head_size"):
+        be.fwd(h[..., :48], h[..., :48], h[..., :48], cu, cu, 16, 16, 0.0, 0.125, False, False, False, None)
+
+
+def test_public_signatures_match_the_reference():
+    """names, order and defaults of flash_attn_interface.py:151-252 and flash_blocksparse_attn_interface.py:135-137"""
+    from flash_attn import flash_attn_interface as fi
+    from flash_attn import flash_blocksparse_attn_interface as bi
+    from flash_attn import bert_padding as bp
+
+    def sig(f):
+        return [(n, p.default if p.default is not inspect.Parameter.empty else "<req>")
+                for n, p in inspect.signature(f).parameters.items()]
+
+    assert sig(fi.flash_attn_unpadded_qkvpacked_func) == [
+        ("qkv", "<req>"), ("cu_seqlens", "<req>"), ("max_seqlen", "<req>"), ("dropout_p", "<req>"),
+        ("softmax_scale", None), ("causal", False), ("return_attn_probs", False)]
+    assert sig(fi.flash_attn_unpadded_kvpacked_func) == [
+        ("q", "<req>"), ("kv", "<req>"), ("cu_seqlens_q", "<req>"), ("cu_seqlens_k", "<req>"),
+        ("max_seqlen_q", "<req>"), ("max_seqlen_k", "<req>"), ("dropout_p", "<req>"), ("softmax_scale", None),
+        ("causal", False), ("return_attn_probs", False)]
+    assert sig(fi.flash_attn_unpadded_func) == [
+        ("q", "<req>"), ("k", "<req>"), ("v", "<req>"), ("cu_seqlens_q", "<req>"), ("cu_seqlens_k", "<req>"),
+        ("max_seqlen_q", "<req>"), ("max_seqlen_k", "<req>"), ("dropout_p", "<req>"), ("softmax_scale", None),
+        ("causal", False), ("return_attn_probs", False)]
+    assert sig(fi.flash_attn_func) == [
+        ("qkv", "<req>"), ("cu_seqlens", "<req>"), ("dropout_p", "<req>"), ("max_s", "<req>"),
+        ("softmax_scale", None), ("causal", False), ("return_attn_probs", False)]
+    assert sig(bi.flash_blocksparse_attn_func) == [
+        ("qkv", "<req>"), ("cu_seqlens", "<req>"), ("blockmask", "<req>"), ("dropout_p", "<req>"), ("max_s", "<req>"),
+        ("softmax_scale", None), ("causal", False), ("return_attn_probs", False), ("convert_mask", True)]
+    assert [n for n, _ in sig(bp.unpad_input)] == ["hidden_states", "attention_mask"]
+    assert [n for n, _ in sig(bp.pad_input)] == ["hidden_states", "indices", "batch", "seqlen"]
+    for cls in ("FlashAttnQKVPackedFunc", "FlashAttnKVPackedFunc", "FlashAttnFunc"):
+        assert issubclass(getattr(fi, cls), torch.autograd.Function)
+    from flash_attn import flash_attn_gfx950 as be
+    assert list(inspect.signature(be.fwd).parameters) == [
+        "q", "k", "v", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k", "p_dropout", "softmax_scale",
+        "zero_tensors", "is_causal", "return_softmax", "gen"]                      # fmha_api.cpp:173-186
+    assert list(inspect.signature(be.bwd_block).parameters) == [
+        "dout", "q", "k", "v", "out", "softmax_lse", "dq", "dk", "dv", "cu_seqlens_q", "cu_seqlens_k", "blockmask",
+        "max_seqlen_q", "max_seqlen_k", "p_dropout", "softmax_scale", "is_causal", "gen"]  # fmha_api.cpp:575-594
+
+
+# ---------------------------------------------------------------- host helpers
+def test_convert_blockmask_matches_spec():
+    from flash_attn.flash_blocksparse_attn_interface import convert_blockmask
+    g = torch.Generator().manual_seed(0)
+    for shape in ((1, 1), (3, 2), (7, 5), (16, 4), (256, 16)):
+        for dens in (0.0, 0.2, 0.6, 1.0):
+            m = torch.rand(shape, generator=g) < dens
+            got = convert_blockmask(m, causal=False)
+            assert got.dtype == torch.int32 and tuple(got.shape) == (shape[1], shape[0])
+            assert np.array_equal(got.numpy(), orc.convert_blockmask_ref(m.numpy()))
+    with pytest.raises(AssertionError):
+        convert_blockmask(torch.ones(2, 2), causal=True)  # flash_blocksparse_attn_interface.py:21
+
+
+def test_unpad_pad_match_spec_and_backprop():
+    from flash_attn.bert_padding import pad_input, unpad_input
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(3, 9, 6, generator=g, dtype=torch.float64, requires_grad=True)
+    lens = torch.tensor([9, 4, 1])
+    mask = torch.arange(9)[None, :] < lens[:, None]
+    rows, idx, cu, mx = unpad_input(x, mask)
+    r_rows, r_idx, r_cu, r_mx = orc.unpad_ref(x.detach().numpy(), mask.numpy())
+    assert np.array_equal(rows.detach().numpy(), r_rows) and np.array_equal(idx.numpy(), r_idx)
+    assert cu.dtype == torch.int32 and cu.tolist() == r_cu.tolist() and mx == r_mx
+    back = pad_input(rows, idx, 3, 9)
+    assert np.array_equal(back.detach().numpy(), orc.pad_ref(r_rows, r_idx, 3, 9))
+    assert torch.equal(back.detach(), x.detach() * mask[..., None])  # pad(unpad(x)) == x o mask
+    w = torch.randn(3, 9, 6, generator=g, dtype=torch.float64)
+    (back * w).sum().backward()
+    assert torch.equal(x.grad, w * mask[..., None])
+
+
+def test_rotary_is_a_rotation_by_position_times_frequency():
+    """closed form of rotary.py:22-42,66-87: pair i at position t is rotated by t * 10000^(-2i/dim)."""
+    from flash_attn.rotary import RotaryEmbedding, RotaryEmbedding2D
+    dim, S = 8, 5
+    rot = RotaryEmbedding(dim)
+    g = torch.Generator().manual_seed(2)
+    q = torch.randn(2, 3, S, dim, generator=g, dtype=torch.float64)
+    k = torch.randn(2, 3, S, dim, generator=g, dtype=torch.float64)
+    rq, rk = rot(q, k)
+    t = torch.arange(S, dtype=torch.float64)[:, None]
+    ang = t * (10000.0 ** (-torch.arange(0, dim, 2, dtype=torch.float64) / dim))[None, :]
+    zq = torch.view_as_complex(q.reshape(2, 3, S, dim // 2, 2).contiguous()) * torch.polar(torch.ones_like(ang), ang)
+    assert torch.allclose(torch.view_as_real(zq).reshape(2, 3, S, dim), rq, atol=1e-6)
+    # norms are preserved and q.k depends only on relative position
+    assert torch.allclose(rq.norm(dim=-1), q.norm(dim=-1), atol=1e-6)
+    q1 = torch.randn(dim, generator=g, dtype=torch.float64).expand(1, 1, S, dim).contiguous()
+    k1 = torch.randn(dim, generator=g, dtype=torch.float64).expand(1, 1, S, dim).contiguous()
+    a, b = RotaryEmbedding(dim)(q1, k1)
+    dots = a[0, 0] @ b[0, 0].T
+    assert torch.allclose(dots[1, 0], dots[3, 2], atol=1e-6) and torch.allclose(dots[0, 2], dots[2, 4], atol=1e-6)
+    # layout (b, s, h, d) gives the same numbers as (b, h, s, d)
+    rq2, _ = RotaryEmbedding(dim)(q.transpose(1, 2), k.transpose(1, 2), seq_dimension=-3)
+    assert torch.allclose(rq2.transpose(1, 2), rq, atol=1e-12)
+    # 2-D: first half of the channels rotates with the column index, second half with the row index
+    side = 3
+    x = torch.randn(1, 2, side * side, 8, generator=g, dtype=torch.float64)
+    r2, _ = RotaryEmbedding2D(8)(x, x)
+    one = RotaryEmbedding(4)
+    grid = x.reshape(1, 2, side, side, 8)
+    cols, _ = one(grid[..., :4], grid[..., :4], seq_dimension=-2)
+    rows, _ = RotaryEmbedding(4)(grid[..., 4:].transpose(2, 3), grid[..., 4:].transpose(2, 3), seq_dimension=-2)
+    want = torch.cat([cols, rows.transpose(2, 3)], dim=-1).reshape(1, 2, side * side, 8)
+    assert torch.allclose(r2, want, atol=1e-12)

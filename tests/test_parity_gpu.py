@@ -1,0 +1,532 @@
+"""GPU parity tests: the HIP kernels (called through the ctypes binding of the C ABI) against the CPU oracle on the
+same seeded inputs.
+
+Tolerance (stated by the build's target): for every output X in {out, dq, dk, dv}
+    max|X_ours - X_ref32| <= 2 * max|X_half - X_ref32| + floor
+where X_ref32 is the fp32 closed form (oracle), X_half the same closed form evaluated by PyTorch in the input dtype
+(fp16/bf16) on the GPU, and floor = 1e-3 (fp16) / 8e-3 (bf16) absorbs outputs that are exactly representable in the
+half evaluation.  softmax_lse is fp32 on both sides: |lse_ours - lse_ref32| <= 2e-3 (fp16 inputs are exact; the
+difference is accumulation order and exp2/log2 approximations).  Dropout masks are compared bit for bit.
+"""
+import ctypes
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+FLOOR = {torch.float16: 1e-3, torch.bfloat16: 8e-3}
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu(lib):
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+
+
+def _cu(lens, device="cuda"):
+    return torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32, device=device)
+
+
+def _inputs(lens_q, lens_k, H, D, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    tq, tk = sum(lens_q), sum(lens_k)
+    mk = lambda n: torch.randn(n, H, D, generator=g).to(dtype)
+    return mk(tq), mk(tk), mk(tk), mk(tq)
+
+
+def half_attention(q, k, v, cu_q, cu_k, scale, causal, keep_mask=None, p=0.0, layout=None, dout=None):
+    """the closed form evaluated in the tensors' own half dtype by PyTorch (the error yardstick)"""
+    q, k, v = (x.detach().clone().requires_grad_(dout is not None) for x in (q, k, v))
+    outs = []
+    for b in range(len(cu_q) - 1):
+        qb = q[cu_q[b]:cu_q[b + 1]].transpose(0, 1)
+        kb = k[cu_k[b]:cu_k[b + 1]].transpose(0, 1)
+        vb = v[cu_k[b]:cu_k[b + 1]].transpose(0, 1)
+        s = torch.matmul(qb, kb.transpose(1, 2)) * scale
+        valid = orc._score_mask(qb.shape[1], kb.shape[1], causal, layout, q.device)
+        s = s.masked_fill(~valid[None], float("-inf"))
+        empty = ~valid.any(-1)
+        s = s.masked_fill(empty[None, :, None], 0.0)
+        pr = torch.softmax(s, dim=-1)
+        pr = pr.masked_fill(~valid[None], 0.0)
+        if keep_mask is not None:
+            pr = pr * keep_mask[b].to(device=q.device, dtype=pr.dtype) / (1.0 - p)
+        outs.append(torch.matmul(pr, vb).transpose(0, 1))
+    out = torch.cat(outs, 0)
+    res = {"out": out.detach()}
+    if dout is not None:
+        out.backward(dout)
+        res.update(dq=q.grad, dk=k.grad, dv=v.grad)
+    return res
+
+
+def _maxerr(a, b):
+    return (a.float().cpu() - b.float().cpu()).abs().max().item()
+
+
+def check_against_oracle(ours, ref, half, dtype, names=("out", "dq", "dk", "dv"), what=""):
+    for n in names:
+        e_ours, e_half = _maxerr(ours[n], ref[n]), _maxerr(half[n], ref[n])
+        assert e_ours <= 2 * e_half + FLOOR[dtype], "%s %s: ours %.3e vs half-precision PyTorch %.3e" % (what, n, e_ours, e_half)
+
+
+def run_ours(q, k, v, do, cu_q, cu_k, max_q, max_k, p, scale, causal, packing="sep", probs=False):
+    from flash_attn import flash_attn_interface as fi
+    dev = "cuda"
+    cu_q, cu_k = cu_q.to(dev), cu_k.to(dev)
+    if packing == "qkv":
+        qkv = torch.stack([q, k, v], 1).to(dev).requires_grad_()
+        res = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu_q, max_q, p, scale, causal, probs)
+    elif packing == "kv":
+        qg = q.to(dev).requires_grad_()
+        kv = torch.stack([k, v], 1).to(dev).requires_grad_()
+        res = fi.flash_attn_unpadded_kvpacked_func(qg, kv, cu_q, cu_k, max_q, max_k, p, scale, causal, probs)
+    else:
+        qg, kg, vg = (x.to(dev).requires_grad_() for x in (q, k, v))
+        res = fi.flash_attn_unpadded_func(qg, kg, vg, cu_q, cu_k, max_q, max_k, p, scale, causal, probs)
+    out = res[0] if probs else res
+    out.backward(do.to(dev))
+    torch.cuda.synchronize()
+    if packing == "qkv":
+        dq, dk, dv = qkv.grad[:, 0], qkv.grad[:, 1], qkv.grad[:, 2]
+    elif packing == "kv":
+        dq, dk, dv = qg.grad, kv.grad[:, 0], kv.grad[:, 1]
+    else:
+        dq, dk, dv = qg.grad, kg.grad, vg.grad
+    r = {"out": out.detach(), "dq": dq, "dk": dk, "dv": dv}
+    if probs:
+        r["lse"], r["S_dmask"] = res[1], res[2]
+    return r
+
+
+def _parity_case(lens_q, lens_k, H, D, dtype, causal, packing="sep", seed=0, scale=None, max_pad=0):
+    q, k, v, do = _inputs(lens_q, lens_k, H, D, dtype, seed)
+    cu_q, cu_k = _cu(lens_q, "cpu"), _cu(lens_k, "cpu")
+    sc = D ** -0.5 if scale is None else scale
+    ours = run_ours(q, k, v, do, cu_q, cu_k, max(lens_q) + max_pad, max(lens_k) + max_pad, 0.0, scale, causal, packing,
+                    probs=True)
+    ref = orc.varlen_attention(q, k, v, cu_q, cu_k, sc, causal, dout=do)
+    half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu_q.tolist(), cu_k.tolist(), sc, causal, dout=do.cuda())
+    what = "q%s k%s H%d D%d %s causal=%s %s" % (lens_q, lens_k, H, D, dtype, causal, packing)
+    check_against_oracle(ours, ref, half, dtype, what=what)
+    for b, L in enumerate(lens_q):  # lse: only rows < seqlen_q are defined
+        got = ours["lse"][b, :, :L].cpu()
+        want = ref["lse"][b]
+        fin = torch.isfinite(want)
+        assert torch.equal(torch.isfinite(got), fin), what
+        assert (got[fin] - want[fin]).abs().max().item() <= 2e-3 if fin.any() else True, what
+    return ours, ref
+
+
+# ------------------------------------------------------------------------------------------------
+# seeded parity at oracle-friendly sizes: every head dim, both dtypes, causal, ragged lengths, packings
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("D", [16, 32, 64, 128])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+def test_parity_head_dims(D, dtype, causal):
+    _parity_case([113, 256, 37], [113, 256, 37], 3, D, dtype, causal, packing="qkv", seed=D)
+
+
+@pytest.mark.parametrize("lens_q,lens_k", [
+    ([1], [1]),                      # single token
+    ([1, 1, 1], [300, 1, 17]),       # decode-like: one query per sequence
+    ([15, 17, 16], [15, 17, 16]),    # around the 16-row granularity
+    ([128, 129, 127], [128, 129, 127]),
+    ([64, 200], [300, 65]),          # seqlen_q != seqlen_k
+    ([257], [513]),
+])
+@pytest.mark.parametrize("causal", [False, True])
+def test_parity_ragged_shapes(lens_q, lens_k, causal):
+    _parity_case(lens_q, lens_k, 2, 64, torch.float16, causal, packing="kv", seed=len(lens_q))
+
+
+def test_parity_separate_qkv_and_scale():
+    _parity_case([100, 140], [90, 260], 4, 32, torch.bfloat16, False, packing="sep", seed=5, scale=0.3)
+    _parity_case([100, 140], [100, 140], 4, 32, torch.float16, True, packing="sep", seed=6, scale=0.05)
+
+
+def test_max_seqlen_may_exceed_the_longest_sequence():
+    _parity_case([70, 33], [70, 33], 2, 64, torch.float16, False, packing="qkv", seed=7, max_pad=200)
+
+
+def test_cpu_reference_config():
+    """BASELINE config 1 (the reference's CPU-runnable case): B=2, H=12, d=64, N=128, packed qkv, non-causal, p=0."""
+    _parity_case([128, 128], [128, 128], 12, 64, torch.float16, False, packing="qkv", seed=0)
+
+
+def test_golden_fixture():
+    z = np.load(os.path.join(GOLDEN, "attention_small.npz"))
+    lens = z["lens"].tolist()
+    cu = torch.tensor(z["cu_seqlens"])
+    for dtype in (torch.float16, torch.bfloat16):
+        q, k, v, do = (torch.tensor(z[n]).to(dtype) for n in ("q", "k", "v", "dout"))  # exact in both dtypes
+        for causal, tag in ((False, "dense"), (True, "causal")):
+            ours = run_ours(q, k, v, do, cu, cu, max(lens), max(lens), 0.0, None, causal, "sep", probs=True)
+            ref = {n: torch.tensor(z["%s_%s" % (tag, n)]) for n in ("out", "dq", "dk", "dv")}
+            half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu.tolist(), cu.tolist(), 16 ** -0.5, causal, dout=do.cuda())
+            check_against_oracle(ours, ref, half, dtype, what="golden " + tag)
+            for b in range(2):
+                assert (ours["lse"][b, :, :lens[b]].cpu() - torch.tensor(z["%s_lse%d" % (tag, b)])).abs().max() < 2e-3
+
+
+def test_softmax_d_and_raw_c_abi():
+    """calls fa_fwd / fa_bwd with raw pointers (no interface layer) and checks softmax_d = rowsum(dO o O)."""
+    from flash_attn import flash_attn_gfx950 as be
+    lens = [50, 77]
+    q, k, v, do = (x.cuda() for x in _inputs(lens, lens, 2, 64, torch.float16, 11))
+    cu = _cu(lens)
+    o, lse = be.fwd(q, k, v, cu, cu, 77, 77, 0.0, 0.125, False, False, False, None)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    _, _, _, sd = be.bwd(do, q, k, v, o, lse, dq, dk, dv, cu, cu, 77, 77, 0.0, 0.125, False, False, None)
+    torch.cuda.synchronize()
+    assert tuple(lse.shape) == (2, 2, 80) and tuple(sd.shape) == (2, 2, 80)
+    ref = orc.varlen_attention(q.cpu(), k.cpu(), v.cpu(), cu.tolist(), cu.tolist(), 0.125, False, dout=do.cpu())
+    for b, L in enumerate(lens):
+        assert (sd[b, :, :L].cpu() - ref["softmax_d"][b]).abs().max() < 2e-2
+    assert _maxerr(dq, ref["dq"]) < 5e-3 and _maxerr(o, ref["out"]) < 2e-3
+    # zero_tensors pre-fills what the kernels do not write (fmha_api.cpp:256-260): lse padding becomes -inf
+    o2, lse2 = be.fwd(q, k, v, cu, cu, 77, 77, 0.0, 0.125, True, False, False, None)
+    torch.cuda.synchronize()
+    assert torch.equal(o2, o) and torch.isinf(lse2[0, :, 50:]).all() and torch.equal(lse2[1, :, :77], lse[1, :, :77])
+
+
+def test_strided_views_and_noncontiguous_grads():
+    """q, k, v as views of a packed tensor with extra padding between rows (row stride != 3*H*D)."""
+    from flash_attn import flash_attn_gfx950 as be
+    lens = [40, 90]
+    H, D = 2, 64
+    tot = sum(lens)
+    g = torch.Generator().manual_seed(3)
+    big = torch.randn(tot, 4, H, D + 8, generator=g).half().cuda()
+    q, k, v = big[:, 0, :, :D], big[:, 1, :, :D], big[:, 3, :, :D]
+    cu = _cu(lens)
+    o, lse = be.fwd(q, k, v, cu, cu, 90, 90, 0.0, 0.125, False, True, False, None)
+    o_c, _ = be.fwd(q.contiguous(), k.contiguous(), v.contiguous(), cu, cu, 90, 90, 0.0, 0.125, False, True, False, None)
+    torch.cuda.synchronize()
+    assert torch.equal(o, o_c)
+    do = torch.randn(tot, H, D, generator=g).half().cuda()
+    dbig = torch.zeros_like(big)
+    be.bwd(do, q, k, v, o, lse, dbig[:, 0, :, :D], dbig[:, 1, :, :D], dbig[:, 3, :, :D], cu, cu, 90, 90, 0.0, 0.125,
+           False, True, None)
+    dq, dk, dv = (torch.empty(tot, H, D, dtype=torch.half, device="cuda") for _ in range(3))
+    be.bwd(do, q.contiguous(), k.contiguous(), v.contiguous(), o, lse, dq, dk, dv, cu, cu, 90, 90, 0.0, 0.125, False,
+           True, None)
+    torch.cuda.synchronize()
+    assert torch.equal(dbig[:, 1, :, :D], dk) and torch.equal(dbig[:, 3, :, :D], dv)
+    assert (dbig[:, 0, :, :D].float() - dq.float()).abs().max() < 2e-3  # dq sums fp32 atomics: order may differ
+    assert dbig[:, 2].abs().max() == 0 and dbig[..., D:].abs().max() == 0  # nothing written outside the views
+
+
+def test_error_behaviour_on_device():
+    from flash_attn import flash_attn_gfx950 as be
+    q = torch.zeros(16, 1, 64, dtype=torch.half, device="cuda")
+    cu = torch.tensor([0, 16], dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="p_dropout"):
+        be.fwd(q, q, q, cu, cu, 16, 16, 1.0, 0.125, False, False, False, None)          # fmha_api.cpp:113
+    with pytest.raises(RuntimeError, match="int32"):
+        be.fwd(q, q, q, cu.long(), cu, 16, 16, 0.0, 0.125, False, False, False, None)   # :201
+    with pytest.raises(RuntimeError, match="contiguous last"):
+        qt = torch.zeros(16, 1, 128, dtype=torch.half, device="cuda")[..., ::2]
+        be.fwd(qt, qt, qt, cu, cu, 16, 16, 0.0, 0.125, False, False, False, None)       # :210
+    with pytest.raises(RuntimeError, match="shape"):
+        be.fwd(q, q[:8], q, cu, cu, 16, 16, 0.0, 0.125, False, False, False, None)      # CHECK_SHAPE :227
+    # an empty sequence in the batch is skipped, not an error
+    cu2 = torch.tensor([0, 0, 16], dtype=torch.int32, device="cuda")
+    o, lse = be.fwd(q, q, q, cu2, cu2, 16, 16, 0.0, 0.125, False, False, False, None)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o).all()
+
+
+# ------------------------------------------------------------------------------------------------
+# dropout: exact mask, exact algebra with that mask, keep rate, RNG semantics
+# ------------------------------------------------------------------------------------------------
+def _gen_state():
+    g = torch.cuda.default_generators[torch.cuda.current_device()]
+    return g.initial_seed(), g.get_offset()
+
+
+@pytest.mark.parametrize("D,dtype,causal", [(64, torch.float16, False), (32, torch.bfloat16, True), (128, torch.float16, False)])
+def test_dropout_mask_is_the_defined_one_and_is_applied(D, dtype, causal):
+    p = 0.17
+    lens_q, lens_k, H = [70, 130], [70, 130], 3
+    q, k, v, do = _inputs(lens_q, lens_k, H, D, dtype, 21)
+    cu = _cu(lens_q, "cpu")
+    torch.manual_seed(1234)
+    seed, offset = _gen_state()
+    ours = run_ours(q, k, v, do, cu, cu, 130, 130, p, None, causal, "qkv", probs=True)
+    S = ours["S_dmask"].cpu()
+    sq_r, sk_r = S.shape[2], S.shape[3]
+    assert (sq_r, sk_r) == (144, 256)
+    masks = []
+    ref_plain = orc.varlen_attention(q, k, v, cu, cu, None, causal)
+    for b, L in enumerate(lens_q):
+        mb = np.stack([orc.dropout_keep_mask(seed, offset, b * H + h, L, L, p) for h in range(H)])
+        masks.append(torch.tensor(mb))
+        dropped = torch.signbit(S[b, :, :L, :L])
+        valid = orc._score_mask(L, L, causal, None)
+        assert torch.equal(dropped[:, valid], ~masks[b][:, valid]), "mask differs from its definition"
+        assert (S[b, :, :L, :L].abs().float() - ref_plain["probs"][b]).abs().max() < (3e-3 if dtype == torch.float16 else 1.6e-2)
+        assert S[b, :, L:, :].abs().max() == 0 and S[b, :, :, L:].abs().max() == 0  # padding region is zero
+    # o and the gradients equal the closed form with exactly that mask
+    ref = orc.varlen_attention(q, k, v, cu, cu, None, causal, p_dropout=p, keep_mask=masks, dout=do)
+    half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu.tolist(), cu.tolist(), D ** -0.5, causal, masks, p, dout=do.cuda())
+    check_against_oracle(ours, ref, half, dtype, what="dropout D%d" % D)
+
+
+def test_dropout_keep_rate_and_rng_semantics():
+    from flash_attn import flash_attn_interface as fi
+    p, N, H, D = 0.1, 512, 4, 64
+    qkv = torch.randn(2 * N, 3, H, D, device="cuda", dtype=torch.float16)
+    cu = _cu([N, N])
+    torch.manual_seed(7)
+    _, _, S1 = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, p, None, False, True)
+    _, _, S2 = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, p, None, False, True)
+    torch.manual_seed(7)
+    _, _, S3 = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, p, None, False, True)
+    k1, k2, k3 = (~torch.signbit(s) for s in (S1, S2, S3))
+    assert torch.equal(k1, k3), "same seed must give the same mask"
+    assert not torch.equal(k1, k2), "successive calls must draw different masks"
+    n = k1.numel()
+    kp = orc.keep_probability(p)
+    z = (k1.sum().item() - n * kp) / math.sqrt(n * kp * (1 - kp))
+    assert abs(z) < 4.5, "keep rate off: z = %.2f" % z
+    per_head = k1.float().mean(dim=(2, 3))
+    assert (per_head - kp).abs().max() < 5e-3
+
+
+def test_dropout_backward_reuses_the_forward_mask_without_probs():
+    """production path (no S_dmask): gradients must match the closed form under the mask defined by the state the
+    generator had when the forward ran, even after other draws moved the generator on."""
+    p, lens, H, D = 0.25, [96, 200], 2, 64
+    q, k, v, do = _inputs(lens, lens, H, D, torch.float16, 31)
+    cu = _cu(lens, "cpu")
+    from flash_attn import flash_attn_interface as fi
+    torch.manual_seed(99)
+    seed, offset = _gen_state()
+    qkv = torch.stack([q, k, v], 1).cuda().requires_grad_()
+    out = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu.cuda(), 200, p)
+    torch.rand(1000, device="cuda")  # advances the generator between forward and backward
+    after = _gen_state()
+    out.backward(do.cuda())
+    assert _gen_state() == after, "backward must leave the generator where it found it"
+    masks = [torch.tensor(np.stack([orc.dropout_keep_mask(seed, offset, b * H + h, L, L, p) for h in range(H)]))
+             for b, L in enumerate(lens)]
+    ref = orc.varlen_attention(q, k, v, cu, cu, None, False, p_dropout=p, keep_mask=masks, dout=do)
+    half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu.tolist(), cu.tolist(), D ** -0.5, False, masks, p, dout=do.cuda())
+    ours = {"out": out.detach(), "dq": qkv.grad[:, 0], "dk": qkv.grad[:, 1], "dv": qkv.grad[:, 2]}
+    check_against_oracle(ours, ref, half, torch.float16, what="dropout production path")
+
+
+# ------------------------------------------------------------------------------------------------
+# block-sparse
+# ------------------------------------------------------------------------------------------------
+def _layout(nrow, ncol, density, seed):
+    g = torch.Generator().manual_seed(seed)
+    band = (torch.arange(nrow)[:, None] // 16 - torch.arange(ncol)[None, :]).abs() <= 0
+    return (band | (torch.rand(nrow, ncol, generator=g) < density))
+
+
+@pytest.mark.parametrize("D,N,p", [(64, 512, 0.0), (32, 700, 0.0), (16, 300, 0.0), (64, 512, 0.2)])
+def test_blocksparse_parity(D, N, p):
+    from flash_attn.flash_blocksparse_attn_interface import flash_blocksparse_attn_func
+    from flash_attn import flash_attn_gfx950 as be
+    H, lens = 2, [N, N - 37]
+    sq_r, sk_r = be.round_seqlens(D, N, N, True)
+    layout = _layout(sq_r // 16, sk_r // 256, 0.3, N)
+    layout[3] = False  # a row block with no active tile: its rows must come out as zeros
+    q, k, v, do = _inputs(lens, lens, H, D, torch.float16, N)
+    cu = _cu(lens, "cpu")
+    qkv = torch.stack([q, k, v], 1).cuda().requires_grad_()
+    torch.manual_seed(5)
+    seed, offset = _gen_state()
+    ctx, S, lse = flash_blocksparse_attn_func(qkv, cu.cuda(), layout.cuda(), p, N, None, False, True)
+    ctx.backward(do.cuda())
+    torch.cuda.synchronize()
+    masks = None
+    if p > 0:
+        masks = [torch.tensor(np.stack([orc.dropout_keep_mask(seed, offset, b * H + h, L, L, p) for h in range(H)]))
+                 for b, L in enumerate(lens)]
+    ref = orc.varlen_attention(q, k, v, cu, cu, None, False, p_dropout=p, keep_mask=masks, layout=layout.numpy(), dout=do)
+    half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu.tolist(), cu.tolist(), D ** -0.5, False, masks, p,
+                          layout=layout.numpy(), dout=do.cuda())
+    ours = {"out": ctx.detach(), "dq": qkv.grad[:, 0], "dk": qkv.grad[:, 1], "dv": qkv.grad[:, 2]}
+    check_against_oracle(ours, ref, half, torch.float16, what="blocksparse D%d N%d" % (D, N))
+    assert ctx[48:64].abs().max() == 0 and torch.isinf(lse[0, :, 48:64]).all()
+    assert qkv.grad[48:64, 0].abs().max() == 0
+    # probabilities are zero on inactive blocks
+    full = orc.expand_block_layout(layout.numpy(), lens[0], lens[0])
+    assert S[0, :, :lens[0], :lens[0]].cpu()[:, ~full].abs().max() == 0
+
+
+def test_blocksparse_full_layout_equals_dense():
+    from flash_attn.flash_blocksparse_attn_interface import flash_blocksparse_attn_func
+    from flash_attn.flash_attn_interface import flash_attn_unpadded_qkvpacked_func
+    N, H, D = 600, 2, 64
+    qkv = torch.randn(2 * N, 3, H, D, device="cuda", dtype=torch.float16)
+    cu = _cu([N, N])
+    layout = torch.ones(608 // 16, 768 // 256, device="cuda")
+    a = flash_blocksparse_attn_func(qkv, cu, layout, 0.0, N)
+    b = flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
+# ------------------------------------------------------------------------------------------------
+# modules
+# ------------------------------------------------------------------------------------------------
+def test_flash_attention_module_three_input_modes():
+    from flash_attn.flash_attention import FlashAttention
+    B, S, H, D = 3, 96, 2, 64
+    g = torch.Generator().manual_seed(8)
+    qkv = torch.randn(B, S, 3, H, D, generator=g).half()
+    lens = torch.tensor([96, 40, 7])
+    mask = torch.arange(S)[None, :] < lens[:, None]
+    m = FlashAttention().eval()
+
+    class KPM:
+        bool_matrix = mask.cuda()
+
+    ref = orc.attention_ref(qkv, mask, 0.0, upcast=True, causal=True).float()
+    out_pad, _ = m(qkv.cuda(), key_padding_mask=KPM(), causal=True)
+    assert tuple(out_pad.shape) == (B, S, H, D)
+    assert (out_pad.cpu().float() - ref)[mask].abs().max() < 2e-3
+    assert out_pad.cpu()[~mask].abs().max() == 0
+    full = torch.ones(B, S, dtype=torch.bool)
+    out_full, _ = m(qkv.cuda(), causal=False)
+    assert (out_full.cpu().float() - orc.attention_ref(qkv, full, 0.0, upcast=True).float()).abs().max() < 2e-3
+    packed = torch.cat([qkv[b, :lens[b]] for b in range(B)], 0).cuda()
+    out_packed, _ = m(packed, cu_seqlens=_cu(lens.tolist()), max_s=96, causal=True)
+    assert torch.equal(out_packed, out_pad[mask.cuda()])
+
+
+def test_flash_mha_matches_torch_multihead_attention():
+    from flash_attn.flash_attention import FlashMHA
+    torch.manual_seed(0)
+    E, H, B, S = 128, 4, 2, 50
+    mha = FlashMHA(E, H, device="cuda", dtype=torch.float16).eval()
+    ref = torch.nn.MultiheadAttention(E, H, batch_first=True, device="cuda", dtype=torch.float32)
+    with torch.no_grad():
+        ref.in_proj_weight.copy_(mha.Wqkv.weight.float())
+        ref.in_proj_bias.copy_(mha.Wqkv.bias.float())
+        ref.out_proj.weight.copy_(mha.out_proj.weight.float())
+        ref.out_proj.bias.copy_(mha.out_proj.bias.float())
+    x = torch.randn(B, S, E, device="cuda", dtype=torch.float16)
+    y, _ = mha(x, None, None)
+    y_ref, _ = ref(x.float(), x.float(), x.float(), need_weights=False)
+    assert (y.float() - y_ref).abs().max() < 1e-2
+    y.sum().backward()
+    assert mha.Wqkv.weight.grad is not None and torch.isfinite(mha.Wqkv.weight.grad).all()
+    rot = FlashMHA(E, H, use_rotary_emb="1d", causal=True, device="cuda", dtype=torch.float16).eval()
+    y2, _ = rot(x, None, None)
+    assert tuple(y2.shape) == (B, S, E) and torch.isfinite(y2).all()
+
+
+# ------------------------------------------------------------------------------------------------
+# BASELINE configurations at full size: fp32 PyTorch on the GPU as the reference, plus size-independent properties
+# ------------------------------------------------------------------------------------------------
+def _full_size_check(lens, H, D, dtype, causal, p=0.0, seed=0):
+    q, k, v, do = (x.cuda() for x in _inputs(lens, lens, H, D, dtype, seed))
+    cu = _cu(lens, "cpu")
+    torch.manual_seed(seed)
+    seed_, offset = _gen_state()
+    ours = run_ours(q, k, v, do, cu, cu, max(lens), max(lens), p, None, causal, "qkv", probs=False)
+    masks = None
+    if p > 0:
+        masks = [torch.tensor(np.stack([orc.dropout_keep_mask(seed_, offset, b * H + h, L, L, p) for h in range(H)]))
+                 for b, L in enumerate(lens)]
+    ref = orc.varlen_attention(q, k, v, cu, cu, None, causal, p_dropout=p, keep_mask=masks, dout=do)  # fp32 on the GPU
+    half = half_attention(q, k, v, cu.tolist(), cu.tolist(), D ** -0.5, causal, masks, p, dout=do)
+    check_against_oracle(ours, ref, half, dtype, what="full size %s" % ((len(lens), H, D, max(lens), causal, p),))
+    return q, k, v, do, cu, ours
+
+
+def test_config_bert_varlen_dropout():
+    """BASELINE config 2: fp16, B=8, H=12, d=64, lengths uniform in [256, 512], p=0.1."""
+    g = torch.Generator().manual_seed(0)
+    lens = torch.randint(256, 513, (8,), generator=g).tolist()
+    _full_size_check(lens, 12, 64, torch.float16, False, p=0.1, seed=2)
+
+
+@pytest.mark.parametrize("N", [1024, 2048, 4096])
+def test_config_gpt2_causal_bf16(N):
+    """BASELINE config 3: bf16, B=8, H=12, d=64, causal."""
+    q, k, v, do, cu, ours = _full_size_check([N] * 8, 12, 64, torch.bfloat16, True, seed=N)
+    # causal first row of every sequence attends to key 0 only: o = v0 exactly
+    first = torch.arange(0, 8 * N, N, device="cuda")
+    assert torch.equal(ours["out"][first], v[first])
+
+
+def test_headline_config_fp16():
+    """the configuration the metric is quoted on: fp16, B=8, H=12, d=64, N=2048, non-causal, p=0."""
+    _full_size_check([2048] * 8, 12, 64, torch.float16, False, seed=1)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_config_head_dim_128(causal):
+    """BASELINE config 4: fp16, B=16, H=12, d=128, N=2048."""
+    _full_size_check([2048] * 16, 12, 128, torch.float16, causal, seed=4)
+
+
+def test_config_blocksparse_long_sequence():
+    """BASELINE config 5: fp16, B=4, H=16, d=64, N=4096, ~25% density band + random blocks."""
+    from flash_attn.flash_blocksparse_attn_interface import flash_blocksparse_attn_func
+    B, H, D, N = 4, 16, 64, 4096
+    g = torch.Generator().manual_seed(0)
+    nrow, ncol = N // 16, N // 256
+    band = (torch.arange(nrow)[:, None] // 16 - torch.arange(ncol)[None, :]).abs() <= 1
+    layout = band | (torch.rand(nrow, ncol, generator=g) < 0.08)
+    assert 0.2 < layout.float().mean() < 0.3
+    lens = [N] * B
+    q, k, v, do = (x.cuda() for x in _inputs(lens, lens, H, D, torch.float16, 5))
+    cu = _cu(lens, "cpu")
+    qkv = torch.stack([q, k, v], 1).requires_grad_()
+    out = flash_blocksparse_attn_func(qkv, cu.cuda(), layout.cuda(), 0.0, N)
+    out.backward(do)
+    torch.cuda.synchronize()
+    ours = {"out": out.detach(), "dq": qkv.grad[:, 0], "dk": qkv.grad[:, 1], "dv": qkv.grad[:, 2]}
+    ref = orc.varlen_attention(q, k, v, cu, cu, None, False, layout=layout.numpy(), dout=do)
+    half = half_attention(q, k, v, cu.tolist(), cu.tolist(), D ** -0.5, False, layout=layout.numpy(), dout=do)
+    check_against_oracle(ours, ref, half, torch.float16, what="blocksparse N4096")
+
+
+def test_size_independent_properties_at_full_size():
+    """varlen == per-sequence dense; batch permutation; linearity in V; uniform attention for q = 0."""
+    from flash_attn.flash_attn_interface import flash_attn_unpadded_func
+    H, D = 12, 64
+    g = torch.Generator().manual_seed(3)
+    lens = torch.randint(256, 2049, (8,), generator=g).tolist()
+    q, k, v, do = (x.cuda() for x in _inputs(lens, lens, H, D, torch.float16, 9))
+    cu = _cu(lens)
+    mx = max(lens)
+    out = flash_attn_unpadded_func(q, k, v, cu, cu, mx, mx, 0.0, None, True)
+    offs = [0] + list(np.cumsum(lens))
+    # (1) packed result == each sequence run alone (bitwise: same tiles, same order)
+    for b in (0, 3, 7):
+        sl = slice(offs[b], offs[b + 1])
+        one = flash_attn_unpadded_func(q[sl], k[sl], v[sl], _cu([lens[b]]), _cu([lens[b]]), lens[b], lens[b], 0.0, None, True)
+        assert torch.equal(one, out[sl])
+    # (2) permuting the batch permutes the result
+    perm = [5, 2, 7, 0, 1, 6, 3, 4]
+    pq, pk, pv = (torch.cat([x[offs[b]:offs[b + 1]] for b in perm]) for x in (q, k, v))
+    pout = flash_attn_unpadded_func(pq, pk, pv, _cu([lens[b] for b in perm]), _cu([lens[b] for b in perm]), mx, mx, 0.0, None, True)
+    assert torch.equal(pout, torch.cat([out[offs[b]:offs[b + 1]] for b in perm]))
+    # (3) linear in V (up to rounding of the half outputs): f(v1 + v2) = f(v1) + f(v2)
+    v2 = torch.randn_like(v)
+    o1 = flash_attn_unpadded_func(q, k, v, cu, cu, mx, mx, 0.0).float()
+    o2 = flash_attn_unpadded_func(q, k, v2, cu, cu, mx, mx, 0.0).float()
+    o12 = flash_attn_unpadded_func(q, k, (v.float() + v2.float()).half(), cu, cu, mx, mx, 0.0).float()
+    assert (o12 - (o1 + o2)).abs().max() < 4e-3
+    # (4) q = 0: uniform weights, o = running/whole mean of v, lse = log(#visible keys)
+    z = torch.zeros_like(q)
+    oz, lse, _ = flash_attn_unpadded_func(z, k, v, cu, cu, mx, mx, 0.0, None, False, True)
+    for b in (1, 4):
+        sl = slice(offs[b], offs[b + 1])
+        assert (oz[sl].float() - v[sl].float().mean(0, keepdim=True)).abs().max() < 2e-3
+        assert (lse[b, :, :lens[b]] - math.log(lens[b])).abs().max() < 1e-4
