@@ -1,0 +1,183 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused attention path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all] [--no-cpu]
+
+One step = one forward + one backward pass of the headline workload (fp16, B=8, H=12, d=64, N=2048, packed qkv,
+non-causal, dropout 0, synthetic N(0,1) data resident in HBM), called through the C ABI.  Prints ONE JSON line:
+whole-job fwd+bwd TFLOP/s (4*B*H*N^2*d forward, 2.5x that backward), the roofline position of the dominant kernel
+(the backward dq/dk/dv kernel, timed with HIP events recorded around it on its stream) and the CPU baseline (the
+oracle's standard attention, fp32 PyTorch on the host cores, timed on a bounded sample of the same workload).
+--all additionally prints, to stderr, a table over the other BASELINE configurations.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "flash-attention_amd"))
+sys.path.insert(0, ROOT)
+
+MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 / bf16
+HBM_PEAK_GBS = 8000.0
+
+
+def attention_flops(B, H, N, D, causal=False):
+    f = 4.0 * B * H * N * N * D
+    return f * (0.5 if causal else 1.0)
+
+
+class Workload:
+    def __init__(self, torch, B, H, D, N, dtype, causal=False, p=0.0, lens=None, seed=0):
+        self.B, self.H, self.D, self.N, self.dtype, self.causal, self.p = B, H, D, N, dtype, causal, p
+        g = torch.Generator(device="cuda").manual_seed(seed)
+        lens = lens or [N] * B
+        self.lens = lens
+        total = sum(lens)
+        self.qkv = torch.randn(total, 3, H, D, device="cuda", dtype=torch.float32, generator=g).to(dtype)
+        self.dout = torch.randn(total, H, D, device="cuda", dtype=torch.float32, generator=g).to(dtype)
+        cu = [0]
+        for L in lens:
+            cu.append(cu[-1] + L)
+        self.cu = torch.tensor(cu, dtype=torch.int32, device="cuda")
+        self.max_s = max(lens)
+        self.dqkv = torch.empty_like(self.qkv)
+        self.scale = D ** -0.5
+        self.fwd_flops = sum(4.0 * H * L * L * D for L in lens) * (0.5 if causal else 1.0)
+        self.bytes_fwd = 4 * total * H * D * 2 + 4 * B * H * self.max_s          # q,k,v read + o written, lse
+        self.bytes_bwd = 8 * total * H * D * 2 + 2 * 4 * B * H * self.max_s      # q,k,v,o,do read + dq,dk,dv written
+
+    def forward(self, be):
+        q, k, v = self.qkv[:, 0], self.qkv[:, 1], self.qkv[:, 2]
+        self.out, self.lse = be.fwd(q, k, v, self.cu, self.cu, self.max_s, self.max_s, self.p, self.scale, False,
+                                    self.causal, False, None)
+
+    def backward(self, be, events=None):
+        q, k, v = self.qkv[:, 0], self.qkv[:, 1], self.qkv[:, 2]
+        dq, dk, dv = self.dqkv[:, 0], self.dqkv[:, 1], self.dqkv[:, 2]
+        be.bwd(self.dout, q, k, v, self.out, self.lse, dq, dk, dv, self.cu, self.cu, self.max_s, self.max_s, self.p,
+               self.scale, False, self.causal, None, main_kernel_events=events)
+
+
+def time_steps(torch, be, w, steps, warmup):
+    for _ in range(warmup):
+        w.forward(be)
+        w.backward(be)
+    torch.cuda.synchronize()
+    ev = lambda: torch.cuda.Event(enable_timing=True)
+    marks = [(ev(), ev(), ev()) for _ in range(steps)]      # step start, after forward, after backward
+    kern = [(ev(), ev()) for _ in range(steps)]             # around the main backward kernel only
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        marks[i][0].record()
+        w.forward(be)
+        marks[i][1].record()
+        w.backward(be, kern[i])
+        marks[i][2].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    fwd_ms = sum(a.elapsed_time(b) for a, b, _ in marks) / steps
+    bwd_ms = sum(b.elapsed_time(c) for _, b, c in marks) / steps
+    bwd_main_ms = sum(a.elapsed_time(b) for a, b in kern) / steps
+    return {"wall_ms": wall_ms, "ms_per_step": wall_ms / steps, "fwd_ms": fwd_ms, "bwd_ms": bwd_ms,
+            "bwd_main_kernel_ms": bwd_main_ms}
+
+
+def cpu_baseline(torch, B, H, D, N, budget_s=20.0):
+    """The oracle's standard attention (attention_ref: fp32, PyTorch ops on the host cores), forward + backward through
+    autograd, on a bounded sample of the headline workload: whole batches of (B, N) are repeated until about
+    `budget_s` seconds of CPU work have been spent (at least one repetition)."""
+    from oracle.attention_oracle import attention_ref
+    torch.manual_seed(0)
+    qkv = torch.randn(B, N, 3, H, D, dtype=torch.float32, requires_grad=True)
+    dout = torch.randn(B, N, H, D, dtype=torch.float32)
+    mask = torch.ones(B, N, dtype=torch.bool)
+    reps, spent = 0, 0.0
+    while reps < 1 or (spent < budget_s and spent + spent / reps < 1.5 * budget_s):
+        t0 = time.perf_counter()
+        out = attention_ref(qkv, mask, 0.0, upcast=True)
+        out.backward(dout)
+        qkv.grad = None
+        spent += time.perf_counter() - t0
+        reps += 1
+    flops = 3.5 * attention_flops(B, H, N, D) * reps
+    return {"value": round(flops / spent / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port", "ms_per_step": round(spent / reps * 1e3, 1),
+            "sample": "%d repetition(s) of the full B=%d H=%d d=%d N=%d fp32 batch, fwd+bwd via autograd, %.1f s of host time"
+                      % (reps, B, H, D, N, spent)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--all", action="store_true", help="also time the other BASELINE configurations (stderr table)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-budget", type=float, default=20.0)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (every (batch, head, tile) is independent; there is no "
+                 "multi-GPU path to measure). Run with --gpus 1.")
+    import torch
+    from flash_attn import flash_attn_gfx950 as be
+    be.load_library()  # fails loudly if the HIP library is not built
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+
+    B, H, D, N = 8, 12, 64, 2048
+    w = Workload(torch, B, H, D, N, torch.float16)
+    t = time_steps(torch, be, w, a.steps, a.warmup)
+    fwd_flops = attention_flops(B, H, N, D)
+    step_flops = 3.5 * fwd_flops
+    value = step_flops / (t["ms_per_step"] * 1e-3) / 1e12
+    bwd_kernel_tflops = 2.5 * fwd_flops / (t["bwd_main_kernel_ms"] * 1e-3) / 1e12
+    res = {
+        "metric": "fwd+bwd TFLOPS, fp16 B8 H12 d64 N=2K (4*B*H*N^2*d fwd, 2.5x bwd)",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(t["ms_per_step"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic N(0,1) q,k,v,dout resident in HBM",
+        "config": {"workload": "headline: fp16 packed qkv [16384,3,12,64], B=8 H=12 d=64 N=2048 equal lengths, "
+                               "non-causal, dropout 0, fwd+bwd with dout~N(0,1)"},
+        "pct_of_mfma_peak": round(100.0 * value / MFMA_PEAK_TFLOPS, 2),
+        "fwd_ms": round(t["fwd_ms"], 4), "bwd_ms": round(t["bwd_ms"], 4),
+        "fwd_tflops": round(fwd_flops / (t["fwd_ms"] * 1e-3) / 1e12, 1),
+        "bwd_tflops": round(2.5 * fwd_flops / (t["bwd_ms"] * 1e-3) / 1e12, 1),
+        "roofline": {"kernel": "fa_bwd_kernel<f16, d64> (dq/dk/dv, 5 GEMMs)", "bound": "mfma",
+                     "achieved": round(bwd_kernel_tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(bwd_kernel_tflops / MFMA_PEAK_TFLOPS, 4),
+                     "avg_launch_ms": round(t["bwd_main_kernel_ms"], 4), "traffic": None},
+    }
+    if not a.no_cpu:
+        res["cpu_baseline"] = cpu_baseline(torch, B, H, D, N, a.cpu_budget)
+    else:
+        res["cpu_baseline"] = None
+
+    if a.all:
+        cfgs = [
+            ("BERT varlen p=0.1 fp16", dict(B=8, H=12, D=64, N=512, dtype=torch.float16, p=0.1,
+                                            lens=torch.randint(256, 513, (8,), generator=torch.Generator().manual_seed(0)).tolist())),
+            ("GPT2 causal bf16 N=1024", dict(B=8, H=12, D=64, N=1024, dtype=torch.bfloat16, causal=True)),
+            ("GPT2 causal bf16 N=2048", dict(B=8, H=12, D=64, N=2048, dtype=torch.bfloat16, causal=True)),
+            ("GPT2 causal bf16 N=4096", dict(B=8, H=12, D=64, N=4096, dtype=torch.bfloat16, causal=True)),
+            ("d128 fp16 N=2048", dict(B=16, H=12, D=128, N=2048, dtype=torch.float16)),
+            ("d128 fp16 N=2048 causal", dict(B=16, H=12, D=128, N=2048, dtype=torch.float16, causal=True)),
+        ]
+        print("%-28s %9s %9s %9s %9s %8s %10s" % ("config", "fwd ms", "bwd ms", "fwd TF", "f+b TF", "% peak", "f+b GB/s"),
+              file=sys.stderr)
+        for name, kw in cfgs:
+            wl = Workload(torch, **kw)
+            tt = time_steps(torch, be, wl, max(10, a.steps // 2), 5)
+            fb = 3.5 * wl.fwd_flops / ((tt["fwd_ms"] + tt["bwd_ms"]) * 1e-3) / 1e12
+            gbs = (wl.bytes_fwd + wl.bytes_bwd) / ((tt["fwd_ms"] + tt["bwd_ms"]) * 1e-3) / 1e9
+            print("%-28s %9.4f %9.4f %9.1f %9.1f %8.2f %10.1f" % (
+                name, tt["fwd_ms"], tt["bwd_ms"], wl.fwd_flops / (tt["fwd_ms"] * 1e-3) / 1e12, fb,
+                100 * fb / MFMA_PEAK_TFLOPS, gbs), file=sys.stderr)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -257,7 +257,9 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
   p.pk = make_key(a->philox_seed, a->philox_offset);
 
   FA_LAUNCH(fa::launch_bwd_preprocess(p, a->dtype, a->head_dim, stream));
+  if (a->ev_main_start) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(a->ev_main_start), stream));
   FA_LAUNCH(fa::launch_bwd(p, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));
+  if (a->ev_main_stop) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(a->ev_main_stop), stream));
   FA_LAUNCH(fa::launch_bwd_postprocess(p, a->dtype, a->head_dim, stream));
   return FA_OK;
 }

@@ -71,6 +71,7 @@ class BwdArgs(ctypes.Structure):
         ("philox_seed", ctypes.c_uint64), ("philox_offset", ctypes.c_uint64),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("stream", ctypes.c_void_p),
+        ("ev_main_start", ctypes.c_void_p), ("ev_main_stop", ctypes.c_void_p),
     ]
 
 
@@ -239,7 +240,7 @@ def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_
 
 
 def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q,
-              max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen):
+              max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen, main_kernel_events=None):
     lib = load_library()
     code = _dtype_code(q)
     _check(q.dim() == 3, "q must be (total_q, nheads, head_size)")
@@ -298,6 +299,12 @@ def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seql
         a.workspace = ws.data_ptr()
         a.workspace_bytes = ws_bytes
         a.stream = _stream_handle(dev)
+        if main_kernel_events is not None:  # (start, stop) torch.cuda.Event created with enable_timing=True
+            for ev in main_kernel_events:
+                if not ev.cuda_event:  # torch creates the HIP event lazily, on first record
+                    ev.record()
+            a.ev_main_start = main_kernel_events[0].cuda_event
+            a.ev_main_stop = main_kernel_events[1].cuda_event
         rc = (lib.fa_bwd_block if sparse else lib.fa_bwd)(ctypes.byref(a))
         if rc != 0:
             _raise(rc, lib)
@@ -312,10 +319,11 @@ def fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, p_dropo
 
 
 def bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-        p_dropout, softmax_scale, zero_tensors, is_causal, gen=None):
-    """mha_bwd (fmha_api.cpp:302-449): fills dq, dk, dv in place, returns [dq, dk, dv, softmax_d]."""
+        p_dropout, softmax_scale, zero_tensors, is_causal, gen=None, main_kernel_events=None):
+    """mha_bwd (fmha_api.cpp:302-449): fills dq, dk, dv in place, returns [dq, dk, dv, softmax_d].
+    main_kernel_events: optional (start, stop) timing events recorded around the dq/dk/dv kernel alone."""
     return _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, None, max_seqlen_q,
-                     max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen)
+                     max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen, main_kernel_events)
 
 
 def fwd_block(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,

@@ -111,6 +111,10 @@ typedef struct fa_bwd_args {
   void* workspace;
   size_t workspace_bytes;
   void* stream;
+  /* Optional profiling hooks (hipEvent_t or NULL): recorded on `stream` immediately before and after the main
+   * dq/dk/dv kernel, i.e. excluding the rowsum(dO o O) pre-pass and the dq conversion post-pass. */
+  void* ev_main_start;
+  void* ev_main_stop;
 } fa_bwd_args;
 
 /* replaces flash_attn_cuda.fwd -> mha_fwd, csrc/flash_attn/fmha_api.cpp:173-299 */
