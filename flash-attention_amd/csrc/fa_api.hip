@@ -210,9 +210,8 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
   const bool dropout = a->p_dropout > 0.f;
   const float p_keep = 1.f - a->p_dropout;
 
-  const size_t dq_bytes = align16((size_t)a->total_q * a->nheads * a->head_dim * sizeof(float));
   const SparseLayout sl = sparse_layout(r);
-  const size_t need = dq_bytes + (sparse ? sl.bytes : 0);
+  const size_t need = sparse ? sl.bytes : 0;  // the dense backward needs no scratch: no dq_tmp (fmha_api.cpp:403-404)
   if (need > 0 && (!a->workspace || a->workspace_bytes < need))
     return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, a->workspace_bytes);
   FA_REQUIRE(need == 0 || aligned16(a->workspace), "workspace must be 16-byte aligned");
@@ -221,7 +220,7 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
   fa::BwdParams p;
   memset(&p, 0, sizeof(p));
   if (sparse) {
-    rc = build_maps(a->blockmask, ws + dq_bytes, sl, &p.sp, stream);
+    rc = build_maps(a->blockmask, ws, sl, &p.sp, stream);
     if (rc) return rc;
   }
   if (a->zero_tensors) {  // fmha_api.cpp:406-411
@@ -231,7 +230,7 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
     FA_LAUNCH(fa::launch_fill_f32(a->softmax_d, (size_t)a->batch * a->nheads * r.sq_r, 0.f, stream));
   }
   p.dout = a->dout; p.q = a->q; p.k = a->k; p.v = a->v; p.out = a->out; p.lse = a->softmax_lse;
-  p.dsoftmax = a->softmax_d; p.dq_acc = reinterpret_cast<float*>(ws);
+  p.dsoftmax = a->softmax_d;
   p.dq = a->dq; p.dk = a->dk; p.dv = a->dv;
   p.cu_q = a->cu_seqlens_q; p.cu_k = a->cu_seqlens_k;
   p.do_rs = a->do_row_stride; p.do_hs = a->do_head_stride;
@@ -246,9 +245,10 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
   p.total_q = a->total_q; p.total_k = a->total_k;
   p.max_sq = a->max_seqlen_q; p.max_sk = a->max_seqlen_k;
   p.sq_r = r.sq_r; p.lse_stride = a->lse_seq_stride;
-  const int bn = fa::bwd_block_n(a->head_dim);
-  p.nk_tiles = (a->max_seqlen_k + bn - 1) / bn;
+  p.nk_tiles = (a->max_seqlen_k + fa::kBwdBN - 1) / fa::kBwdBN;
   p.total_tiles = p.nk_tiles * a->nheads * a->batch;
+  p.nq_tiles = (a->max_seqlen_q + fa::kFwdBM - 1) / fa::kFwdBM;
+  p.total_qtiles = p.nq_tiles * a->nheads * a->batch;
   p.scale = a->softmax_scale;
   p.scale_log2 = a->softmax_scale * fa::kLog2e;
   p.p_keep = p_keep;
@@ -257,10 +257,10 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
   p.pk = make_key(a->philox_seed, a->philox_offset);
 
   FA_LAUNCH(fa::launch_bwd_preprocess(p, a->dtype, a->head_dim, stream));
+  FA_LAUNCH(fa::launch_bwd(p, 0, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));  // dQ
   if (a->ev_main_start) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(a->ev_main_start), stream));
-  FA_LAUNCH(fa::launch_bwd(p, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));
+  FA_LAUNCH(fa::launch_bwd(p, 1, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));  // dK, dV
   if (a->ev_main_stop) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(a->ev_main_stop), stream));
-  FA_LAUNCH(fa::launch_bwd_postprocess(p, a->dtype, a->head_dim, stream));
   return FA_OK;
 }
 
@@ -280,7 +280,7 @@ size_t fa_fwd_workspace_bytes(const fa_fwd_args* a) {
 
 size_t fa_bwd_workspace_bytes(const fa_bwd_args* a) {
   if (!a) return 0;
-  size_t n = align16((size_t)a->total_q * a->nheads * a->head_dim * sizeof(float));
+  size_t n = 0;
   if (a->blockmask) n += sparse_layout(round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, true)).bytes;
   return n;
 }

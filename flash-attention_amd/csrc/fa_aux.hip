@@ -1,5 +1,5 @@
 // Small HBM-bound helper kernels around the two attention kernels: fills, the block-sparse activity
-// maps, the backward's rowsum(dO o O) pre-pass and dQ conversion post-pass, and the probability dump
+// maps, the backward's rowsum(dO o O) pre-pass, and the probability dump
 // behind return_softmax.
 #include "fa_params.h"
 
@@ -61,9 +61,6 @@ __global__ void __launch_bounds__(256) bwd_preprocess_kernel(const BwdParams p) 
   for (int i = 0; i < 8; i++) acc += (float)a[i] * (float)b[i];
 #pragma unroll
   for (int off = TPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
-  float* dqa = p.dq_acc + rh * D + sub * 8;
-  *reinterpret_cast<f32x4*>(dqa) = f32x4{0.f, 0.f, 0.f, 0.f};
-  *reinterpret_cast<f32x4*>(dqa + 4) = f32x4{0.f, 0.f, 0.f, 0.f};
   if (sub == 0) {
     // locate (batch, position) of this row: binary search in cu_seqlens_q
     int lo = 0, hi = p.B;
@@ -74,24 +71,6 @@ __global__ void __launch_bounds__(256) bwd_preprocess_kernel(const BwdParams p) 
     const int pos = (int)(row - p.cu_q[lo]);
     if (pos >= 0 && pos < p.sq_r) p.dsoftmax[((int64_t)lo * p.H + h) * p.sq_r + pos] = acc * p.p_keep;
   }
-}
-
-template <typename T, int D>
-__global__ void __launch_bounds__(256) bwd_postprocess_kernel(const BwdParams p) {
-  constexpr int TPR = D / 8;
-  constexpr int RPB = 256 / TPR;
-  const int sub = threadIdx.x % TPR;
-  const int64_t rh = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
-  const int64_t n = (int64_t)p.total_q * p.H;
-  if (rh >= n) return;
-  const int h = (int)(rh % p.H);
-  const int64_t row = rh / p.H;
-  const float* src = p.dq_acc + rh * D + sub * 8;
-  const f32x4 x0 = *reinterpret_cast<const f32x4*>(src), x1 = *reinterpret_cast<const f32x4*>(src + 4);
-  const float f = p.scale * p.rp_keep;
-  f32x8 y = {x0[0] * f, x0[1] * f, x0[2] * f, x0[3] * f, x1[0] * f, x1[1] * f, x1[2] * f, x1[3] * f};
-  T* dst = reinterpret_cast<T*>(p.dq) + row * p.dq_rs + (int64_t)h * p.dq_hs + sub * 8;
-  st_global16(dst, bitcast<u32x4>(cvt8<T>(y)));
 }
 
 // One thread per (query row, key) element of S_dmask.  Slow scalar dot products: this path exists for tests
@@ -170,13 +149,6 @@ hipError_t pre_one(const BwdParams& p, hipStream_t stream) {
   hipLaunchKernelGGL((bwd_preprocess_kernel<T, D>), dim3((unsigned)((n + RPB - 1) / RPB)), dim3(256), 0, stream, p);
   return hipGetLastError();
 }
-template <typename T, int D>
-hipError_t post_one(const BwdParams& p, hipStream_t stream) {
-  const int64_t n = (int64_t)p.total_q * p.H;
-  constexpr int RPB = 256 / (D / 8);
-  hipLaunchKernelGGL((bwd_postprocess_kernel<T, D>), dim3((unsigned)((n + RPB - 1) / RPB)), dim3(256), 0, stream, p);
-  return hipGetLastError();
-}
 }  // namespace
 
 #define FA_DISPATCH_TD(fn)                                                          \
@@ -192,11 +164,6 @@ hipError_t launch_bwd_preprocess(const BwdParams& p, int dtype, int head_dim, hi
   if ((int64_t)p.total_q * p.H == 0) return hipSuccess;
   FA_DISPATCH_TD(pre_one)
 }
-hipError_t launch_bwd_postprocess(const BwdParams& p, int dtype, int head_dim, hipStream_t stream) {
-  if ((int64_t)p.total_q * p.H == 0) return hipSuccess;
-  FA_DISPATCH_TD(post_one)
-}
-
 hipError_t launch_dump_probs(const DumpParams& p, int dtype, hipStream_t stream) {
   dim3 grid((p.sk_r + 255) / 256, p.sq_r, p.B * p.H);
   if (dtype == 0) hipLaunchKernelGGL(dump_probs_kernel<_Float16>, grid, dim3(256), 0, stream, p);

@@ -1,20 +1,27 @@
-// Backward attention kernel for gfx950.
+// Backward attention kernels for gfx950.
 //
-// Computes what the reference's compute_dq_dk_dv_1xN does (csrc/flash_attn/src/fmha_dgrad_kernel_1xN_loop.h:34-700):
+// Together they compute what the reference's compute_dq_dk_dv_1xN does
+// (csrc/flash_attn/src/fmha_dgrad_kernel_1xN_loop.h:34-700):
 //   P  = exp(scale * S - lse) recomputed from Q, K;  dP = dO V^T;  dS' = P o (M o dP - Dk)   (M = dropout keep mask,
 //   Dk = keep * rowsum(dO o O));  dV = (P o M)^T dO / keep;  dK = dS'^T Q * scale / keep;  dQ = dS' K * scale / keep.
-// Organisation: one workgroup owns a tile of BN = 128 keys of one (batch, head) (wave w owns keys 32w..32w+31), keeps
-// its K and V fragments and the dK^T / dV^T accumulators in registers, and streams 64-row tiles of Q, dO, lse, Dk
-// through LDS.  Per step:
-//   S  = Q K^T, dP = dO V^T   A = Q / dO rows from LDS, B = K / V fragments in registers; C layout: lane -> key,
-//                             registers -> 16 query rows
-//   dV^T += dO^T P, dK^T += Q^T dS'   B = P / dS' straight from the accumulator registers (rounded to fp16/bf16, as the
-//                             reference does before these GEMMs), A = dO^T / Q^T via ds_read_b64_tr_b16
-//   dQ += dS' K               dS' goes through LDS once ([key][query] layout); the (64 x D) dQ tile of the step is split
-//                             over the 4 waves as 32x32 tiles, contraction over the 128 keys, both operands read with
-//                             ds_read_b64_tr_b16; the result is added to an fp32 accumulator in global memory with
-//                             atomics (the reference's dq_tmp, fmha_dgrad_kernel_1xN_loop.h:444-461,571-592) and is
-//                             converted to fp16/bf16 by a separate pass.
+//
+// The work is split in two kernels so that every output has exactly one owner and nothing is accumulated through
+// global memory (the reference carries dQ across key blocks in an fp32 dq_tmp buffer, :444-461,571-592; on this
+// part fp32 global atomics for that buffer cost more than recomputing S and dP):
+//
+// fa_bwd_dkdv_kernel  one workgroup owns 128 keys of one (batch, head) (wave w: keys 32w..32w+31), keeps its K and V
+//   fragments and the dK^T / dV^T accumulators in registers and streams 64-row tiles of Q, dO, lse, Dk through LDS.
+//     S  = Q K^T, dP = dO V^T           A = Q / dO rows from LDS, B = K / V fragments in registers;
+//                                       C layout: lane -> key, registers -> 16 query rows
+//     dV^T += dO^T P, dK^T += Q^T dS'   B = P / dS' straight from the accumulator registers (rounded to fp16/bf16 as
+//                                       the reference does before these GEMMs, :344,435), A = dO^T / Q^T read from the
+//                                       same row-major LDS tiles with ds_read_b64_tr_b16
+//
+// fa_bwd_dq_kernel    one workgroup owns 128 query rows (wave w: rows 32w..32w+31), keeps Q, dO fragments, lse, Dk and
+//   the dQ^T accumulator in registers and streams 64-key tiles of K and V through LDS; everything transposed so one
+//   lane owns one query row (as in the forward kernel):
+//     S^T = K Q^T, dP^T = V dO^T        A = K / V rows from LDS, B = Q / dO fragments in registers
+//     dQ^T += K^T dS'^T                 B = dS'^T from the accumulator registers, A = K^T via ds_read_b64_tr_b16
 #pragma once
 
 #include "fa_common.h"
@@ -22,46 +29,43 @@
 
 namespace fa {
 
+// ---------------------------------------------------------------------------------------------------------------
+// dK, dV
+// ---------------------------------------------------------------------------------------------------------------
 template <typename T, int D>
 struct BwdCfg {
   static constexpr int BM = kBwdBM;  // query rows per step
-  static constexpr int BN = 128;     // keys per workgroup
-  static constexpr int NW = 4;
+  static constexpr int BN = kBwdBN;  // keys per workgroup
   static constexpr int DV = D < 32 ? 32 : D;
-  static constexpr int RS = DV + 8;   // row stride (elements) of the K, Q, dO tiles in LDS
-  static constexpr int DSS = BM + 8;  // row stride of the dS'^T tile [key][query]
-  static constexpr int kOffK = 0;
-  static constexpr int kOffQ = kOffK + BN * RS * 2;
+  static constexpr int RS = DV + (D == 128 ? 24 : 8);  // row stride (elements) of the Q / dO tiles: conflict-free for
+                                                       // both the row-fragment and the transposed reads
+  static constexpr int kOffQ = 0;
   static constexpr int kOffDO = kOffQ + BM * RS * 2;
-  static constexpr int kOffDS = kOffDO + BM * RS * 2;
-  static constexpr int kOffLse = kOffDS + BN * DSS * 2;
+  static constexpr int kOffLse = kOffDO + BM * RS * 2;
   static constexpr int kOffDk = kOffLse + BM * 4;
-  static constexpr int kLdsBytes = kOffDk + BM * 4;
+  static constexpr int kTileBytes = kOffDk + BM * 4;
+  static constexpr int kEpiBytes = BN * (D + 8) * 2;
+  static constexpr int kLdsBytes = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
   static constexpr int CH = D / 8;
-  static constexpr int CPT = (BM * CH + 255) / 256;   // 16-byte chunks per thread for a Q / dO tile
-  static constexpr int CPTK = (BN * CH + 255) / 256;  // for the K tile
+  static constexpr int CPT = (BM * CH + 255) / 256;  // 16-byte chunks per thread for a Q / dO tile
   static constexpr int kMinBlocks = D <= 64 ? 2 : 1;
 };
 
 template <typename T, int D, bool kCausal, bool kDropout, bool kSparse>
-__global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
   using Cfg = BwdCfg<T, D>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
   using vec4 = typename E::vec4;
-  constexpr int BM = Cfg::BM, BN = Cfg::BN, DV = Cfg::DV, RS = Cfg::RS, DSS = Cfg::DSS, CH = Cfg::CH;
-  constexpr int CPT = Cfg::CPT, CPTK = Cfg::CPTK;
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, DV = Cfg::DV, RS = Cfg::RS, CH = Cfg::CH, CPT = Cfg::CPT;
 
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
-  T* Kl = reinterpret_cast<T*>(lds_raw + Cfg::kOffK);
   T* Ql = reinterpret_cast<T*>(lds_raw + Cfg::kOffQ);
   T* dOl = reinterpret_cast<T*>(lds_raw + Cfg::kOffDO);
-  T* dSl = reinterpret_cast<T*>(lds_raw + Cfg::kOffDS);
   float* lse_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffLse);
   float* dk_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffDk);
 
-  // XCD-aware id remap: all key tiles of one (batch, head) run on one XCD and share its L2 for Q, dO and
-  // the dQ accumulator.
+  // XCD-aware id remap: all key tiles of one (batch, head) run on one XCD and share its L2 copy of Q and dO.
   const int per_xcd = (p.total_tiles + 7) >> 3;
   const int vid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   if (vid >= p.total_tiles) return;
@@ -80,7 +84,8 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_kernel
   const int j16 = lane & 15, g16 = lane >> 4;
   const int key = n0 + wave * 32 + c;  // this lane's key (sequence-local)
 
-  // ---- K and V fragments of this wave's 32 keys (B operands), registers for the whole kernel
+  // ---- K and V fragments of this wave's 32 keys (B operands), registers for the whole kernel.
+  // Keys past the end are zero: their P is finite, their dK / dV rows are never stored.
   vec8 kreg[D / 16], vreg[D / 16];
   {
     const int kr = key < Lk ? key : Lk - 1;
@@ -94,25 +99,10 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_kernel
       vreg[ks] = bitcast<vec8>(bb);
     }
   }
-  // ---- K tile, row-major in LDS (B operand of the dQ GEMM)
-  {
-    const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)k_begin * p.k_rs + (int64_t)h * p.k_hs;
-#pragma unroll
-    for (int i = 0; i < CPTK; i++) {
-      const int ch = tid + i * 256;
-      const int row = ch / CH, col = (ch % CH) * 8;
-      if (BN * CH % 256 == 0 || ch < BN * CH) {
-        u32x4 a = u32x4{0, 0, 0, 0};
-        if (n0 + row < Lk) a = ld_global16(kbase + (int64_t)(n0 + row) * p.k_rs + col);
-        *reinterpret_cast<u32x4*>(Kl + row * RS + col) = a;
-      }
-    }
-    if (D < 32) {  // zero padding columns of all three row-major tiles
-      for (int i = tid; i < BN * (DV - D); i += 256) Kl[(i / (DV - D)) * RS + D + i % (DV - D)] = (T)0.f;
-      for (int i = tid; i < BM * (DV - D); i += 256) {
-        Ql[(i / (DV - D)) * RS + D + i % (DV - D)] = (T)0.f;
-        dOl[(i / (DV - D)) * RS + D + i % (DV - D)] = (T)0.f;
-      }
+  if (D < 32) {  // zero padding columns of the row-major tiles (read by the 32-wide transposed fragments)
+    for (int i = tid; i < BM * (DV - D); i += 256) {
+      Ql[(i / (DV - D)) * RS + D + i % (DV - D)] = (T)0.f;
+      dOl[(i / (DV - D)) * RS + D + i % (DV - D)] = (T)0.f;
     }
   }
 
@@ -124,7 +114,6 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_kernel
   const T* dobase = reinterpret_cast<const T*>(p.dout) + (int64_t)q_begin * p.do_rs + (int64_t)h * p.do_hs;
   const float* lsebase = p.lse + ((int64_t)b * p.H + h) * p.lse_stride;
   const float* dsbase = p.dsoftmax + ((int64_t)b * p.H + h) * p.sq_r;
-  float* dqbase = p.dq_acc + (int64_t)q_begin * p.H * D + (int64_t)h * D;
 
   u32x4 qpre[CPT], dopre[CPT];
   float statpre = 0.f;
@@ -142,7 +131,7 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_kernel
         dopre[i] = u32x4{0, 0, 0, 0};
       }
     }
-    if (tid < BM) {  // lse (scaled to base 2; +inf switches a row off)
+    if (tid < BM) {  // lse, scaled to base 2; +inf switches a row off (P = 0)
       const int row = m0 + tid;
       float x = INFINITY;
       if (row < Lq) {
@@ -189,8 +178,7 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_kernel
 
   const float cs = p.scale_log2;
   // element offset of a transposed read: row (4*hf + j16/4) [+8], column 16*(g16&1) + 4*(j16&3)
-  const int tr_row = 4 * hf + (j16 >> 2);
-  const int tr_col = 16 * (g16 & 1) + 4 * (j16 & 3);
+  const int tr_off = (4 * hf + (j16 >> 2)) * RS + 16 * (g16 & 1) + 4 * (j16 & 3);
 
   int mt = next_active(mt_begin);
   if (mt < mt_end) prefetch(mt);
@@ -230,17 +218,8 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_kernel
           rb_on[u] = p.sp.act16[rb * p.sp.ncb + (n0 >> 8)] != 0;
         }
       }
-      uint32_t keepbits[4];
-      if (kDropout) {
-        const int t = c & 3;
-        const uint32_t K4 = (uint32_t)key >> 2;
-        const uint32_t Q4 = ((uint32_t)(m0 + qb * 32) >> 2) + 2 * t + hf;
-        const uint32_t mine = dropout_keep_bits16(p.pk, (uint32_t)bh, Q4, K4, p.keep_thr);
-        keepbits[0] = quad_bcast<0>(mine) >> t;
-        keepbits[1] = quad_bcast<1>(mine) >> t;
-        keepbits[2] = quad_bcast<2>(mine) >> t;
-        keepbits[3] = quad_bcast<3>(mine) >> t;
-      }
+      uint32_t keep = 0xffffu;
+      if (kDropout) keep = keep16_col_layout(p.pk, (uint32_t)bh, m0 + qb * 32, key, hf, p.keep_thr);
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_l + qb * 32 + 8 * j + 4 * hf);
@@ -256,22 +235,12 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_kernel
           if (kSparse && !rb_on[j >> 1]) pe = 0.f;
           float dpe = dp[r];
           float pm = pe;
-          if (kDropout) {
-            const bool keep = (keepbits[j] >> (4 * i)) & 1u;
-            if (!keep) { dpe = 0.f; pm = 0.f; }
-          }
-          s[r] = pm;                      // P o M, feeds dV
-          dp[r] = pe * (dpe - dk4[i]);    // dS', feeds dK and dQ
+          if (kDropout && !((keep >> r) & 1u)) { dpe = 0.f; pm = 0.f; }
+          s[r] = pm;                    // P o M, feeds dV
+          dp[r] = pe * (dpe - dk4[i]);  // dS', feeds dK
         }
       }
-      // ---- round to the element type; dS'^T to LDS ([key][query]); dV^T += dO^T P; dK^T += Q^T dS'
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        f32x4 x;
-#pragma unroll
-        for (int i = 0; i < 4; i++) x[i] = dp[4 * j + i];
-        *reinterpret_cast<vec4*>(dSl + (wave * 32 + c) * DSS + qb * 32 + 8 * j + 4 * hf) = cvt4<T>(x);
-      }
+      // ---- dV^T += dO^T P; dK^T += Q^T dS'
 #pragma unroll
       for (int t = 0; t < 2; t++) {
         f32x8 pf, df;
@@ -281,7 +250,7 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_kernel
         const vec8 db8 = cvt8<T>(df);
 #pragma unroll
         for (int db = 0; db < DV / 32; db++) {
-          const int off = (qb * 32 + 16 * t + tr_row) * RS + db * 32 + tr_col;
+          const int off = (qb * 32 + 16 * t) * RS + db * 32 + tr_off;
           u32x2 lo = lds_read_tr16(dOl + off), hi = lds_read_tr16(dOl + off + 8 * RS);
           u32x4 av = {lo[0], lo[1], hi[0], hi[1]};
           acc_dv[db] = E::mfma32(bitcast<vec8>(av), pb, acc_dv[db]);
@@ -292,43 +261,13 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_kernel
         }
       }
     }
-    __syncthreads();  // dS'^T of all four waves is in LDS
-
-    // ---- dQ (BM x D) = dS' (BM x BN) K (BN x D); 32x32 tiles over the waves
-    constexpr int kTiles = (BM / 32) * (DV / 32);
-#pragma unroll
-    for (int tile = 0; tile < (kTiles + 3) / 4; tile++) {
-      const int tl = wave + tile * 4;
-      if (kTiles % 4 == 0 || tl < kTiles) {
-        const int qtile = tl / (DV / 32), dtile = tl % (DV / 32);
-        f32x16 acc;
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[r] = 0.f;
-#pragma unroll
-        for (int kk = 0; kk < BN / 16; kk++) {
-          const int offa = (kk * 16 + tr_row) * DSS + qtile * 32 + tr_col;
-          const int offb = (kk * 16 + tr_row) * RS + dtile * 32 + tr_col;
-          u32x2 alo = lds_read_tr16(dSl + offa), ahi = lds_read_tr16(dSl + offa + 8 * DSS);
-          u32x2 blo = lds_read_tr16(Kl + offb), bhi = lds_read_tr16(Kl + offb + 8 * RS);
-          u32x4 av = {alo[0], alo[1], ahi[0], ahi[1]};
-          u32x4 bv = {blo[0], blo[1], bhi[0], bhi[1]};
-          acc = E::mfma32(bitcast<vec8>(av), bitcast<vec8>(bv), acc);
-        }
-        if (dtile * 32 + c < D) {
-#pragma unroll
-          for (int r = 0; r < 16; r++) {
-            const int qrow = m0 + qtile * 32 + (r >> 2) * 8 + hf * 4 + (r & 3);
-            if (qrow < Lq) atomicAdd(dqbase + (int64_t)qrow * p.H * D + dtile * 32 + c, acc[r]);
-          }
-        }
-      }
-    }
     mt = mt_next;
   }
 
   // ---- epilogue: scale, transpose dK^T / dV^T through LDS, coalesced stores
   __syncthreads();
-  T* Stg = reinterpret_cast<T*>(lds_raw) + wave * 32 * RS;  // 32 keys x D per wave, reusing the K tile region
+  constexpr int ES = D + 8;
+  T* Stg = reinterpret_cast<T*>(lds_raw) + wave * 32 * ES;  // 32 keys x D per wave
   const float fv = p.rp_keep, fk = p.scale * p.rp_keep;
 #pragma unroll
   for (int which = 0; which < 2; which++) {
@@ -342,7 +281,7 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_kernel
 #pragma unroll
           for (int i = 0; i < 4; i++)
             x[i] = which == 0 ? acc_dk[db][g4 * 4 + i] * fk : acc_dv[db][g4 * 4 + i] * fv;
-          *reinterpret_cast<vec4*>(Stg + c * RS + d0) = cvt4<T>(x);
+          *reinterpret_cast<vec4*>(Stg + c * ES + d0) = cvt4<T>(x);
         }
       }
     __builtin_amdgcn_wave_barrier();
@@ -356,11 +295,233 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_kernel
       const int row = ch / CH, col = (ch % CH) * 8;
       const int krow = n0 + wave * 32 + row;
       if ((32 * CH % 64 == 0 || ch < 32 * CH) && krow < Lk) {
-        u32x4 val = *reinterpret_cast<const u32x4*>(Stg + row * RS + col);
+        u32x4 val = *reinterpret_cast<const u32x4*>(Stg + row * ES + col);
         st_global16(gbase + (int64_t)krow * grs + col, val);
       }
     }
     __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// dQ
+// ---------------------------------------------------------------------------------------------------------------
+template <typename T, int D, int BN>
+struct DqCfg {
+  static constexpr int BM = kFwdBM;  // query rows per workgroup (same tiling as the forward: shares its sparse map)
+  static constexpr int DV = D < 32 ? 32 : D;
+  static constexpr int KS = DV + (D == 128 ? 24 : 8);  // K tile: read both as row fragments and transposed
+  static constexpr int VS = D + 8;                     // V tile: row fragments only
+  static constexpr int OS = D + 8;
+  static constexpr int kTileBytes = BN * (KS + VS) * 2;
+  static constexpr int kEpiBytes = BM * OS * 2;
+  static constexpr int kLdsBytes = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
+  static constexpr int CH = D / 8;
+  static constexpr int CPT = (BN * CH + 255) / 256;
+};
+
+template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse>
+__global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
+  using Cfg = DqCfg<T, D, BN>;
+  using E = Elem<T>;
+  using vec8 = typename E::vec8;
+  constexpr int BM = Cfg::BM, DV = Cfg::DV, KS = Cfg::KS, VS = Cfg::VS, CH = Cfg::CH, CPT = Cfg::CPT;
+
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
+  T* Ks = reinterpret_cast<T*>(lds_raw);
+  T* Vs = Ks + BN * KS;
+
+  const int per_xcd = (p.total_qtiles + 7) >> 3;
+  const int vid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (vid >= p.total_qtiles) return;
+  const int bh = vid / p.nq_tiles;
+  const int qt = kCausal ? (p.nq_tiles - 1 - vid % p.nq_tiles) : (vid % p.nq_tiles);
+  const int b = bh / p.H, h = bh % p.H;
+
+  int q_begin, Lq, k_begin = 0, Lk = 0;
+  if (!seq_extent(p.cu_q, b, p.total_q, p.max_sq, &q_begin, &Lq)) return;
+  if (!seq_extent(p.cu_k, b, p.total_k, p.max_sk, &k_begin, &Lk)) Lk = 0;  // no keys: dQ = 0
+  const int m0 = qt * BM;
+  if (m0 >= Lq) return;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 31, hf = lane >> 5;
+  const int mw = m0 + wave * 32;
+  const int qrow = mw + c;
+
+  // ---- Q and dO fragments (B operands), lse and Dk of this lane's query row
+  vec8 qreg[D / 16], doreg[D / 16];
+  float lse2 = INFINITY, dkv = 0.f;  // +inf switches the row off
+  {
+    const int qr = qrow < Lq ? qrow : Lq - 1;
+    const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)(q_begin + qr) * p.q_rs + (int64_t)h * p.q_hs + hf * 8;
+    const T* dp_ = reinterpret_cast<const T*>(p.dout) + (int64_t)(q_begin + qr) * p.do_rs + (int64_t)h * p.do_hs + hf * 8;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ks++) {
+      u32x4 a = ld_global16(qp + ks * 16), bb = ld_global16(dp_ + ks * 16);
+      if (qrow >= Lq) { a = u32x4{0, 0, 0, 0}; bb = u32x4{0, 0, 0, 0}; }
+      qreg[ks] = bitcast<vec8>(a);
+      doreg[ks] = bitcast<vec8>(bb);
+    }
+    if (qrow < Lq) {
+      const float x = p.lse[((int64_t)b * p.H + h) * p.lse_stride + qrow];
+      lse2 = (x == -INFINITY) ? INFINITY : x * kLog2e;
+      dkv = p.dsoftmax[((int64_t)b * p.H + h) * p.sq_r + qrow];
+    }
+  }
+  if (D < 32) {
+    for (int i = tid; i < BN * (DV - D); i += 256) Ks[(i / (DV - D)) * KS + D + i % (DV - D)] = (T)0.f;
+  }
+
+  int n_end = Lk;
+  if (kCausal) n_end = n_end < m0 + BM ? n_end : m0 + BM;
+  const int ntiles = (n_end + BN - 1) / BN;
+
+  const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)k_begin * p.k_rs + (int64_t)h * p.k_hs;
+  const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)k_begin * p.v_rs + (int64_t)h * p.v_hs;
+
+  u32x4 kpre[CPT], vpre[CPT];
+  auto prefetch = [&](int it) {
+    const int n0 = it * BN;
+#pragma unroll
+    for (int i = 0; i < CPT; i++) {
+      const int ch = tid + i * 256;
+      const int row = ch / CH, col = (ch % CH) * 8;
+      const int key = n0 + row;
+      if ((BN * CH % 256 == 0 || ch < BN * CH) && key < Lk) {
+        kpre[i] = ld_global16(kbase + (int64_t)key * p.k_rs + col);
+        vpre[i] = ld_global16(vbase + (int64_t)key * p.v_rs + col);
+      } else {  // zero keys contribute dS' * 0 to dQ
+        kpre[i] = u32x4{0, 0, 0, 0};
+        vpre[i] = u32x4{0, 0, 0, 0};
+      }
+    }
+  };
+  auto commit = [&]() {
+#pragma unroll
+    for (int i = 0; i < CPT; i++) {
+      const int ch = tid + i * 256;
+      const int row = ch / CH, col = (ch % CH) * 8;
+      if (BN * CH % 256 == 0 || ch < BN * CH) {
+        *reinterpret_cast<u32x4*>(Ks + row * KS + col) = kpre[i];
+        *reinterpret_cast<u32x4*>(Vs + row * VS + col) = vpre[i];
+      }
+    }
+  };
+  auto tile_active = [&](int it) -> bool {
+    if (!kSparse) return true;
+    return p.sp.actq[qt * p.sp.ncb + ((it * BN) >> 8)] != 0;
+  };
+  auto next_active = [&](int it) -> int {
+    while (it < ntiles && !tile_active(it)) it++;
+    return it;
+  };
+
+  f32x16 acc[DV / 32];
+#pragma unroll
+  for (int i = 0; i < DV / 32; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
+
+  const float cs = p.scale_log2;
+  const int j16 = lane & 15, g16 = lane >> 4;
+  const int ktr_off = (4 * hf + (j16 >> 2)) * KS + 16 * (g16 & 1) + 4 * (j16 & 3);
+
+  int it = next_active(0);
+  if (it < ntiles) prefetch(it);
+  while (it < ntiles) {
+    const int n0 = it * BN;
+    __syncthreads();
+    commit();
+    __syncthreads();
+    const int it_next = next_active(it + 1);
+    if (it_next < ntiles) prefetch(it_next);
+
+    bool wave_work = true;
+    if (kCausal && n0 > mw + 31) wave_work = false;
+    bool row_on = true;
+    if (kSparse) {
+      const int rb = (qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1;
+      row_on = p.sp.act16[rb * p.sp.ncb + (n0 >> 8)] != 0;
+      if (__ballot(row_on) == 0) wave_work = false;
+    }
+    if (wave_work) {
+      const bool diag = kCausal && (n0 + BN - 1 > mw);
+#pragma unroll
+      for (int kb = 0; kb < BN / 32; kb++) {
+        f32x16 s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ks++) {
+          vec8 a = *reinterpret_cast<const vec8*>(Ks + (kb * 32 + c) * KS + ks * 16 + hf * 8);
+          s = E::mfma32(a, qreg[ks], s);
+        }
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ks++) {
+          vec8 a = *reinterpret_cast<const vec8*>(Vs + (kb * 32 + c) * VS + ks * 16 + hf * 8);
+          dp = E::mfma32(a, doreg[ks], dp);
+        }
+        uint32_t keep = 0xffffu;
+        if (kDropout) keep = keep16_row_layout(p.pk, (uint32_t)bh, qrow, n0 + kb * 32, hf, p.keep_thr);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          float pe = fast_exp2(__builtin_fmaf(s[r], cs, -lse2));
+          if (kCausal && diag) {
+            const int key = n0 + kb * 32 + (r >> 2) * 8 + hf * 4 + (r & 3);
+            if (key > qrow) pe = 0.f;
+          }
+          if (kSparse && !row_on) pe = 0.f;
+          float dpe = dp[r];
+          if (kDropout && !((keep >> r) & 1u)) dpe = 0.f;
+          s[r] = pe * (dpe - dkv);  // dS'
+        }
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+          f32x8 df;
+#pragma unroll
+          for (int i = 0; i < 8; i++) df[i] = s[8 * t + i];
+          const vec8 dsb = cvt8<T>(df);
+#pragma unroll
+          for (int db = 0; db < DV / 32; db++) {
+            const T* kp = Ks + (kb * 32 + 16 * t) * KS + db * 32 + ktr_off;
+            u32x2 lo = lds_read_tr16(kp), hi = lds_read_tr16(kp + 8 * KS);
+            u32x4 av = {lo[0], lo[1], hi[0], hi[1]};
+            acc[db] = E::mfma32(bitcast<vec8>(av), dsb, acc[db]);
+          }
+        }
+      }
+    }
+    it = it_next;
+  }
+
+  // ---- epilogue: dQ = dQ^T acc * scale / keep, transposed through LDS, coalesced stores
+  const float f = p.scale * p.rp_keep;
+  __syncthreads();
+  constexpr int OS = Cfg::OS;
+  T* Os = reinterpret_cast<T*>(lds_raw) + wave * 32 * OS;
+#pragma unroll
+  for (int db = 0; db < DV / 32; db++)
+#pragma unroll
+    for (int g4 = 0; g4 < 4; g4++) {
+      const int d0 = db * 32 + g4 * 8 + hf * 4;
+      if (d0 < D) {
+        f32x4 x;
+#pragma unroll
+        for (int i = 0; i < 4; i++) x[i] = acc[db][g4 * 4 + i] * f;
+        *reinterpret_cast<typename E::vec4*>(Os + c * OS + d0) = cvt4<T>(x);
+      }
+    }
+  __builtin_amdgcn_wave_barrier();
+  T* gbase = reinterpret_cast<T*>(p.dq) + (int64_t)q_begin * p.dq_rs + (int64_t)h * p.dq_hs;
+#pragma unroll
+  for (int i = 0; i < (32 * CH + 63) / 64; i++) {
+    const int ch = lane + i * 64;
+    const int row = ch / CH, col = (ch % CH) * 8;
+    if ((32 * CH % 64 == 0 || ch < 32 * CH) && mw + row < Lq) {
+      u32x4 val = *reinterpret_cast<const u32x4*>(Os + row * OS + col);
+      st_global16(gbase + (int64_t)(mw + row) * p.dq_rs + col, val);
+    }
   }
 }
 

@@ -157,4 +157,32 @@ FA_DEVICE uint32_t quad_bcast(uint32_t x) {
   return (uint32_t)__builtin_amdgcn_mov_dpp((int)x, J | (J << 2) | (J << 4) | (J << 6), 0xf, 0xf, true);
 }
 
+// Keep bits of the 16 score elements one lane owns in a 32x32 MFMA accumulator tile; bit r <=> register r is kept.
+// "Row layout" (S^T = K Q^T tiles: lane -> query row `qrow`, register r -> key key0 + 8*(r/4) + 4*hf + r%4) and
+// "column layout" (S = Q K^T tiles: lane -> key `key`, register r -> query row q0 + 8*(r/4) + 4*hf + r%4).
+// The four lanes of a quad own the four rows (columns) of the same four micro-blocks; lane t of the quad draws the
+// Philox numbers of micro-block t and the quad exchanges the resulting 16-bit masks with DPP broadcasts.
+FA_DEVICE uint32_t keep16_row_layout(const PhiloxKey& pk, uint32_t bh, int qrow, int key0, int hf, uint32_t thr) {
+  const int t = qrow & 3;
+  const uint32_t mine = dropout_keep_bits16(pk, bh, (uint32_t)qrow >> 2, ((uint32_t)key0 >> 2) + 2 * t + hf, thr);
+  uint32_t r = ((quad_bcast<0>(mine) >> (4 * t)) & 0xfu);
+  r |= ((quad_bcast<1>(mine) >> (4 * t)) & 0xfu) << 4;
+  r |= ((quad_bcast<2>(mine) >> (4 * t)) & 0xfu) << 8;
+  r |= ((quad_bcast<3>(mine) >> (4 * t)) & 0xfu) << 12;
+  return r;
+}
+
+FA_DEVICE uint32_t keep16_col_layout(const PhiloxKey& pk, uint32_t bh, int q0, int key, int hf, uint32_t thr) {
+  const int t = key & 3;
+  const uint32_t mine = dropout_keep_bits16(pk, bh, ((uint32_t)q0 >> 2) + 2 * t + hf, (uint32_t)key >> 2, thr);
+  const uint32_t b[4] = {quad_bcast<0>(mine) >> t, quad_bcast<1>(mine) >> t, quad_bcast<2>(mine) >> t,
+                         quad_bcast<3>(mine) >> t};
+  uint32_t r = 0;
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) r |= ((b[j] >> (4 * i)) & 1u) << (4 * j + i);
+  return r;
+}
+
 }  // namespace fa

@@ -218,25 +218,12 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
         for (int r = 0; r < 16; r++) o_acc[i][r] *= alpha;
 
       if (kDropout) {
-        const uint32_t bhu = (uint32_t)bh;
-        const uint32_t Q4 = (uint32_t)qrow >> 2;
-        const int t = c & 3;
 #pragma unroll
         for (int kb = 0; kb < BN / 32; kb++) {
-          const uint32_t K4 = ((uint32_t)(n0 + kb * 32) >> 2) + 2 * t + hf;
-          const uint32_t mine = dropout_keep_bits16(p.pk, bhu, Q4, K4, p.keep_thr);
-          uint32_t bj[4];
-          bj[0] = quad_bcast<0>(mine);
-          bj[1] = quad_bcast<1>(mine);
-          bj[2] = quad_bcast<2>(mine);
-          bj[3] = quad_bcast<3>(mine);
+          const uint32_t keep = keep16_row_layout(p.pk, (uint32_t)bh, qrow, n0 + kb * 32, hf, p.keep_thr);
 #pragma unroll
-          for (int j = 0; j < 4; j++) {
-            const uint32_t rowbits = bj[j] >> (4 * t);
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-              if (!((rowbits >> i) & 1u)) s[kb][4 * j + i] = 0.f;
-          }
+          for (int r = 0; r < 16; r++)
+            if (!((keep >> r) & 1u)) s[kb][r] = 0.f;
         }
       }
 

@@ -74,7 +74,6 @@ struct BwdParams {
   const void* out;
   const float* lse;
   float* dsoftmax;  // softmax_d [B, H, sq_r]
-  float* dq_acc;    // fp32 [total_q, H, D] accumulator (workspace)
   void* dq;
   void* dk;
   void* dv;
@@ -87,8 +86,10 @@ struct BwdParams {
   int max_sq, max_sk;
   int sq_r;        // innermost extent of dsoftmax
   int lse_stride;  // innermost extent of lse
-  int nk_tiles;
-  int total_tiles;
+  int nk_tiles;      // key tiles of the dK/dV kernel
+  int total_tiles;   // nk_tiles * H * B
+  int nq_tiles;      // query tiles of the dQ kernel
+  int total_qtiles;  // nq_tiles * H * B
   float scale;
   float scale_log2;
   float p_keep;
@@ -113,7 +114,8 @@ FA_DEVICE bool seq_extent(const int32_t* cu, int b, int total, int max_len, int*
 hipError_t launch_fwd(const FwdParams& p, int dtype, int head_dim, bool causal, bool dropout, bool sparse,
                       hipStream_t stream);
 hipError_t launch_dump_probs(const DumpParams& p, int dtype, hipStream_t stream);
-hipError_t launch_bwd(const BwdParams& p, int dtype, int head_dim, bool causal, bool dropout, bool sparse,
+// which: 0 = dQ kernel, 1 = dK/dV kernel
+hipError_t launch_bwd(const BwdParams& p, int which, int dtype, int head_dim, bool causal, bool dropout, bool sparse,
                       hipStream_t stream);
 hipError_t launch_build_sparse_maps(const int32_t* blockmask, uint8_t* act16, uint8_t* actq, uint8_t* actk, int nrb,
                                     int ncb, int rows_per_qt, int nqt, int rows_per_qt2, int nqt2, hipStream_t stream);
@@ -121,14 +123,12 @@ hipError_t launch_fill_f32(float* p, size_t n, float value, hipStream_t stream);
 // Zero a strided [total, H, D] tensor of 16-bit elements.
 hipError_t launch_zero_rows(void* base, int64_t row_stride, int64_t head_stride, int total, int H, int D,
                             hipStream_t stream);
-// softmax_d = keep * rowsum(dO o O) and dq_acc = 0 (fmha_dgrad_kernel_1xN_loop.h:15-30).
+// softmax_d = keep * rowsum(dO o O) (fmha_dgrad_kernel_1xN_loop.h:15-30).
 hipError_t launch_bwd_preprocess(const BwdParams& p, int dtype, int head_dim, hipStream_t stream);
-// dq = dq_acc * scale / keep, rounded to the element type (fmha_dgrad_kernel_1xN_loop.h:571-592).
-hipError_t launch_bwd_postprocess(const BwdParams& p, int dtype, int head_dim, hipStream_t stream);
 
 // Tile shapes, needed by the front end for grid sizes and workspace layout.
 constexpr int kFwdBM = 128;   // query rows per forward workgroup
-int bwd_block_n(int head_dim);  // keys per backward workgroup
-constexpr int kBwdBM = 64;    // query rows per backward inner step
+constexpr int kBwdBN = 128;   // keys per dK/dV workgroup
+constexpr int kBwdBM = 64;    // query rows per dK/dV inner step
 
 }  // namespace fa

@@ -111,8 +111,8 @@ typedef struct fa_bwd_args {
   void* workspace;
   size_t workspace_bytes;
   void* stream;
-  /* Optional profiling hooks (hipEvent_t or NULL): recorded on `stream` immediately before and after the main
-   * dq/dk/dv kernel, i.e. excluding the rowsum(dO o O) pre-pass and the dq conversion post-pass. */
+  /* Optional profiling hooks (hipEvent_t or NULL): recorded on `stream` immediately before and after the dK/dV
+   * kernel, the longest of the three kernels of a backward call (rowsum(dO o O) pre-pass, dQ kernel, dK/dV kernel). */
   void* ev_main_start;
   void* ev_main_stop;
 } fa_bwd_args;
@@ -127,8 +127,9 @@ int fa_fwd_block(const fa_fwd_args* args);
 /* replaces flash_attn_cuda.bwd_block -> mha_bwd_block, csrc/flash_attn/fmha_api.cpp:575-718 */
 int fa_bwd_block(const fa_bwd_args* args);
 
-/* Scratch the caller must provide; stands in for the o_tmp / dq_tmp / softmax_d allocations of
- * fmha_api.cpp:243-254,401-404.  Only shapes, dtype and blockmask!=NULL are read. */
+/* Scratch the caller must provide.  The dense paths need none (there is no o_tmp / dq_tmp, fmha_api.cpp:247,
+ * 403-404); the block-sparse paths need room for their block activity maps.  Only shapes and blockmask!=NULL
+ * are read. */
 size_t fa_fwd_workspace_bytes(const fa_fwd_args* args);
 size_t fa_bwd_workspace_bytes(const fa_bwd_args* args);
 

@@ -109,7 +109,9 @@ def test_workspace_sizes(lib):
     g.struct_bytes = ctypes.sizeof(g)
     g.batch, g.nheads, g.head_dim, g.total_q, g.total_k = 2, 3, 64, 100, 100
     g.max_seqlen_q = g.max_seqlen_k = 64
-    assert lib.fa_bwd_workspace_bytes(ctypes.byref(g)) == 100 * 3 * 64 * 4  # the fp32 dq accumulator (dq_tmp)
+    assert lib.fa_bwd_workspace_bytes(ctypes.byref(g)) == 0  # nor the dense backward (no fp32 dq_tmp)
+    g.blockmask = 0x1000
+    assert lib.fa_bwd_workspace_bytes(ctypes.byref(g)) > 0   # block-sparse: room for the block activity maps
 
 
 @pytest.mark.parametrize("d,sq,sk,sparse,want", [

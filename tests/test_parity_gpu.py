@@ -220,7 +220,7 @@ def test_strided_views_and_noncontiguous_grads():
            True, None)
     torch.cuda.synchronize()
     assert torch.equal(dbig[:, 1, :, :D], dk) and torch.equal(dbig[:, 3, :, :D], dv)
-    assert (dbig[:, 0, :, :D].float() - dq.float()).abs().max() < 2e-3  # dq sums fp32 atomics: order may differ
+    assert torch.equal(dbig[:, 0, :, :D], dq)  # no atomics anywhere: results are bitwise reproducible
     assert dbig[:, 2].abs().max() == 0 and dbig[..., D:].abs().max() == 0  # nothing written outside the views
 
 
