@@ -118,6 +118,8 @@ def main():
     ap.add_argument("--all", action="store_true", help="also time the other BASELINE configurations (stderr table)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every (batch, head, tile) is independent; there is no "
@@ -127,6 +129,13 @@ def main():
     be.load_library()  # fails loudly if the HIP library is not built
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
+
+    if a.calibrate_copy:  # a kernel whose HBM traffic is known: reads 256 MiB, writes 256 MiB
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     B, H, D, N = 8, 12, 64, 2048
     w = Workload(torch, B, H, D, N, torch.float16)

@@ -25,7 +25,7 @@ struct FwdCfg {
   static constexpr int NW = 4;                 // waves per workgroup, 32 query rows each
   static constexpr int DV = D < 32 ? 32 : D;   // V tile width in LDS (zero padded for D = 16)
   static constexpr int KS = D + 8;             // K row stride in LDS, elements
-  static constexpr int VS = DV + 8;            // V row stride in LDS, elements
+  static constexpr int VS = DV + (D == 128 ? 16 : 8);  // V row stride in LDS: conflict-free for transposed reads
   static constexpr int OS = D + 8;             // epilogue staging row stride
   static constexpr int kTileBytes = BN * (KS + VS) * 2;
   static constexpr int kEpiBytes = BM * OS * 2;
