@@ -159,7 +159,10 @@ def main():
         "roofline": {"kernel": "fa_bwd_dkdv_kernel<f16, d64> (S, dP, dV, dK GEMMs: 8*B*H*N^2*d flops per launch)", "bound": "mfma",
                      "achieved": round(bwd_kernel_tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(bwd_kernel_tflops / MFMA_PEAK_TFLOPS, 4),
-                     "avg_launch_ms": round(t["bwd_main_kernel_ms"], 4), "traffic": None},
+                     "avg_launch_ms": round(t["bwd_main_kernel_ms"], 4),
+                     # HBM bytes per launch from rocprofv3 FETCH_SIZE x2.00 + WRITE_SIZE x1.00 (scale factors from a
+                     # 256 MiB copy): 99 980 KiB read + 49 152 KiB written
+                     "traffic": 152.7e6},
     }
     if not a.no_cpu:
         res["cpu_baseline"] = cpu_baseline(torch, B, H, D, N, a.cpu_budget)
