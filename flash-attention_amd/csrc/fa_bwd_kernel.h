@@ -65,12 +65,9 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
   float* lse_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffLse);
   float* dk_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffDk);
 
-  // XCD-aware id remap: all key tiles of one (batch, head) run on one XCD and share its L2 copy of Q and dO.
-  const int per_xcd = (p.total_tiles + 7) >> 3;
-  const int vid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (vid >= p.total_tiles) return;
-  const int bh = vid / p.nk_tiles;
-  const int kt = vid % p.nk_tiles;
+  // XCD-aware id map (see map_tile): the key tiles of one (batch, head) share one XCD's L2 copy of Q and dO.
+  int bh, kt;  // under a causal mask the first key tiles see the most query rows: rank order is already heavy-first
+  if (!map_tile<kCausal>(blockIdx.x, p.nk_tiles, p.B * p.H, &bh, &kt)) return;
   const int b = bh / p.H, h = bh % p.H;
 
   int q_begin = 0, Lq = 0, k_begin, Lk;
@@ -141,7 +138,7 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
       statpre = x;
     } else if (tid < 2 * BM) {
       const int row = m0 + tid - BM;
-      statpre = row < Lq ? dsbase[row] : 0.f;
+      statpre = row < Lq ? -dsbase[row] : 0.f;  // kept negated: the dP accumulator starts from -Dk
     }
   };
   auto commit = [&]() {
@@ -195,9 +192,14 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
 #pragma unroll
     for (int qb = 0; qb < BM / 32; qb++) {
       // ---- S = Q K^T and dP = dO V^T for 32 query rows x this wave's 32 keys
+      // dP starts from -Dk of its query row (fmha_dgrad_kernel_1xN_loop.h:361-371), so the MFMA delivers dP - Dk
       f32x16 s, dp;
 #pragma unroll
-      for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
+      for (int j = 0; j < 4; j++) {
+        const f32x4 nd4 = *reinterpret_cast<const f32x4*>(dk_l + qb * 32 + 8 * j + 4 * hf);
+#pragma unroll
+        for (int i = 0; i < 4; i++) { s[4 * j + i] = 0.f; dp[4 * j + i] = nd4[i]; }
+      }
 #pragma unroll
       for (int ks = 0; ks < D / 16; ks++) {
         vec8 aq = *reinterpret_cast<const vec8*>(Ql + (qb * 32 + c) * RS + ks * 16 + hf * 8);
@@ -223,7 +225,8 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_l + qb * 32 + 8 * j + 4 * hf);
-        const f32x4 dk4 = *reinterpret_cast<const f32x4*>(dk_l + qb * 32 + 8 * j + 4 * hf);
+        f32x4 nd4 = {0.f, 0.f, 0.f, 0.f};
+        if (kDropout) nd4 = *reinterpret_cast<const f32x4*>(dk_l + qb * 32 + 8 * j + 4 * hf);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           const int r = 4 * j + i;
@@ -233,11 +236,11 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
             if (key > qrow) pe = 0.f;
           }
           if (kSparse && !rb_on[j >> 1]) pe = 0.f;
-          float dpe = dp[r];
+          float dpe = dp[r];  // dP - Dk
           float pm = pe;
-          if (kDropout && !((keep >> r) & 1u)) { dpe = 0.f; pm = 0.f; }
-          s[r] = pm;                    // P o M, feeds dV
-          dp[r] = pe * (dpe - dk4[i]);  // dS', feeds dK
+          if (kDropout && !((keep >> r) & 1u)) { dpe = nd4[i]; pm = 0.f; }  // dropped: M o dP = 0
+          s[r] = pm;          // P o M, feeds dV
+          dp[r] = pe * dpe;   // dS' = P o (M o dP - Dk), feeds dK
         }
       }
       // ---- dV^T += dO^T P; dK^T += Q^T dS'
@@ -331,11 +334,9 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
   T* Ks = reinterpret_cast<T*>(lds_raw);
   T* Vs = Ks + BN * KS;
 
-  const int per_xcd = (p.total_qtiles + 7) >> 3;
-  const int vid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (vid >= p.total_qtiles) return;
-  const int bh = vid / p.nq_tiles;
-  const int qt = kCausal ? (p.nq_tiles - 1 - vid % p.nq_tiles) : (vid % p.nq_tiles);
+  int bh, rank;
+  if (!map_tile<kCausal>(blockIdx.x, p.nq_tiles, p.B * p.H, &bh, &rank)) return;
+  const int qt = kCausal ? p.nq_tiles - 1 - rank : rank;
   const int b = bh / p.H, h = bh % p.H;
 
   int q_begin, Lq, k_begin = 0, Lk = 0;
@@ -369,6 +370,12 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
       dkv = p.dsoftmax[((int64_t)b * p.H + h) * p.sq_r + qrow];
     }
   }
+  // For d <= 64 the dP^T accumulator starts from -Dk of this lane's query row (16 registers that save 16 subtractions
+  // per 32x32 tile); at d = 128 those registers would push the kernel below two waves per SIMD.
+  constexpr bool kInitNegD = D <= 64;
+  f32x16 negd;
+#pragma unroll
+  for (int r = 0; r < 16; r++) negd[r] = kInitNegD ? -dkv : 0.f;
   if (D < 32) {
     for (int i = tid; i < BN * (DV - D); i += 256) Ks[(i / (DV - D)) * KS + D + i % (DV - D)] = (T)0.f;
   }
@@ -449,9 +456,9 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
       const bool diag = kCausal && (n0 + BN - 1 > mw);
 #pragma unroll
       for (int kb = 0; kb < BN / 32; kb++) {
-        f32x16 s, dp;
+        f32x16 s, dp = negd;
 #pragma unroll
-        for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
+        for (int r = 0; r < 16; r++) s[r] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < D / 16; ks++) {
           vec8 a = *reinterpret_cast<const vec8*>(Ks + (kb * 32 + c) * KS + ks * 16 + hf * 8);
@@ -472,9 +479,9 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
             if (key > qrow) pe = 0.f;
           }
           if (kSparse && !row_on) pe = 0.f;
-          float dpe = dp[r];
-          if (kDropout && !((keep >> r) & 1u)) dpe = 0.f;
-          s[r] = pe * (dpe - dkv);  // dS'
+          float dpe = kInitNegD ? dp[r] : dp[r] - dkv;  // dP - Dk
+          if (kDropout && !((keep >> r) & 1u)) dpe = -dkv;
+          s[r] = pe * dpe;  // dS'
         }
 #pragma unroll
         for (int t = 0; t < 2; t++) {

@@ -45,15 +45,11 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
   T* Ks = reinterpret_cast<T*>(lds_raw);
   T* Vs = Ks + BN * KS;
 
-  // Workgroup -> (batch, head, query tile).  Consecutive workgroup ids go to different XCDs, so the
-  // id is re-mapped to give every XCD a contiguous range of tiles: all query tiles of one (batch, head)
-  // then share that XCD's L2 copy of K and V.
-  const int per_xcd = (p.total_tiles + 7) >> 3;
-  const int vid = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (vid >= p.total_tiles) return;
-  const int bh = vid / p.nq_tiles;
-  // heaviest (last) query tiles first under a causal mask
-  const int qt = kCausal ? (p.nq_tiles - 1 - vid % p.nq_tiles) : (vid % p.nq_tiles);
+  // Workgroup -> (batch, head, query tile), XCD-aware (see map_tile): the query tiles of one (batch, head) share
+  // one XCD's L2 copy of K and V.
+  int bh, rank;
+  if (!map_tile<kCausal>(blockIdx.x, p.nq_tiles, p.B * p.H, &bh, &rank)) return;
+  const int qt = kCausal ? p.nq_tiles - 1 - rank : rank;  // under a causal mask the last query tiles cost most
   const int b = bh / p.H, h = bh % p.H;
 
   int q_begin, Lq, k_begin = 0, Lk = 0;

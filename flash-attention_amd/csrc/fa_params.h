@@ -110,6 +110,32 @@ FA_DEVICE bool seq_extent(const int32_t* cu, int b, int total, int max_len, int*
   return true;
 }
 
+// Workgroup id -> (batch*head, tile rank).  The hardware deals consecutive workgroup ids to the 8 XCDs in turn
+// (id % 8), and each XCD has its own L2.
+//   kTileMajor = false (tiles of equal cost): every XCD gets a contiguous range of (bh, tile) pairs, so the tiles of
+//     one (batch, head) run on one XCD at about the same time and share its L2 copy of the streamed operand.
+//   kTileMajor = true (causal: tile cost grows with the rank reversed): ids enumerate tile ranks outermost, so the
+//     most expensive tiles of all (batch, head) pairs start first; batch*head is padded to a multiple of 8 so that a
+//     given (batch, head) still always lands on the same XCD.
+template <bool kTileMajor>
+FA_DEVICE bool map_tile(int block, int tiles_per_bh, int BH, int* bh, int* rank) {
+  if (kTileMajor) {
+    const int bhp = (BH + 7) & ~7;
+    *rank = block / bhp;
+    *bh = block - *rank * bhp;
+    return *bh < BH && *rank < tiles_per_bh;
+  }
+  const int total = tiles_per_bh * BH;
+  const int per_xcd = (total + 7) >> 3;
+  const int vid = (block & 7) * per_xcd + (block >> 3);
+  *bh = vid / tiles_per_bh;
+  *rank = vid - *bh * tiles_per_bh;
+  return vid < total;
+}
+inline int tile_grid(bool tile_major, int tiles_per_bh, int BH) {
+  return tile_major ? ((BH + 7) & ~7) * tiles_per_bh : ((tiles_per_bh * BH + 7) / 8) * 8;
+}
+
 // Launchers (defined in fa_fwd.hip / fa_bwd.hip / fa_aux.hip).  Return hipError_t of the launch.
 hipError_t launch_fwd(const FwdParams& p, int dtype, int head_dim, bool causal, bool dropout, bool sparse,
                       hipStream_t stream);
