@@ -72,6 +72,9 @@ FA_DEVICE typename Elem<T>::vec4 cvt4(f32x4 x) {
   return __builtin_convertvector(x, typename Elem<T>::vec4);
 }
 
+// Threshold (log2 units) of the forward kernel's lazy accumulator rescale.
+constexpr float kRescaleLog2 = 8.f;
+
 FA_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 FA_DEVICE float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 FA_DEVICE float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }

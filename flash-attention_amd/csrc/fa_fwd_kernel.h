@@ -193,11 +193,20 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
 #pragma unroll
         for (int r = 0; r < 16; r++) mt = fmaxf(mt, s[kb][r]);
       mt = half_max(mt);
-      const float m_new = fmaxf(m_i, mt);
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      const float mc = m_use * cs;
-      const float alpha = fast_exp2(m_i * cs - mc);
-      m_i = m_new;
+      // The reference point m_i of the exponentials only moves when some row's maximum has grown by more than
+      // 2^kRescaleLog2 since it was set; until then P may exceed 1 by at most that factor, which the fp32 accumulators and
+      // the fp16/bf16 rounding of P absorb, and the accumulators need no rescaling (numerator and denominator carry the
+      // same factor, so the result is unchanged).
+      if (__builtin_expect(__any((mt - m_i) * cs > kRescaleLog2), 0)) {  // wave-uniform; true on the first tile
+        const float m_new = fmaxf(m_i, mt);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = fast_exp2(m_i * cs - m_use * cs);
+        m_i = m_new;
+        l_i *= alpha;
+#pragma unroll
+        for (int i = 0; i < DV / 32; i++) o_acc[i] = o_acc[i] * alpha;
+      }
+      const float mc = ((m_i == -INFINITY) ? 0.f : m_i) * cs;
       float rs = 0.f;
 #pragma unroll
       for (int kb = 0; kb < BN / 32; kb++)
@@ -207,11 +216,7 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
           s[kb][r] = pe;
           rs += pe;
         }
-      l_i = l_i * alpha + rs;  // the sum uses P before dropout (fmha_fprop_kernel_1xN.h:454 vs :471)
-#pragma unroll
-      for (int i = 0; i < DV / 32; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) o_acc[i][r] *= alpha;
+      l_i += rs;  // the sum uses P before dropout (fmha_fprop_kernel_1xN.h:454 vs :471)
 
       if (kDropout) {
 #pragma unroll
