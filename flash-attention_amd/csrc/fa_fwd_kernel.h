@@ -23,15 +23,27 @@ template <typename T, int D, int BN>
 struct FwdCfg {
   static constexpr int BM = kFwdBM;
   static constexpr int NW = 4;                 // waves per workgroup, 32 query rows each
-  static constexpr int DV = D < 32 ? 32 : D;   // V tile width in LDS (zero padded for D = 16)
-  static constexpr int KS = D + 8;             // K row stride in LDS, elements
-  static constexpr int VS = DV + (D == 128 ? 16 : 8);  // V row stride in LDS: conflict-free for transposed reads
+  static constexpr int DV = D < 32 ? 32 : D;   // rows of the V^T MFMA operand (for D = 16 the upper 16 are don't-care)
   static constexpr int OS = D + 8;             // epilogue staging row stride
-  static constexpr int kTileBytes = BN * (KS + VS) * 2;
+  // K and V tiles sit in LDS unpadded, BN rows of CH 16-byte chunks, filled by direct-to-LDS loads (each wave
+  // instruction deposits 64 consecutive chunks).  Bank conflicts are avoided by permuting the chunks of a row:
+  // chunk ch of tile row r is stored at position ch ^ k_swz(r) (K, read as row fragments with ds_read_b128) or
+  // ch ^ v_swz(r) (V, read transposed with ds_read_b64_tr_b16, which fetches aligned chunk pairs).
+  static constexpr int CH = D / 8;
+  static constexpr int RPB = CH >= 16 ? 1 : 16 / CH;            // tile rows per 256 bytes
+  static constexpr int kKBytes = BN * D * 2;
+  static constexpr int kBufBytes = 2 * kKBytes;                 // one K tile followed by one V tile
+  static constexpr int kSlack = D < 32 ? 64 : 0;                // the 32-wide transposed reads run past a 16-wide V row
+  static constexpr int kTileBytes = 2 * kBufBytes + kSlack;     // double buffered
   static constexpr int kEpiBytes = BM * OS * 2;
   static constexpr int kLdsBytes = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
-  static constexpr int CH = D / 8;                              // 16-byte chunks per row
-  static constexpr int CPT = (BN * CH + 255) / 256;             // chunks per thread per tile
+  static constexpr int TI = 2 * BN * CH / 64;                   // direct-to-LDS wave instructions per tile (K, then V)
+  static constexpr int NI = TI / NW;                            // per wave: waves 0,1 fetch K, waves 2,3 fetch V
+  static constexpr int RPI = 64 / CH;                           // tile rows per instruction
+  static constexpr int NOFF = 16 / RPI > 0 ? 16 / RPI : 1;      // distinct per-lane source offsets (swizzle period 16 rows)
+  static_assert(TI % NW == 0 && NI % NOFF == 0, "tile does not split evenly over the waves");
+  static __device__ __forceinline__ int k_swz(int r) { return (r / RPB) % CH; }
+  static __device__ __forceinline__ int v_swz(int r) { return CH >= 4 ? 2 * ((r / RPB) % (CH / 2)) : 0; }
 };
 
 template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse>
@@ -39,11 +51,12 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
   using Cfg = FwdCfg<T, D, BN>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
-  constexpr int BM = Cfg::BM, DV = Cfg::DV, KS = Cfg::KS, VS = Cfg::VS, CH = Cfg::CH, CPT = Cfg::CPT;
+  constexpr int BM = Cfg::BM, DV = Cfg::DV, CH = Cfg::CH, NI = Cfg::NI, RPI = Cfg::RPI, NOFF = Cfg::NOFF;
+  constexpr int kKBytes = Cfg::kKBytes, kBufBytes = Cfg::kBufBytes;
+  typedef __attribute__((address_space(1))) const void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
 
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
-  T* Ks = reinterpret_cast<T*>(lds_raw);
-  T* Vs = Ks + BN * KS;
 
   // Workgroup -> (batch, head, query tile), XCD-aware (see map_tile): the query tiles of one (batch, head) share
   // one XCD's L2 copy of K and V.
@@ -58,7 +71,8 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
   const int m0 = qt * BM;
   if (m0 >= Lq) return;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 31, hf = lane >> 5;
   const int mw = m0 + wave * 32;  // first query row of this wave
   const int qrow = mw + c;        // this lane's query row (sequence-local)
@@ -76,42 +90,43 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
     }
   }
 
-  if (D < 32) {  // zero the padding columns of the V tile once
-    for (int i = tid; i < BN * (DV - D); i += 256) Vs[(i / (DV - D)) * VS + D + i % (DV - D)] = (T)0.f;
-  }
-
   int n_end = Lk;
   if (kCausal) n_end = n_end < m0 + BM ? n_end : m0 + BM;
   const int ntiles = (n_end + BN - 1) / BN;
 
-  const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)k_begin * p.k_rs + (int64_t)h * p.k_hs;
-  const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)k_begin * p.v_rs + (int64_t)h * p.v_hs;
-
-  u32x4 kpre[CPT], vpre[CPT];
-  auto prefetch = [&](int it) {
+  // ---- K/V staging: global -> LDS without passing through registers.  Waves 0,1 bring in the K tile, waves 2,3 the V
+  // tile, NI instructions of RPI rows each.  The source address is a wave-uniform row base plus a per-lane offset that
+  // encodes the lane's row within the instruction and the (swizzled) chunk it fetches.
+  const bool stage_k = wave < 2;
+  const int g0 = (wave & 1) * NI;  // first instruction slot of this wave inside its tile
+  const char* const tbase = stage_k
+      ? reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.k) + (int64_t)k_begin * p.k_rs + (int64_t)h * p.k_hs)
+      : reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.v) + (int64_t)k_begin * p.v_rs + (int64_t)h * p.v_hs);
+  const int64_t rsb = (stage_k ? p.k_rs : p.v_rs) * 2;  // source row stride in bytes
+  const int lds_dst0 = (stage_k ? 0 : kKBytes) + g0 * 1024;
+  const int rl = lane / CH, pch = lane % CH;
+  uint32_t src_off[NOFF];
+#pragma unroll
+  for (int j = 0; j < NOFF; j++) {
+    const int r = j * RPI + rl;
+    src_off[j] = (uint32_t)(rl * rsb) + 16u * (pch ^ (stage_k ? Cfg::k_swz(r) : Cfg::v_swz(r)));
+  }
+  auto stage = [&](int it, int buf) {
     const int n0 = it * BN;
+    const char* const tb = tbase + ((int64_t)n0 + g0 * RPI) * rsb;
+    if (__builtin_expect(n0 + BN <= Lk, 1)) {
 #pragma unroll
-    for (int i = 0; i < CPT; i++) {
-      const int ch = tid + i * 256;
-      const int row = ch / CH, col = (ch % CH) * 8;
-      const int key = n0 + row;
-      if ((BN * CH % 256 == 0 || ch < BN * CH) && key < Lk) {
-        kpre[i] = ld_global16(kbase + (int64_t)key * p.k_rs + col);
-        vpre[i] = ld_global16(vbase + (int64_t)key * p.v_rs + col);
-      } else {
-        kpre[i] = u32x4{0, 0, 0, 0};
-        vpre[i] = u32x4{0, 0, 0, 0};
-      }
-    }
-  };
-  auto commit = [&]() {
+      for (int i = 0; i < NI; i++)
+        __builtin_amdgcn_global_load_lds((gptr_t)(tb + i * RPI * rsb + src_off[i % NOFF]),
+                                         (lptr_t)(lds_raw + buf * kBufBytes + lds_dst0 + i * 1024), 16, 0, 0);
+    } else {  // last, partial tile: rows past the end re-read the last valid row (their scores are masked below)
 #pragma unroll
-    for (int i = 0; i < CPT; i++) {
-      const int ch = tid + i * 256;
-      const int row = ch / CH, col = (ch % CH) * 8;
-      if (BN * CH % 256 == 0 || ch < BN * CH) {
-        *reinterpret_cast<u32x4*>(Ks + row * KS + col) = kpre[i];
-        *reinterpret_cast<u32x4*>(Vs + row * VS + col) = vpre[i];
+      for (int i = 0; i < NI; i++) {
+        const int r = (g0 + i) * RPI + rl;
+        const int rc = n0 + r < Lk ? r : Lk - 1 - n0;
+        const int ch = pch ^ (stage_k ? Cfg::k_swz(r) : Cfg::v_swz(r));
+        __builtin_amdgcn_global_load_lds((gptr_t)(tbase + ((int64_t)n0 + rc) * rsb + 16 * ch),
+                                         (lptr_t)(lds_raw + buf * kBufBytes + lds_dst0 + i * 1024), 16, 0, 0);
       }
     }
   };
@@ -138,17 +153,33 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
   const float cs = p.scale_log2;
   // operand addressing of the transposed V reads (see lds_read_tr16)
   const int j16 = lane & 15, g16 = lane >> 4;
-  const int vtr_off = (4 * hf + (j16 >> 2)) * VS + 16 * (g16 & 1) + 4 * (j16 & 3);
+  int voff[DV / 32];  // element offsets of this lane's transposed V reads
+  {
+    const int vr = 4 * hf + (j16 >> 2);
+#pragma unroll
+    for (int db = 0; db < DV / 32; db++)
+      voff[db] = vr * D + (((db * 4 + 2 * (g16 & 1)) ^ Cfg::v_swz(vr)) * 8) + 4 * (j16 & 3);
+  }
+  int koff[D / 16];  // element offsets of this lane's K row fragments
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ks++) koff[ks] = c * D + (((ks * 2 + hf) ^ Cfg::k_swz(c)) * 8);
+  int buf = 0;
 
   int it = next_active(0);
-  if (it < ntiles) prefetch(it);
+  if (it < ntiles) stage(it, 0);
   while (it < ntiles) {
     const int n0 = it * BN;
-    __syncthreads();  // everyone is done reading the previous tile
-    commit();
-    __syncthreads();
+    // Opaque redefinition of the accumulators at the top of every iteration: without it the register allocator
+    // ties the last MFMA's result to the registers the epilogue reads and copies all of O back on every trip.
+#pragma unroll
+    for (int i = 0; i < DV / 32; i++) asm volatile("" : "+v"(o_acc[i]));
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile `it` is in LDS
+    __syncthreads();                     // so is everyone else's, and nobody still reads the other buffer
     const int it_next = next_active(it + 1);
-    if (it_next < ntiles) prefetch(it_next);
+    if (it_next < ntiles) stage(it_next, buf ^ 1);
+    const T* Ks = reinterpret_cast<const T*>(lds_raw + buf * kBufBytes);
+    const T* Vs = Ks + BN * D;
+    buf ^= 1;
 
     bool wave_work = true;
     if (kCausal && n0 > mw + 31) wave_work = false;  // every key of this tile is above the wave's diagonal
@@ -168,7 +199,7 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
         for (int r = 0; r < 16; r++) s[kb][r] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < D / 16; ks++) {
-          vec8 a = *reinterpret_cast<const vec8*>(Ks + (kb * 32 + c) * KS + ks * 16 + hf * 8);
+          vec8 a = *reinterpret_cast<const vec8*>(Ks + kb * 32 * D + koff[ks]);
           s[kb] = E::mfma32(a, qreg[ks], s[kb]);
         }
       }
@@ -214,9 +245,9 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
         for (int r = 0; r < 16; r++) {
           const float pe = fast_exp2(__builtin_fmaf(s[kb][r], cs, -mc));
           s[kb][r] = pe;
-          rs += pe;
+          if (kDropout) rs += pe;
         }
-      l_i += rs;  // the sum uses P before dropout (fmha_fprop_kernel_1xN.h:454 vs :471)
+      if (kDropout) l_i += rs;  // the sum uses P before dropout (fmha_fprop_kernel_1xN.h:454 vs :471)
 
       if (kDropout) {
 #pragma unroll
@@ -237,11 +268,12 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
 #pragma unroll
           for (int i = 0; i < 8; i++) pf[i] = s[kb][8 * t + i];
           const vec8 pb = cvt8<T>(pf);
+          if (!kDropout) l_i = sum8_acc(pb, l_i);
 #pragma unroll
           for (int db = 0; db < DV / 32; db++) {
-            const T* vp = Vs + (kb * 32 + 16 * t) * VS + db * 32 + vtr_off;
+            const T* vp = Vs + (kb * 32 + 16 * t) * D + voff[db];
             u32x2 lo = lds_read_tr16(vp);
-            u32x2 hi = lds_read_tr16(vp + 8 * VS);
+            u32x2 hi = lds_read_tr16(vp + 8 * D);
             u32x4 av = {lo[0], lo[1], hi[0], hi[1]};
             o_acc[db] = E::mfma32(bitcast<vec8>(av), pb, o_acc[db]);
           }
