@@ -26,6 +26,7 @@
 
 #include "fa_common.h"
 #include "fa_params.h"
+#include "fa_stage.h"
 
 namespace fa {
 
@@ -37,17 +38,17 @@ struct BwdCfg {
   static constexpr int BM = kBwdBM;  // query rows per step
   static constexpr int BN = kBwdBN;  // keys per workgroup
   static constexpr int DV = D < 32 ? 32 : D;
-  static constexpr int RS = DV + (D == 128 ? 24 : 8);  // row stride (elements) of the Q / dO tiles: conflict-free for
-                                                       // both the row-fragment and the transposed reads
-  static constexpr int kOffQ = 0;
-  static constexpr int kOffDO = kOffQ + BM * RS * 2;
-  static constexpr int kOffLse = kOffDO + BM * RS * 2;
-  static constexpr int kOffDk = kOffLse + BM * 4;
-  static constexpr int kTileBytes = kOffDk + BM * 4;
+  // Q tile followed by dO tile, both read as row fragments and transposed, double buffered (see fa_stage.h),
+  // then two buffers of per-row statistics (lse and -Dk)
+  typedef TilePairStager<D, BM, kSwzDual, kSwzDual> Stager;
+  static constexpr int kBufBytes = Stager::kPairBytes;
+  static constexpr int kSlack = D < 32 ? 64 : 0;  // the 32-wide transposed reads run past a 16-wide row
+  static constexpr int kOffStat = 2 * kBufBytes + kSlack;
+  static constexpr int kStatBytes = 2 * BM * 4;   // lse[BM], -Dk[BM]
+  static constexpr int kTileBytes = kOffStat + 2 * kStatBytes;
   static constexpr int kEpiBytes = BN * (D + 8) * 2;
   static constexpr int kLdsBytes = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
   static constexpr int CH = D / 8;
-  static constexpr int CPT = (BM * CH + 255) / 256;  // 16-byte chunks per thread for a Q / dO tile
   static constexpr int kMinBlocks = D <= 64 ? 2 : 1;
 };
 
@@ -57,13 +58,9 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
   using E = Elem<T>;
   using vec8 = typename E::vec8;
   using vec4 = typename E::vec4;
-  constexpr int BM = Cfg::BM, BN = Cfg::BN, DV = Cfg::DV, RS = Cfg::RS, CH = Cfg::CH, CPT = Cfg::CPT;
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, DV = Cfg::DV, CH = Cfg::CH, kBufBytes = Cfg::kBufBytes;
 
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
-  T* Ql = reinterpret_cast<T*>(lds_raw + Cfg::kOffQ);
-  T* dOl = reinterpret_cast<T*>(lds_raw + Cfg::kOffDO);
-  float* lse_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffLse);
-  float* dk_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffDk);
 
   // XCD-aware id map (see map_tile): the key tiles of one (batch, head) share one XCD's L2 copy of Q and dO.
   int bh, kt;  // under a causal mask the first key tiles see the most query rows: rank order is already heavy-first
@@ -76,9 +73,9 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
   const int n0 = kt * BN;
   if (n0 >= Lk) return;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 31, hf = lane >> 5;
-  const int j16 = lane & 15, g16 = lane >> 4;
   const int key = n0 + wave * 32 + c;  // this lane's key (sequence-local)
 
   // ---- K and V fragments of this wave's 32 keys (B operands), registers for the whole kernel.
@@ -96,38 +93,22 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
       vreg[ks] = bitcast<vec8>(bb);
     }
   }
-  if (D < 32) {  // zero padding columns of the row-major tiles (read by the 32-wide transposed fragments)
-    for (int i = tid; i < BM * (DV - D); i += 256) {
-      Ql[(i / (DV - D)) * RS + D + i % (DV - D)] = (T)0.f;
-      dOl[(i / (DV - D)) * RS + D + i % (DV - D)] = (T)0.f;
-    }
-  }
-
   int mt_begin = 0;
   if (kCausal) mt_begin = n0 / BM;  // query rows above the tile's first key see none of its keys
   const int mt_end = (Lq + BM - 1) / BM;
 
-  const T* qbase = reinterpret_cast<const T*>(p.q) + (int64_t)q_begin * p.q_rs + (int64_t)h * p.q_hs;
-  const T* dobase = reinterpret_cast<const T*>(p.dout) + (int64_t)q_begin * p.do_rs + (int64_t)h * p.do_hs;
   const float* lsebase = p.lse + ((int64_t)b * p.H + h) * p.lse_stride;
   const float* dsbase = p.dsoftmax + ((int64_t)b * p.H + h) * p.sq_r;
 
-  u32x4 qpre[CPT], dopre[CPT];
+  // ---- staging: Q and dO tiles go global -> LDS directly (waves 0,1: Q, waves 2,3: dO); the 2 x BM row statistics
+  // pass through one register of threads 0 .. 2*BM-1 because they are transformed on the way.
+  typename Cfg::Stager stager;
+  stager.init(wave, lane, reinterpret_cast<const T*>(p.q) + (int64_t)q_begin * p.q_rs + (int64_t)h * p.q_hs, p.q_rs,
+              reinterpret_cast<const T*>(p.dout) + (int64_t)q_begin * p.do_rs + (int64_t)h * p.do_hs, p.do_rs);
   float statpre = 0.f;
-  auto prefetch = [&](int mt) {
+  auto stage = [&](int mt, int buf) {
     const int m0 = mt * BM;
-#pragma unroll
-    for (int i = 0; i < CPT; i++) {
-      const int ch = tid + i * 256;
-      const int row = ch / CH, col = (ch % CH) * 8;
-      if ((BM * CH % 256 == 0 || ch < BM * CH) && m0 + row < Lq) {
-        qpre[i] = ld_global16(qbase + (int64_t)(m0 + row) * p.q_rs + col);
-        dopre[i] = ld_global16(dobase + (int64_t)(m0 + row) * p.do_rs + col);
-      } else {
-        qpre[i] = u32x4{0, 0, 0, 0};
-        dopre[i] = u32x4{0, 0, 0, 0};
-      }
-    }
+    stager.issue(lds_raw + buf * kBufBytes, m0, Lq);
     if (tid < BM) {  // lse, scaled to base 2; +inf switches a row off (P = 0)
       const int row = m0 + tid;
       float x = INFINITY;
@@ -140,19 +121,6 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
       const int row = m0 + tid - BM;
       statpre = row < Lq ? -dsbase[row] : 0.f;  // kept negated: the dP accumulator starts from -Dk
     }
-  };
-  auto commit = [&]() {
-#pragma unroll
-    for (int i = 0; i < CPT; i++) {
-      const int ch = tid + i * 256;
-      const int row = ch / CH, col = (ch % CH) * 8;
-      if (BM * CH % 256 == 0 || ch < BM * CH) {
-        *reinterpret_cast<u32x4*>(Ql + row * RS + col) = qpre[i];
-        *reinterpret_cast<u32x4*>(dOl + row * RS + col) = dopre[i];
-      }
-    }
-    if (tid < BM) lse_l[tid] = statpre;
-    else if (tid < 2 * BM) dk_l[tid - BM] = statpre;
   };
 
   auto tile_active = [&](int mt) -> bool {
@@ -174,18 +142,31 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
     }
 
   const float cs = p.scale_log2;
-  // element offset of a transposed read: row (4*hf + j16/4) [+8], column 16*(g16&1) + 4*(j16&3)
-  const int tr_off = (4 * hf + (j16 >> 2)) * RS + 16 * (g16 & 1) + 4 * (j16 & 3);
+  // element offsets inside a tile of this lane's row fragments and of its transposed reads (rows +0 and +8)
+  int foff[D / 16], tlo[DV / 32], thi[DV / 32];
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ks++) foff[ks] = frag_off<D, kSwzDual>(c, ks * 2 + hf);
+#pragma unroll
+  for (int db = 0; db < DV / 32; db++) {
+    tlo[db] = tr_off<D, kSwzDual>(0, db * 4, lane);
+    thi[db] = tr_off<D, kSwzDual>(8, db * 4, lane);
+  }
+  int buf = 0;
 
   int mt = next_active(mt_begin);
-  if (mt < mt_end) prefetch(mt);
+  if (mt < mt_end) stage(mt, 0);
   while (mt < mt_end) {
     const int m0 = mt * BM;
-    __syncthreads();
-    commit();
-    __syncthreads();
+    wait_vmem();  // this thread's share of tile `mt` has arrived (LDS) / is in statpre
+    float* const lse_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffStat + buf * Cfg::kStatBytes);
+    float* const dk_l = lse_l + BM;
+    if (tid < 2 * BM) lse_l[tid] = statpre;
+    __syncthreads();  // tile `mt` is complete, and nobody still reads the other buffer
     const int mt_next = next_active(mt + 1);
-    if (mt_next < mt_end) prefetch(mt_next);
+    if (mt_next < mt_end) stage(mt_next, buf ^ 1);
+    const T* const Ql = reinterpret_cast<const T*>(lds_raw + buf * kBufBytes);
+    const T* const dOl = Ql + BM * D;
+    buf ^= 1;
 
     const bool diag = kCausal && (m0 < n0 + wave * 32 + 32);  // some (q, key) of this wave's slab has key > q
 
@@ -202,12 +183,12 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
       }
 #pragma unroll
       for (int ks = 0; ks < D / 16; ks++) {
-        vec8 aq = *reinterpret_cast<const vec8*>(Ql + (qb * 32 + c) * RS + ks * 16 + hf * 8);
+        vec8 aq = *reinterpret_cast<const vec8*>(Ql + qb * 32 * D + foff[ks]);
         s = E::mfma32(aq, kreg[ks], s);
       }
 #pragma unroll
       for (int ks = 0; ks < D / 16; ks++) {
-        vec8 ad = *reinterpret_cast<const vec8*>(dOl + (qb * 32 + c) * RS + ks * 16 + hf * 8);
+        vec8 ad = *reinterpret_cast<const vec8*>(dOl + qb * 32 * D + foff[ks]);
         dp = E::mfma32(ad, vreg[ks], dp);
       }
       // ---- P and dS'
@@ -253,12 +234,12 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
         const vec8 db8 = cvt8<T>(df);
 #pragma unroll
         for (int db = 0; db < DV / 32; db++) {
-          const int off = (qb * 32 + 16 * t) * RS + db * 32 + tr_off;
-          u32x2 lo = lds_read_tr16(dOl + off), hi = lds_read_tr16(dOl + off + 8 * RS);
+          const int off = (qb * 32 + 16 * t) * D;
+          u32x2 lo = lds_read_tr16(dOl + off + tlo[db]), hi = lds_read_tr16(dOl + off + thi[db]);
           u32x4 av = {lo[0], lo[1], hi[0], hi[1]};
           acc_dv[db] = E::mfma32(bitcast<vec8>(av), pb, acc_dv[db]);
-          lo = lds_read_tr16(Ql + off);
-          hi = lds_read_tr16(Ql + off + 8 * RS);
+          lo = lds_read_tr16(Ql + off + tlo[db]);
+          hi = lds_read_tr16(Ql + off + thi[db]);
           u32x4 aq = {lo[0], lo[1], hi[0], hi[1]};
           acc_dk[db] = E::mfma32(bitcast<vec8>(aq), db8, acc_dk[db]);
         }
@@ -313,14 +294,15 @@ template <typename T, int D, int BN>
 struct DqCfg {
   static constexpr int BM = kFwdBM;  // query rows per workgroup (same tiling as the forward: shares its sparse map)
   static constexpr int DV = D < 32 ? 32 : D;
-  static constexpr int KS = DV + (D == 128 ? 24 : 8);  // K tile: read both as row fragments and transposed
-  static constexpr int VS = D + 8;                     // V tile: row fragments only
   static constexpr int OS = D + 8;
-  static constexpr int kTileBytes = BN * (KS + VS) * 2;
+  // K tile (read as row fragments and transposed) followed by V tile (row fragments), double buffered (fa_stage.h)
+  typedef TilePairStager<D, BN, kSwzDual, kSwzRow> Stager;
+  static constexpr int kBufBytes = Stager::kPairBytes;
+  static constexpr int kSlack = D < 32 ? 64 : 0;  // the 32-wide transposed reads run past a 16-wide K row
+  static constexpr int kTileBytes = 2 * kBufBytes + kSlack;
   static constexpr int kEpiBytes = BM * OS * 2;
   static constexpr int kLdsBytes = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
   static constexpr int CH = D / 8;
-  static constexpr int CPT = (BN * CH + 255) / 256;
 };
 
 template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse>
@@ -328,11 +310,9 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
   using Cfg = DqCfg<T, D, BN>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
-  constexpr int BM = Cfg::BM, DV = Cfg::DV, KS = Cfg::KS, VS = Cfg::VS, CH = Cfg::CH, CPT = Cfg::CPT;
+  constexpr int BM = Cfg::BM, DV = Cfg::DV, CH = Cfg::CH, kBufBytes = Cfg::kBufBytes;
 
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
-  T* Ks = reinterpret_cast<T*>(lds_raw);
-  T* Vs = Ks + BN * KS;
 
   int bh, rank;
   if (!map_tile<kCausal>(blockIdx.x, p.nq_tiles, p.B * p.H, &bh, &rank)) return;
@@ -345,7 +325,8 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
   const int m0 = qt * BM;
   if (m0 >= Lq) return;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 31, hf = lane >> 5;
   const int mw = m0 + wave * 32;
   const int qrow = mw + c;
@@ -376,45 +357,17 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
   f32x16 negd;
 #pragma unroll
   for (int r = 0; r < 16; r++) negd[r] = kInitNegD ? -dkv : 0.f;
-  if (D < 32) {
-    for (int i = tid; i < BN * (DV - D); i += 256) Ks[(i / (DV - D)) * KS + D + i % (DV - D)] = (T)0.f;
-  }
-
   int n_end = Lk;
   if (kCausal) n_end = n_end < m0 + BM ? n_end : m0 + BM;
   const int ntiles = (n_end + BN - 1) / BN;
 
-  const T* kbase = reinterpret_cast<const T*>(p.k) + (int64_t)k_begin * p.k_rs + (int64_t)h * p.k_hs;
-  const T* vbase = reinterpret_cast<const T*>(p.v) + (int64_t)k_begin * p.v_rs + (int64_t)h * p.v_hs;
+  // ---- K/V staging: global -> LDS without passing through registers (waves 0,1 fetch K tiles, waves 2,3 V tiles).
+  // Keys past the end re-read the last key: their P is masked to 0 below, so they add 0 * finite to dQ.
+  typename Cfg::Stager stager;
+  stager.init(wave, lane, reinterpret_cast<const T*>(p.k) + (int64_t)k_begin * p.k_rs + (int64_t)h * p.k_hs, p.k_rs,
+              reinterpret_cast<const T*>(p.v) + (int64_t)k_begin * p.v_rs + (int64_t)h * p.v_hs, p.v_rs);
+  auto stage = [&](int it, int buf) { stager.issue(lds_raw + buf * kBufBytes, it * BN, Lk); };
 
-  u32x4 kpre[CPT], vpre[CPT];
-  auto prefetch = [&](int it) {
-    const int n0 = it * BN;
-#pragma unroll
-    for (int i = 0; i < CPT; i++) {
-      const int ch = tid + i * 256;
-      const int row = ch / CH, col = (ch % CH) * 8;
-      const int key = n0 + row;
-      if ((BN * CH % 256 == 0 || ch < BN * CH) && key < Lk) {
-        kpre[i] = ld_global16(kbase + (int64_t)key * p.k_rs + col);
-        vpre[i] = ld_global16(vbase + (int64_t)key * p.v_rs + col);
-      } else {  // zero keys contribute dS' * 0 to dQ
-        kpre[i] = u32x4{0, 0, 0, 0};
-        vpre[i] = u32x4{0, 0, 0, 0};
-      }
-    }
-  };
-  auto commit = [&]() {
-#pragma unroll
-    for (int i = 0; i < CPT; i++) {
-      const int ch = tid + i * 256;
-      const int row = ch / CH, col = (ch % CH) * 8;
-      if (BN * CH % 256 == 0 || ch < BN * CH) {
-        *reinterpret_cast<u32x4*>(Ks + row * KS + col) = kpre[i];
-        *reinterpret_cast<u32x4*>(Vs + row * VS + col) = vpre[i];
-      }
-    }
-  };
   auto tile_active = [&](int it) -> bool {
     if (!kSparse) return true;
     return p.sp.actq[qt * p.sp.ncb + ((it * BN) >> 8)] != 0;
@@ -431,18 +384,34 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
     for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
 
   const float cs = p.scale_log2;
-  const int j16 = lane & 15, g16 = lane >> 4;
-  const int ktr_off = (4 * hf + (j16 >> 2)) * KS + 16 * (g16 & 1) + 4 * (j16 & 3);
+  // element offsets inside a tile: row fragments of K (dual swizzle) and V, transposed reads of K (rows +0, +8)
+  int kfoff[D / 16], vfoff[D / 16], tlo[DV / 32], thi[DV / 32];
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ks++) {
+    kfoff[ks] = frag_off<D, kSwzDual>(c, ks * 2 + hf);
+    vfoff[ks] = frag_off<D, kSwzRow>(c, ks * 2 + hf);
+  }
+#pragma unroll
+  for (int db = 0; db < DV / 32; db++) {
+    tlo[db] = tr_off<D, kSwzDual>(0, db * 4, lane);
+    thi[db] = tr_off<D, kSwzDual>(8, db * 4, lane);
+  }
+  int buf = 0;
 
   int it = next_active(0);
-  if (it < ntiles) prefetch(it);
+  if (it < ntiles) stage(it, 0);
   while (it < ntiles) {
     const int n0 = it * BN;
-    __syncthreads();
-    commit();
-    __syncthreads();
+    // Opaque redefinition of the accumulators (keeps the register allocator from copying them around the loop)
+#pragma unroll
+    for (int i = 0; i < DV / 32; i++) asm volatile("" : "+v"(acc[i]));
+    wait_vmem();      // this wave's share of tile `it` is in LDS
+    __syncthreads();  // so is everyone else's, and nobody still reads the other buffer
     const int it_next = next_active(it + 1);
-    if (it_next < ntiles) prefetch(it_next);
+    if (it_next < ntiles) stage(it_next, buf ^ 1);
+    const T* const Ks = reinterpret_cast<const T*>(lds_raw + buf * kBufBytes);
+    const T* const Vs = Ks + BN * D;
+    buf ^= 1;
 
     bool wave_work = true;
     if (kCausal && n0 > mw + 31) wave_work = false;
@@ -453,7 +422,8 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
       if (__ballot(row_on) == 0) wave_work = false;
     }
     if (wave_work) {
-      const bool diag = kCausal && (n0 + BN - 1 > mw);
+      // tiles that straddle the key length, the diagonal or an inactive row block get their dead scores set to -inf
+      const bool need_mask = (n0 + BN > Lk) || (kCausal && (n0 + BN - 1 > mw)) || (kSparse && !row_on);
 #pragma unroll
       for (int kb = 0; kb < BN / 32; kb++) {
         f32x16 s, dp = negd;
@@ -461,24 +431,29 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
         for (int r = 0; r < 16; r++) s[r] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < D / 16; ks++) {
-          vec8 a = *reinterpret_cast<const vec8*>(Ks + (kb * 32 + c) * KS + ks * 16 + hf * 8);
+          vec8 a = *reinterpret_cast<const vec8*>(Ks + kb * 32 * D + kfoff[ks]);
           s = E::mfma32(a, qreg[ks], s);
         }
 #pragma unroll
         for (int ks = 0; ks < D / 16; ks++) {
-          vec8 a = *reinterpret_cast<const vec8*>(Vs + (kb * 32 + c) * VS + ks * 16 + hf * 8);
+          vec8 a = *reinterpret_cast<const vec8*>(Vs + kb * 32 * D + vfoff[ks]);
           dp = E::mfma32(a, doreg[ks], dp);
+        }
+        if (need_mask) {
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int key = n0 + kb * 32 + (r >> 2) * 8 + hf * 4 + (r & 3);
+            bool dead = key >= Lk;
+            if (kCausal) dead = dead || key > qrow;
+            if (kSparse) dead = dead || !row_on;
+            if (dead) s[r] = -INFINITY;
+          }
         }
         uint32_t keep = 0xffffu;
         if (kDropout) keep = keep16_row_layout(p.pk, (uint32_t)bh, qrow, n0 + kb * 32, hf, p.keep_thr);
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          float pe = fast_exp2(__builtin_fmaf(s[r], cs, -lse2));
-          if (kCausal && diag) {
-            const int key = n0 + kb * 32 + (r >> 2) * 8 + hf * 4 + (r & 3);
-            if (key > qrow) pe = 0.f;
-          }
-          if (kSparse && !row_on) pe = 0.f;
+          const float pe = fast_exp2(__builtin_fmaf(s[r], cs, -lse2));  // 0 for dead scores and switched-off rows
           float dpe = kInitNegD ? dp[r] : dp[r] - dkv;  // dP - Dk
           if (kDropout && !((keep >> r) & 1u)) dpe = -dkv;
           s[r] = pe * dpe;  // dS'
@@ -491,8 +466,8 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
           const vec8 dsb = cvt8<T>(df);
 #pragma unroll
           for (int db = 0; db < DV / 32; db++) {
-            const T* kp = Ks + (kb * 32 + 16 * t) * KS + db * 32 + ktr_off;
-            u32x2 lo = lds_read_tr16(kp), hi = lds_read_tr16(kp + 8 * KS);
+            const T* kp = Ks + (kb * 32 + 16 * t) * D;
+            u32x2 lo = lds_read_tr16(kp + tlo[db]), hi = lds_read_tr16(kp + thi[db]);
             u32x4 av = {lo[0], lo[1], hi[0], hi[1]};
             acc[db] = E::mfma32(bitcast<vec8>(av), dsb, acc[db]);
           }

@@ -16,6 +16,7 @@
 
 #include "fa_common.h"
 #include "fa_params.h"
+#include "fa_stage.h"
 
 namespace fa {
 
@@ -25,25 +26,14 @@ struct FwdCfg {
   static constexpr int NW = 4;                 // waves per workgroup, 32 query rows each
   static constexpr int DV = D < 32 ? 32 : D;   // rows of the V^T MFMA operand (for D = 16 the upper 16 are don't-care)
   static constexpr int OS = D + 8;             // epilogue staging row stride
-  // K and V tiles sit in LDS unpadded, BN rows of CH 16-byte chunks, filled by direct-to-LDS loads (each wave
-  // instruction deposits 64 consecutive chunks).  Bank conflicts are avoided by permuting the chunks of a row:
-  // chunk ch of tile row r is stored at position ch ^ k_swz(r) (K, read as row fragments with ds_read_b128) or
-  // ch ^ v_swz(r) (V, read transposed with ds_read_b64_tr_b16, which fetches aligned chunk pairs).
-  static constexpr int CH = D / 8;
-  static constexpr int RPB = CH >= 16 ? 1 : 16 / CH;            // tile rows per 256 bytes
-  static constexpr int kKBytes = BN * D * 2;
-  static constexpr int kBufBytes = 2 * kKBytes;                 // one K tile followed by one V tile
+  // K tile (read as row fragments) followed by V tile (read transposed), double buffered; see fa_stage.h
+  typedef TilePairStager<D, BN, kSwzRow, kSwzTr> Stager;
+  static constexpr int kBufBytes = Stager::kPairBytes;
   static constexpr int kSlack = D < 32 ? 64 : 0;                // the 32-wide transposed reads run past a 16-wide V row
-  static constexpr int kTileBytes = 2 * kBufBytes + kSlack;     // double buffered
+  static constexpr int kTileBytes = 2 * kBufBytes + kSlack;
   static constexpr int kEpiBytes = BM * OS * 2;
   static constexpr int kLdsBytes = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
-  static constexpr int TI = 2 * BN * CH / 64;                   // direct-to-LDS wave instructions per tile (K, then V)
-  static constexpr int NI = TI / NW;                            // per wave: waves 0,1 fetch K, waves 2,3 fetch V
-  static constexpr int RPI = 64 / CH;                           // tile rows per instruction
-  static constexpr int NOFF = 16 / RPI > 0 ? 16 / RPI : 1;      // distinct per-lane source offsets (swizzle period 16 rows)
-  static_assert(TI % NW == 0 && NI % NOFF == 0, "tile does not split evenly over the waves");
-  static __device__ __forceinline__ int k_swz(int r) { return (r / RPB) % CH; }
-  static __device__ __forceinline__ int v_swz(int r) { return CH >= 4 ? 2 * ((r / RPB) % (CH / 2)) : 0; }
+  static constexpr int CH = D / 8;
 };
 
 template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse>
@@ -51,10 +41,7 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
   using Cfg = FwdCfg<T, D, BN>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
-  constexpr int BM = Cfg::BM, DV = Cfg::DV, CH = Cfg::CH, NI = Cfg::NI, RPI = Cfg::RPI, NOFF = Cfg::NOFF;
-  constexpr int kKBytes = Cfg::kKBytes, kBufBytes = Cfg::kBufBytes;
-  typedef __attribute__((address_space(1))) const void* gptr_t;
-  typedef __attribute__((address_space(3))) void* lptr_t;
+  constexpr int BM = Cfg::BM, DV = Cfg::DV, CH = Cfg::CH, kBufBytes = Cfg::kBufBytes;
 
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
 
@@ -94,42 +81,11 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
   if (kCausal) n_end = n_end < m0 + BM ? n_end : m0 + BM;
   const int ntiles = (n_end + BN - 1) / BN;
 
-  // ---- K/V staging: global -> LDS without passing through registers.  Waves 0,1 bring in the K tile, waves 2,3 the V
-  // tile, NI instructions of RPI rows each.  The source address is a wave-uniform row base plus a per-lane offset that
-  // encodes the lane's row within the instruction and the (swizzled) chunk it fetches.
-  const bool stage_k = wave < 2;
-  const int g0 = (wave & 1) * NI;  // first instruction slot of this wave inside its tile
-  const char* const tbase = stage_k
-      ? reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.k) + (int64_t)k_begin * p.k_rs + (int64_t)h * p.k_hs)
-      : reinterpret_cast<const char*>(reinterpret_cast<const T*>(p.v) + (int64_t)k_begin * p.v_rs + (int64_t)h * p.v_hs);
-  const int64_t rsb = (stage_k ? p.k_rs : p.v_rs) * 2;  // source row stride in bytes
-  const int lds_dst0 = (stage_k ? 0 : kKBytes) + g0 * 1024;
-  const int rl = lane / CH, pch = lane % CH;
-  uint32_t src_off[NOFF];
-#pragma unroll
-  for (int j = 0; j < NOFF; j++) {
-    const int r = j * RPI + rl;
-    src_off[j] = (uint32_t)(rl * rsb) + 16u * (pch ^ (stage_k ? Cfg::k_swz(r) : Cfg::v_swz(r)));
-  }
-  auto stage = [&](int it, int buf) {
-    const int n0 = it * BN;
-    const char* const tb = tbase + ((int64_t)n0 + g0 * RPI) * rsb;
-    if (__builtin_expect(n0 + BN <= Lk, 1)) {
-#pragma unroll
-      for (int i = 0; i < NI; i++)
-        __builtin_amdgcn_global_load_lds((gptr_t)(tb + i * RPI * rsb + src_off[i % NOFF]),
-                                         (lptr_t)(lds_raw + buf * kBufBytes + lds_dst0 + i * 1024), 16, 0, 0);
-    } else {  // last, partial tile: rows past the end re-read the last valid row (their scores are masked below)
-#pragma unroll
-      for (int i = 0; i < NI; i++) {
-        const int r = (g0 + i) * RPI + rl;
-        const int rc = n0 + r < Lk ? r : Lk - 1 - n0;
-        const int ch = pch ^ (stage_k ? Cfg::k_swz(r) : Cfg::v_swz(r));
-        __builtin_amdgcn_global_load_lds((gptr_t)(tbase + ((int64_t)n0 + rc) * rsb + 16 * ch),
-                                         (lptr_t)(lds_raw + buf * kBufBytes + lds_dst0 + i * 1024), 16, 0, 0);
-      }
-    }
-  };
+  // ---- K/V staging: global -> LDS without passing through registers (waves 0,1 fetch K tiles, waves 2,3 V tiles)
+  typename Cfg::Stager stager;
+  stager.init(wave, lane, reinterpret_cast<const T*>(p.k) + (int64_t)k_begin * p.k_rs + (int64_t)h * p.k_hs, p.k_rs,
+              reinterpret_cast<const T*>(p.v) + (int64_t)k_begin * p.v_rs + (int64_t)h * p.v_hs, p.v_rs);
+  auto stage = [&](int it, int buf) { stager.issue(lds_raw + buf * kBufBytes, it * BN, Lk); };
 
   // Sparse: tile `it` is computed iff its 256-key block is active for any 16-row block of this query tile.
   auto tile_active = [&](int it) -> bool {
@@ -151,18 +107,12 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
   float l_i = 0.f;        // this lane's share of the running row sum (other share in lane^32)
 
   const float cs = p.scale_log2;
-  // operand addressing of the transposed V reads (see lds_read_tr16)
-  const int j16 = lane & 15, g16 = lane >> 4;
-  int voff[DV / 32];  // element offsets of this lane's transposed V reads
-  {
-    const int vr = 4 * hf + (j16 >> 2);
+  int voff[DV / 32];  // element offsets of this lane's transposed V reads and K row fragments inside a tile
 #pragma unroll
-    for (int db = 0; db < DV / 32; db++)
-      voff[db] = vr * D + (((db * 4 + 2 * (g16 & 1)) ^ Cfg::v_swz(vr)) * 8) + 4 * (j16 & 3);
-  }
-  int koff[D / 16];  // element offsets of this lane's K row fragments
+  for (int db = 0; db < DV / 32; db++) voff[db] = tr_off<D, kSwzTr>(0, db * 4, lane);
+  int koff[D / 16];
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ks++) koff[ks] = c * D + (((ks * 2 + hf) ^ Cfg::k_swz(c)) * 8);
+  for (int ks = 0; ks < D / 16; ks++) koff[ks] = frag_off<D, kSwzRow>(c, ks * 2 + hf);
   int buf = 0;
 
   int it = next_active(0);
@@ -173,7 +123,7 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
     // ties the last MFMA's result to the registers the epilogue reads and copies all of O back on every trip.
 #pragma unroll
     for (int i = 0; i < DV / 32; i++) asm volatile("" : "+v"(o_acc[i]));
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile `it` is in LDS
+    wait_vmem();                         // this wave's share of tile `it` is in LDS
     __syncthreads();                     // so is everyone else's, and nobody still reads the other buffer
     const int it_next = next_active(it + 1);
     if (it_next < ntiles) stage(it_next, buf ^ 1);
