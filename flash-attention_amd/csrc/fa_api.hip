@@ -256,8 +256,7 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
   p.keep_thr = (uint32_t)std::floor(p_keep * 65535.0);
   p.pk = make_key(a->philox_seed, a->philox_offset);
 
-  FA_LAUNCH(fa::launch_bwd_preprocess(p, a->dtype, a->head_dim, stream));
-  FA_LAUNCH(fa::launch_bwd(p, 0, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));  // dQ
+  FA_LAUNCH(fa::launch_bwd(p, 0, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));  // dQ, softmax_d
   if (a->ev_main_start) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(a->ev_main_start), stream));
   FA_LAUNCH(fa::launch_bwd(p, 1, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));  // dK, dV
   if (a->ev_main_stop) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(a->ev_main_stop), stream));

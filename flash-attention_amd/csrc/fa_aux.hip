@@ -42,37 +42,6 @@ __global__ void sparse_maps_kernel(const int32_t* blockmask, uint8_t* act16, uin
   if (rb / rpq2 < nqt2) actk[cb * nqt2 + rb / rpq2] = 1;
 }
 
-template <typename T, int D>
-__global__ void __launch_bounds__(256) bwd_preprocess_kernel(const BwdParams p) {
-  constexpr int TPR = D / 8;         // threads per (row, head)
-  constexpr int RPB = 256 / TPR;     // (row, head) pairs per block
-  const int sub = threadIdx.x % TPR;
-  const int64_t rh = (int64_t)blockIdx.x * RPB + threadIdx.x / TPR;
-  const int64_t n = (int64_t)p.total_q * p.H;
-  if (rh >= n) return;
-  const int h = (int)(rh % p.H);
-  const int64_t row = rh / p.H;
-  const T* dop = reinterpret_cast<const T*>(p.dout) + row * p.do_rs + (int64_t)h * p.do_hs + sub * 8;
-  const T* op = reinterpret_cast<const T*>(p.out) + row * p.o_rs + (int64_t)h * p.o_hs + sub * 8;
-  typedef typename Elem<T>::vec8 vec8;
-  const vec8 a = bitcast<vec8>(ld_global16(dop)), b = bitcast<vec8>(ld_global16(op));
-  float acc = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; i++) acc += (float)a[i] * (float)b[i];
-#pragma unroll
-  for (int off = TPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
-  if (sub == 0) {
-    // locate (batch, position) of this row: binary search in cu_seqlens_q
-    int lo = 0, hi = p.B;
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (p.cu_q[mid] <= row) lo = mid; else hi = mid;
-    }
-    const int pos = (int)(row - p.cu_q[lo]);
-    if (pos >= 0 && pos < p.sq_r) p.dsoftmax[((int64_t)lo * p.H + h) * p.sq_r + pos] = acc * p.p_keep;
-  }
-}
-
 // One thread per (query row, key) element of S_dmask.  Slow scalar dot products: this path exists for tests
 // (flash_attn_interface.py:163-173).  The value is the normalised probability exp(scale*s - lse); its sign
 // bit is set when dropout dropped the element.
@@ -141,29 +110,6 @@ hipError_t launch_build_sparse_maps(const int32_t* blockmask, uint8_t* act16, ui
   return hipGetLastError();
 }
 
-namespace {
-template <typename T, int D>
-hipError_t pre_one(const BwdParams& p, hipStream_t stream) {
-  const int64_t n = (int64_t)p.total_q * p.H;
-  constexpr int RPB = 256 / (D / 8);
-  hipLaunchKernelGGL((bwd_preprocess_kernel<T, D>), dim3((unsigned)((n + RPB - 1) / RPB)), dim3(256), 0, stream, p);
-  return hipGetLastError();
-}
-}  // namespace
-
-#define FA_DISPATCH_TD(fn)                                                          \
-  switch (head_dim) {                                                               \
-    case 16: return dtype == 0 ? fn<_Float16, 16>(p, stream) : fn<__bf16, 16>(p, stream);   \
-    case 32: return dtype == 0 ? fn<_Float16, 32>(p, stream) : fn<__bf16, 32>(p, stream);   \
-    case 64: return dtype == 0 ? fn<_Float16, 64>(p, stream) : fn<__bf16, 64>(p, stream);   \
-    case 128: return dtype == 0 ? fn<_Float16, 128>(p, stream) : fn<__bf16, 128>(p, stream); \
-    default: return hipErrorInvalidValue;                                           \
-  }
-
-hipError_t launch_bwd_preprocess(const BwdParams& p, int dtype, int head_dim, hipStream_t stream) {
-  if ((int64_t)p.total_q * p.H == 0) return hipSuccess;
-  FA_DISPATCH_TD(pre_one)
-}
 hipError_t launch_dump_probs(const DumpParams& p, int dtype, hipStream_t stream) {
   dim3 grid((p.sk_r + 255) / 256, p.sq_r, p.B * p.H);
   if (dtype == 0) hipLaunchKernelGGL(dump_probs_kernel<_Float16>, grid, dim3(256), 0, stream, p);

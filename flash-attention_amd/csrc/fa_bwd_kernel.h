@@ -331,24 +331,33 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
   const int mw = m0 + wave * 32;
   const int qrow = mw + c;
 
-  // ---- Q and dO fragments (B operands), lse and Dk of this lane's query row
+  // ---- Q and dO fragments (B operands), lse and Dk of this lane's query row.  Dk = keep * rowsum(dO o O) is computed
+  // here (fmha_dgrad_kernel_1xN_loop.h:15-30 does it on the first column block) and stored to softmax_d, which the
+  // dK/dV kernel, launched after this one, reads.
   vec8 qreg[D / 16], doreg[D / 16];
   float lse2 = INFINITY, dkv = 0.f;  // +inf switches the row off
   {
     const int qr = qrow < Lq ? qrow : Lq - 1;
     const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)(q_begin + qr) * p.q_rs + (int64_t)h * p.q_hs + hf * 8;
     const T* dp_ = reinterpret_cast<const T*>(p.dout) + (int64_t)(q_begin + qr) * p.do_rs + (int64_t)h * p.do_hs + hf * 8;
+    const T* op = reinterpret_cast<const T*>(p.out) + (int64_t)(q_begin + qr) * p.o_rs + (int64_t)h * p.o_hs + hf * 8;
+    float dsum = 0.f;
 #pragma unroll
     for (int ks = 0; ks < D / 16; ks++) {
       u32x4 a = ld_global16(qp + ks * 16), bb = ld_global16(dp_ + ks * 16);
+      const vec8 ov = bitcast<vec8>(ld_global16(op + ks * 16));
       if (qrow >= Lq) { a = u32x4{0, 0, 0, 0}; bb = u32x4{0, 0, 0, 0}; }
       qreg[ks] = bitcast<vec8>(a);
       doreg[ks] = bitcast<vec8>(bb);
+#pragma unroll
+      for (int i = 0; i < 8; i++) dsum = __builtin_fmaf((float)doreg[ks][i], (float)ov[i], dsum);
     }
+    dsum = half_sum(dsum) * p.p_keep;  // lanes l and l^32 hold the two halves of each 16-element group of the row
     if (qrow < Lq) {
       const float x = p.lse[((int64_t)b * p.H + h) * p.lse_stride + qrow];
       lse2 = (x == -INFINITY) ? INFINITY : x * kLog2e;
-      dkv = p.dsoftmax[((int64_t)b * p.H + h) * p.sq_r + qrow];
+      dkv = dsum;
+      if (hf == 0) p.dsoftmax[((int64_t)b * p.H + h) * p.sq_r + qrow] = dsum;
     }
   }
   // For d <= 64 the dP^T accumulator starts from -Dk of this lane's query row (16 registers that save 16 subtractions

@@ -150,7 +150,6 @@ hipError_t launch_fill_f32(float* p, size_t n, float value, hipStream_t stream);
 hipError_t launch_zero_rows(void* base, int64_t row_stride, int64_t head_stride, int total, int H, int D,
                             hipStream_t stream);
 // softmax_d = keep * rowsum(dO o O) (fmha_dgrad_kernel_1xN_loop.h:15-30).
-hipError_t launch_bwd_preprocess(const BwdParams& p, int dtype, int head_dim, hipStream_t stream);
 
 // Tile shapes, needed by the front end for grid sizes and workspace layout.
 constexpr int kFwdBM = 128;   // query rows per forward workgroup
