@@ -135,6 +135,8 @@ def main():
     ap.add_argument("--all", action="store_true", help="also time the other BASELINE configurations (stderr table)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
+    ap.add_argument("--settle", type=float, default=0.2,
+                    help="seconds of untimed steps before the warm-up (0 for counter-collection runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     a = ap.parse_args()
@@ -156,7 +158,7 @@ def main():
 
     B, H, D, N = 8, 12, 64, 2048
     w = Workload(torch, B, H, D, N, torch.float16)
-    t = time_steps(torch, be, w, a.steps, a.warmup)
+    t = time_steps(torch, be, w, a.steps, a.warmup, a.settle)
     fwd_flops = attention_flops(B, H, N, D)
     step_flops = 3.5 * fwd_flops
     value = step_flops / (t["ms_per_step"] * 1e-3) / 1e12
@@ -167,7 +169,7 @@ def main():
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(t["ms_per_step"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic N(0,1) q,k,v,dout resident in HBM",
-        "settle": "0.2 s of untimed steps before the warm-up steps (clock governor)",
+        "settle": "%.1f s of untimed steps before the warm-up steps (clock governor)" % a.settle,
         "config": {"workload": "headline: fp16 packed qkv [16384,3,12,64], B=8 H=12 d=64 N=2048 equal lengths, "
                                "non-causal, dropout 0, fwd+bwd with dout~N(0,1)"},
         "pct_of_mfma_peak": round(100.0 * value / MFMA_PEAK_TFLOPS, 2),
@@ -201,7 +203,7 @@ def main():
               file=sys.stderr)
         for name, kw in cfgs:
             wl = Workload(torch, **kw)
-            tt = time_steps(torch, be, wl, max(10, a.steps // 2), 5)
+            tt = time_steps(torch, be, wl, max(10, a.steps // 2), 5, a.settle)
             fb = 3.5 * wl.fwd_flops / ((tt["fwd_ms"] + tt["bwd_ms"]) * 1e-3) / 1e12
             gbs = (wl.bytes_fwd + wl.bytes_bwd) / ((tt["fwd_ms"] + tt["bwd_ms"]) * 1e-3) / 1e9
             print("%-28s %9.4f %9.4f %9.1f %9.1f %8.2f %10.1f" % (
