@@ -209,6 +209,31 @@ def main():
             print("%-28s %9.4f %9.4f %9.1f %9.1f %8.2f %10.1f" % (
                 name, tt["fwd_ms"], tt["bwd_ms"], wl.fwd_flops / (tt["fwd_ms"] * 1e-3) / 1e12, fb,
                 100 * fb / MFMA_PEAK_TFLOPS, gbs), file=sys.stderr)
+        # unpad / pad (row gather and scatter, HBM-bound): BERT-large-like padded batch, 75 % of the tokens valid
+        from flash_attn.bert_padding import pad_input, unpad_input
+        Bp, Sp, dim = 64, 512, 1024
+        gen = torch.Generator().manual_seed(0)
+        lens_p = torch.randint(Sp // 2, Sp + 1, (Bp,), generator=gen)
+        mask = (torch.arange(Sp)[None, :] < lens_p[:, None]).cuda()
+        hidden = torch.randn(Bp, Sp, dim, device="cuda", dtype=torch.float16)
+        rows, idx, _, _ = unpad_input(hidden, mask)
+        nnz = rows.shape[0]
+        for name, fn, nbytes in (
+                ("unpad_input (gather)", lambda: be.gather_rows(hidden.view(Bp * Sp, dim), idx), 2 * nnz * dim * 2 + nnz * 8),
+                ("pad_input (scatter)", lambda: be.scatter_rows(rows, idx, Bp * Sp), (nnz + Bp * Sp) * dim * 2 + nnz * 8)):
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(50):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / 50
+            print("%-28s %9.4f ms  %8.1f GB/s of %d (%.1f %% of HBM peak)  [B=%d S=%d dim=%d fp16, %d of %d tokens valid]"
+                  % (name, ms, nbytes / ms / 1e6, HBM_PEAK_GBS, 100 * nbytes / ms / 1e6 / HBM_PEAK_GBS, Bp, Sp, dim, nnz, Bp * Sp),
+                  file=sys.stderr)
     print(json.dumps(res))
 
 

@@ -293,6 +293,47 @@ void fa_round_seqlens(int32_t head_dim, int32_t max_seqlen_q, int32_t max_seqlen
 
 uint64_t fa_philox_offset_increment(void) { return 4; }
 
+namespace {
+// widest chunk (bytes, power of two <= 16) that divides the row width and every address involved
+int row_vector_bytes(const void* a, const void* b, int64_t row_bytes, int64_t sa, int64_t sb) {
+  uint64_t m = (uint64_t)reinterpret_cast<uintptr_t>(a) | (uint64_t)reinterpret_cast<uintptr_t>(b) | (uint64_t)row_bytes |
+               (uint64_t)sa | (uint64_t)sb | 16u;
+  return (int)(m & (~m + 1));  // lowest set bit
+}
+}  // namespace
+
+int fa_gather_rows(const void* src, void* dst, const int64_t* indices, int64_t n_indices, int64_t n_src_rows,
+                   int64_t row_bytes, int64_t src_row_stride, int64_t dst_row_stride, void* stream) {
+  FA_REQUIRE(n_indices >= 0 && n_src_rows >= 0 && row_bytes >= 0, "fa_gather_rows: negative size");
+  FA_REQUIRE(src_row_stride >= row_bytes && dst_row_stride >= row_bytes, "fa_gather_rows: row stride smaller than row");
+  if (n_indices == 0 || row_bytes == 0) return FA_OK;
+  FA_REQUIRE(src && dst && indices, "fa_gather_rows: null pointer");
+  const int vec = row_vector_bytes(src, dst, row_bytes, src_row_stride, dst_row_stride);
+  FA_LAUNCH(fa::launch_gather_rows(src, dst, indices, n_indices, n_src_rows, row_bytes, src_row_stride, dst_row_stride, vec,
+                                   reinterpret_cast<hipStream_t>(stream)));
+  return FA_OK;
+}
+
+size_t fa_scatter_rows_workspace_bytes(int64_t n_dst_rows) { return n_dst_rows > 0 ? (size_t)n_dst_rows * 4 : 0; }
+
+int fa_scatter_rows(const void* src, void* dst, const int64_t* indices, int64_t n_indices, int64_t n_dst_rows,
+                    int64_t row_bytes, int64_t src_row_stride, int64_t dst_row_stride, void* workspace,
+                    size_t workspace_bytes, void* stream) {
+  FA_REQUIRE(n_indices >= 0 && n_dst_rows >= 0 && row_bytes >= 0, "fa_scatter_rows: negative size");
+  FA_REQUIRE(n_dst_rows < ((int64_t)1 << 31) && n_indices < ((int64_t)1 << 31), "fa_scatter_rows: more than 2^31 rows");
+  FA_REQUIRE(src_row_stride >= row_bytes && dst_row_stride >= row_bytes, "fa_scatter_rows: row stride smaller than row");
+  if (n_dst_rows == 0 || row_bytes == 0) return FA_OK;
+  FA_REQUIRE(dst && (n_indices == 0 || (src && indices)), "fa_scatter_rows: null pointer");
+  if (!workspace || workspace_bytes < fa_scatter_rows_workspace_bytes(n_dst_rows) ||
+      (reinterpret_cast<uintptr_t>(workspace) & 3))
+    return fail(FA_ERR_WORKSPACE, "fa_scatter_rows: needs %zu bytes of 4-byte aligned workspace",
+                fa_scatter_rows_workspace_bytes(n_dst_rows));
+  const int vec = row_vector_bytes(n_indices ? src : dst, dst, row_bytes, src_row_stride, dst_row_stride);
+  FA_LAUNCH(fa::launch_scatter_rows(src, dst, indices, n_indices, n_dst_rows, row_bytes, src_row_stride, dst_row_stride,
+                                    vec, reinterpret_cast<int32_t*>(workspace), reinterpret_cast<hipStream_t>(stream)));
+  return FA_OK;
+}
+
 const char* fa_last_error(void) { return g_err; }
 int fa_abi_version(void) { return FA_ABI_VERSION; }
 

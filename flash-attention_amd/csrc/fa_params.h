@@ -139,6 +139,11 @@ inline int tile_grid(bool tile_major, int tiles_per_bh, int BH) {
 // Launchers (defined in fa_fwd.hip / fa_bwd.hip / fa_aux.hip).  Return hipError_t of the launch.
 hipError_t launch_fwd(const FwdParams& p, int dtype, int head_dim, bool causal, bool dropout, bool sparse,
                       hipStream_t stream);
+hipError_t launch_gather_rows(const void* src, void* dst, const int64_t* idx, int64_t n_idx, int64_t n_src,
+                              int64_t row_bytes, int64_t src_stride, int64_t dst_stride, int vec, hipStream_t stream);
+hipError_t launch_scatter_rows(const void* src, void* dst, const int64_t* idx, int64_t n_idx, int64_t n_dst,
+                               int64_t row_bytes, int64_t src_stride, int64_t dst_stride, int vec, int32_t* inv,
+                               hipStream_t stream);
 hipError_t launch_dump_probs(const DumpParams& p, int dtype, hipStream_t stream);
 // which: 0 = dQ kernel, 1 = dK/dV kernel
 hipError_t launch_bwd(const BwdParams& p, int which, int dtype, int head_dim, bool causal, bool dropout, bool sparse,

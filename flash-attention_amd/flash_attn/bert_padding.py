@@ -2,9 +2,29 @@
 Same names and semantics as the reference's flash_attn/bert_padding.py (:9-95): `unpad_input` gathers the valid
 tokens of a (batch, seqlen, ...) tensor into (total, ...) rows and returns the cumulative sequence lengths;
 `pad_input` scatters rows back into a zero-filled padded tensor.  Both are differentiable.
+
+For GPU tensors the row gather / scatter run as HIP kernels of the attention library (fa_gather_rows /
+fa_scatter_rows; the scatter writes the padded tensor in one pass, without a zero fill); host tensors use the
+equivalent torch indexing, which is what the reference does on every device.
 """
 import torch
 import torch.nn.functional as F
+
+from . import flash_attn_gfx950 as _backend
+
+
+def _gather(input, indices):
+    if input.is_cuda:
+        return _backend.gather_rows(input, indices)
+    return input.index_select(0, indices)
+
+
+def _scatter(values, indices, first_axis_dim):
+    if values.is_cuda:
+        return _backend.scatter_rows(values, indices, first_axis_dim)
+    out = values.new_zeros((first_axis_dim,) + tuple(values.shape[1:]))
+    out.index_copy_(0, indices, values)
+    return out
 
 
 class IndexFirstAxis(torch.autograd.Function):
@@ -15,14 +35,13 @@ class IndexFirstAxis(torch.autograd.Function):
         assert input.ndim == 2
         ctx.save_for_backward(indices)
         ctx.first_axis_dim = input.shape[0]
-        return input.index_select(0, indices)
+        return _gather(input if input.stride(-1) == 1 else input.contiguous(), indices)
 
     @staticmethod
     def backward(ctx, grad_output):
         (indices,) = ctx.saved_tensors
-        grad_input = grad_output.new_zeros((ctx.first_axis_dim,) + tuple(grad_output.shape[1:]))
-        grad_input.index_copy_(0, indices, grad_output)
-        return grad_input, None
+        return _scatter(grad_output if grad_output.stride(-1) == 1 else grad_output.contiguous(), indices,
+                        ctx.first_axis_dim), None
 
 
 index_first_axis = IndexFirstAxis.apply
@@ -36,14 +55,12 @@ class IndexPutFirstAxis(torch.autograd.Function):
         assert indices.ndim == 1
         assert values.ndim == 2
         ctx.save_for_backward(indices)
-        output = values.new_zeros((first_axis_dim, values.shape[1]))
-        output.index_copy_(0, indices, values)
-        return output
+        return _scatter(values if values.stride(-1) == 1 else values.contiguous(), indices, first_axis_dim)
 
     @staticmethod
     def backward(ctx, grad_output):
         (indices,) = ctx.saved_tensors
-        return grad_output.index_select(0, indices), None, None
+        return _gather(grad_output if grad_output.stride(-1) == 1 else grad_output.contiguous(), indices), None, None
 
 
 index_put_first_axis = IndexPutFirstAxis.apply

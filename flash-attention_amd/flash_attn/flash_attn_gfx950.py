@@ -78,6 +78,7 @@ class BwdArgs(ctypes.Structure):
 EXPORTED_SYMBOLS = (
     "fa_fwd", "fa_bwd", "fa_fwd_block", "fa_bwd_block", "fa_fwd_workspace_bytes", "fa_bwd_workspace_bytes",
     "fa_round_seqlens", "fa_philox_offset_increment", "fa_last_error", "fa_abi_version",
+    "fa_gather_rows", "fa_scatter_rows", "fa_scatter_rows_workspace_bytes",
 )
 
 _lib = None
@@ -117,6 +118,13 @@ def load_library():
         lib.fa_last_error.restype = ctypes.c_char_p
         lib.fa_abi_version.argtypes = []
         lib.fa_abi_version.restype = ctypes.c_int
+        lib.fa_gather_rows.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int64] * 5 + [ctypes.c_void_p]
+        lib.fa_gather_rows.restype = ctypes.c_int
+        lib.fa_scatter_rows.argtypes = ([ctypes.c_void_p] * 3 + [ctypes.c_int64] * 5 +
+                                        [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p])
+        lib.fa_scatter_rows.restype = ctypes.c_int
+        lib.fa_scatter_rows_workspace_bytes.argtypes = [ctypes.c_int64]
+        lib.fa_scatter_rows_workspace_bytes.restype = ctypes.c_size_t
         if lib.fa_abi_version() != FA_ABI_VERSION:
             raise RuntimeError("%s has ABI version %d, binding expects %d" % (LIB_NAME, lib.fa_abi_version(), FA_ABI_VERSION))
         _lib = lib
@@ -340,3 +348,56 @@ def bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seql
     _check(blockmask is not None, "blockmask is required")
     return _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q,
                      max_seqlen_k, p_dropout, softmax_scale, False, is_causal, gen)
+
+
+def _check_rows(name, t):
+    _check(t.is_cuda, "%s must be on the GPU" % name)
+    _check(t.ndim == 2 and (t.shape[1] == 0 or t.stride(1) == 1), "%s must be 2-D with a contiguous last dimension" % name)
+
+
+def _index_i64(indices, device):
+    _check(indices.ndim == 1 and indices.device == device, "indices must be 1-D and on the same device")
+    _check(indices.dtype in (torch.int64, torch.int32), "indices must be int64 or int32")
+    return indices.to(torch.int64).contiguous()
+
+
+def gather_rows(input, indices):
+    """input[indices] for a 2-D GPU tensor: the gather of IndexFirstAxis.forward / IndexPutFirstAxis.backward
+    (flash_attn/bert_padding.py:12-19, 51-57), done by fa_gather_rows."""
+    _check_rows("input", input)
+    if input.stride(0) < input.shape[1]:  # broadcast rows
+        input = input.contiguous()
+    idx = _index_i64(indices, input.device)
+    lib = load_library()
+    out = torch.empty((idx.numel(), input.shape[1]), dtype=input.dtype, device=input.device)
+    es = input.element_size()
+    with torch.cuda.device(input.device):
+        rc = lib.fa_gather_rows(input.data_ptr(), out.data_ptr(), idx.data_ptr(), idx.numel(), input.shape[0],
+                                input.shape[1] * es, input.stride(0) * es, out.stride(0) * es,
+                                _stream_handle(input.device))
+    if rc != 0:
+        _raise(rc, lib)
+    return out
+
+
+def scatter_rows(values, indices, first_axis_dim):
+    """zeros(first_axis_dim, dim) with rows `indices` set to `values`: the scatter of IndexPutFirstAxis.forward /
+    IndexFirstAxis.backward (flash_attn/bert_padding.py:21-30, 38-48), done in one pass by fa_scatter_rows (the output is
+    not zero-filled first).  `indices` must be unique."""
+    _check_rows("values", values)
+    if values.stride(0) < values.shape[1]:
+        values = values.contiguous()
+    idx = _index_i64(indices, values.device)
+    _check(idx.numel() == values.shape[0], "one index per row of values")
+    lib = load_library()
+    out = torch.empty((first_axis_dim, values.shape[1]), dtype=values.dtype, device=values.device)
+    ws_bytes = lib.fa_scatter_rows_workspace_bytes(first_axis_dim)
+    ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.int32, device=values.device)
+    es = values.element_size()
+    with torch.cuda.device(values.device):
+        rc = lib.fa_scatter_rows(values.data_ptr(), out.data_ptr(), idx.data_ptr(), idx.numel(), first_axis_dim,
+                                 values.shape[1] * es, values.stride(0) * es, out.stride(0) * es,
+                                 ws.data_ptr(), ws_bytes, _stream_handle(values.device))
+    if rc != 0:
+        _raise(rc, lib)
+    return out

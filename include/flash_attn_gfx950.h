@@ -112,7 +112,7 @@ typedef struct fa_bwd_args {
   size_t workspace_bytes;
   void* stream;
   /* Optional profiling hooks (hipEvent_t or NULL): recorded on `stream` immediately before and after the dK/dV
-   * kernel, the longest of the three kernels of a backward call (rowsum(dO o O) pre-pass, dQ kernel, dK/dV kernel). */
+   * kernel, the longer of the two kernels of a backward call (dQ + softmax_d kernel, dK/dV kernel). */
   void* ev_main_start;
   void* ev_main_stop;
 } fa_bwd_args;
@@ -141,6 +141,24 @@ void fa_round_seqlens(int32_t head_dim, int32_t max_seqlen_q, int32_t max_seqlen
 /* Number of 64-bit Philox offsets one forward call consumes; the caller advances its generator
  * by this much (the role of launch_params.elts_per_thread, fmha_api.cpp:282-292). */
 uint64_t fa_philox_offset_increment(void);
+
+/* Row gather / scatter: the device side of unpad_input / pad_input (flash_attn/bert_padding.py:9-95, where they
+ * are torch.gather and index assignment inside IndexFirstAxis / IndexPutFirstAxis).  Rows are `row_bytes` wide,
+ * `*_row_stride` bytes apart; `indices` is a device array of int64 (what torch.nonzero returns).
+ *
+ * fa_gather_rows:  dst[i, :] = src[indices[i], :]  for i < n_indices      (IndexFirstAxis.forward :12-19,
+ *                  IndexPutFirstAxis.backward :51-57).  An index outside [0, n_src_rows) gives a zero row.
+ * fa_scatter_rows: dst[indices[i], :] = src[i, :], every other row of dst[0 .. n_dst_rows) = 0
+ *                  (IndexPutFirstAxis.forward :38-48, IndexFirstAxis.backward :21-30).  dst is written exactly once
+ *                  and needs no prior zero fill; indices must be unique (duplicates: one of the rows wins); indices
+ *                  outside [0, n_dst_rows) are ignored.  `workspace`: fa_scatter_rows_workspace_bytes(n_dst_rows)
+ *                  bytes of device scratch (the inverse index). */
+int fa_gather_rows(const void* src, void* dst, const int64_t* indices, int64_t n_indices, int64_t n_src_rows,
+                   int64_t row_bytes, int64_t src_row_stride, int64_t dst_row_stride, void* stream);
+int fa_scatter_rows(const void* src, void* dst, const int64_t* indices, int64_t n_indices, int64_t n_dst_rows,
+                    int64_t row_bytes, int64_t src_row_stride, int64_t dst_row_stride, void* workspace,
+                    size_t workspace_bytes, void* stream);
+size_t fa_scatter_rows_workspace_bytes(int64_t n_dst_rows);
 
 /* Message for the last non-zero status returned on the calling thread. */
 const char* fa_last_error(void);

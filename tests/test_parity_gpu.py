@@ -141,6 +141,7 @@ def test_parity_head_dims(D, dtype, causal):
     ([128, 129, 127], [128, 129, 127]),
     ([64, 200], [300, 65]),          # seqlen_q != seqlen_k
     ([257], [513]),
+    ([5, 0, 9], [5, 0, 9]),          # an empty sequence in the batch
 ])
 @pytest.mark.parametrize("causal", [False, True])
 def test_parity_ragged_shapes(lens_q, lens_k, causal):
@@ -530,3 +531,91 @@ def test_size_independent_properties_at_full_size():
         sl = slice(offs[b], offs[b + 1])
         assert (oz[sl].float() - v[sl].float().mean(0, keepdim=True)).abs().max() < 2e-3
         assert (lse[b, :, :lens[b]] - math.log(lens[b])).abs().max() < 1e-4
+
+
+# ------------------------------------------------------------------------------------------------
+# unpad / pad: byte movement, compared bit for bit with the oracle (bert_padding.py:9-95)
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,dim", [(torch.float16, 768), (torch.bfloat16, 40), (torch.float32, 5), (torch.float16, 3),
+                                       (torch.float16, 1024)])
+def test_unpad_pad_rows_bit_exact(dtype, dim):
+    """unpad_input / pad_input on the GPU run fa_gather_rows / fa_scatter_rows; rows of 6 .. 2048 bytes exercise every
+    chunk width.  Forward results and both backward directions equal the oracle's index arithmetic exactly."""
+    from flash_attn.bert_padding import pad_input, unpad_input
+    g = torch.Generator().manual_seed(dim)
+    B, S = 5, 37
+    lens = [37, 0, 1, 20, 36]
+    mask = torch.zeros(B, S, dtype=torch.bool)
+    for b, L in enumerate(lens):
+        mask[b, :L] = True
+    mask[3, 5] = False  # a hole in the middle: indices need not be a prefix per row
+    x = torch.randn(B, S, dim, generator=g).to(dtype)
+    xg = x.cuda().requires_grad_(True)
+    rows, idx, cu, mx = unpad_input(xg, mask.cuda())
+    r_rows, r_idx, r_cu, r_mx = orc.unpad_ref(x.view(torch.int16 if x.element_size() == 2 else torch.int32).numpy(), mask.numpy())
+    as_int = lambda t: t.detach().cpu().view(torch.int16 if t.element_size() == 2 else torch.int32).numpy()
+    assert np.array_equal(as_int(rows), r_rows)
+    assert np.array_equal(idx.cpu().numpy(), r_idx) and np.array_equal(cu.cpu().numpy(), r_cu) and mx == r_mx
+    # backward of the gather = scatter into zeros
+    gr = torch.randn(rows.shape, generator=g).to(dtype)
+    rows.backward(gr.cuda())
+    assert np.array_equal(as_int(xg.grad), orc.pad_ref(as_int(gr), r_idx, B, S).reshape(B, S, dim))
+    # pad_input and its backward (a gather)
+    vg = gr.cuda().requires_grad_(True)
+    padded = pad_input(vg, idx, B, S)
+    assert np.array_equal(as_int(padded), orc.pad_ref(as_int(gr), r_idx, B, S))
+    gp = torch.randn(B, S, dim, generator=g).to(dtype)
+    padded.backward(gp.cuda())
+    assert np.array_equal(as_int(vg.grad), as_int(gp).reshape(B * S, dim)[r_idx])
+
+
+def test_rows_raw_c_abi_unsorted_strided_and_errors():
+    """fa_gather_rows / fa_scatter_rows called directly: unsorted unique indices, strided rows, out-of-range indices,
+    empty inputs, missing workspace."""
+    import ctypes
+    from flash_attn import flash_attn_gfx950 as be
+    lib = be.load_library()
+    g = torch.Generator().manual_seed(3)
+    n_src, dim = 50, 24
+    base = torch.randn(n_src, 2 * dim, generator=g).half().cuda()
+    src = base[:, :dim]                                  # row stride 96 bytes, row width 48 bytes
+    perm = torch.randperm(n_src, generator=g)[:31]
+    idx = perm.clone()
+    idx[4] = n_src + 7                                   # out of range: zero row
+    idx[9] = -1
+    idx_d = idx.cuda()
+    dst = torch.full((31, dim), 7.0, dtype=torch.float16, device="cuda")
+    rc = lib.fa_gather_rows(src.data_ptr(), dst.data_ptr(), idx_d.data_ptr(), 31, n_src, dim * 2, src.stride(0) * 2,
+                            dim * 2, None)
+    assert rc == 0, lib.fa_last_error()
+    want = src.cpu()[perm]
+    want[4] = 0
+    want[9] = 0
+    assert torch.equal(dst.cpu(), want)
+    # scatter with unsorted indices into a strided destination; rows that receive nothing become zero
+    n_dst = 64
+    out_base = torch.full((n_dst, 2 * dim), 5.0, dtype=torch.float16, device="cuda")
+    out = out_base[:, dim:]
+    ws = torch.empty(n_dst, dtype=torch.int32, device="cuda")
+    vals = torch.randn(31, dim, generator=g).half().cuda()
+    sidx = torch.randperm(n_dst, generator=g)[:31]
+    sidx_bad = sidx.clone()
+    sidx_bad[0] = n_dst                                   # ignored
+    rc = lib.fa_scatter_rows(vals.data_ptr(), out.data_ptr(), sidx_bad.cuda().data_ptr(), 31, n_dst, dim * 2, dim * 2,
+                             out.stride(0) * 2, ws.data_ptr(), n_dst * 4, None)
+    assert rc == 0, lib.fa_last_error()
+    torch.cuda.synchronize()
+    want = torch.zeros(n_dst, dim, dtype=torch.float16)
+    want[sidx[1:]] = vals.cpu()[1:]
+    assert torch.equal(out.cpu(), want)
+    assert torch.equal(out_base[:, :dim].cpu(), torch.full((n_dst, dim), 5.0, dtype=torch.float16))  # neighbours untouched
+    # empty and error cases
+    assert lib.fa_gather_rows(None, None, None, 0, 0, 16, 16, 16, None) == 0
+    assert lib.fa_scatter_rows(None, out.data_ptr(), None, 0, n_dst, dim * 2, dim * 2, out.stride(0) * 2, ws.data_ptr(),
+                               n_dst * 4, None) == 0
+    torch.cuda.synchronize()
+    assert not out.cpu().any()
+    assert lib.fa_scatter_rows(vals.data_ptr(), out.data_ptr(), sidx.cuda().data_ptr(), 31, n_dst, dim * 2, dim * 2,
+                               out.stride(0) * 2, None, 0, None) == -2
+    assert b"workspace" in lib.fa_last_error()
+    assert lib.fa_gather_rows(src.data_ptr(), dst.data_ptr(), idx_d.data_ptr(), 31, n_src, dim * 2, 8, dim * 2, None) == -1
