@@ -248,3 +248,30 @@ def test_rotary_is_a_rotation_by_position_times_frequency():
     rows, _ = RotaryEmbedding(4)(grid[..., 4:].transpose(2, 3), grid[..., 4:].transpose(2, 3), seq_dimension=-2)
     want = torch.cat([cols, rows.transpose(2, 3)], dim=-1).reshape(1, 2, side * side, 8)
     assert torch.allclose(r2, want, atol=1e-12)
+
+
+def test_blocksparse_module_layout_handling_on_host():
+    """FlashBlocksparseAttention keeps the layout and its converted form as buffers (flash_blocksparse_attention.py:31-36)
+    and accepts a tensor, a make_layout() object or, only with hydra installed, a _target_ mapping."""
+    import importlib.util
+    from flash_attn.flash_blocksparse_attention import FlashBlocksparseAttention
+    layout = (torch.arange(48 * 3).reshape(48, 3) % 4 != 1).to(torch.int32)
+
+    class Cfg:
+        def make_layout(self, seqlen):
+            assert seqlen == 768  # 700 rounded up to a multiple of 256
+            return layout
+
+    m = FlashBlocksparseAttention(Cfg(), max_seq_length=700)
+    assert set(dict(m.named_buffers())) == {"layout", "blockmask_converted"}
+    assert torch.equal(m.blockmask_converted, torch.tensor(orc.convert_blockmask_ref(layout.numpy())))
+    assert tuple(m._blockmask(300).shape) == (19, 2) and tuple(m._blockmask(768).shape) == (48, 3)
+    with pytest.raises(AssertionError):
+        m._blockmask(769)
+    with pytest.raises(ValueError):
+        FlashBlocksparseAttention(layout[:10], max_seq_length=700)
+    with pytest.raises(TypeError):
+        FlashBlocksparseAttention("not a layout")
+    if importlib.util.find_spec("hydra") is None:
+        with pytest.raises(RuntimeError, match="hydra"):
+            FlashBlocksparseAttention({"_target_": "some.module.Config"})

@@ -619,3 +619,63 @@ def test_rows_raw_c_abi_unsorted_strided_and_errors():
                                out.stride(0) * 2, None, 0, None) == -2
     assert b"workspace" in lib.fa_last_error()
     assert lib.fa_gather_rows(src.data_ptr(), dst.data_ptr(), idx_d.data_ptr(), 31, n_src, dim * 2, 8, dim * 2, None) == -1
+
+
+def test_blocksparse_modules_layout_sources_and_padding():
+    """FlashBlocksparseAttention / FlashBlocksparseMHA (flash_blocksparse_attention.py:14-136) built from a layout
+    tensor and from an object with make_layout(); padded, packed and key_padding_mask inputs agree with the oracle on
+    the expanded layout."""
+    from flash_attn.flash_blocksparse_attention import FlashBlocksparseAttention, FlashBlocksparseMHA
+    torch.manual_seed(0)
+    S, H, D, B = 512, 2, 64, 2
+    g = torch.Generator().manual_seed(1)
+    layout = (torch.rand(S // 16, S // 256, generator=g) < 0.5).to(torch.int32)
+    layout[:, 0] |= (torch.arange(S // 16) % 3 != 0).to(torch.int32)
+
+    class Cfg:
+        def make_layout(self, seqlen):
+            assert seqlen == S
+            return layout
+
+    m_t = FlashBlocksparseAttention(layout, max_seq_length=S).cuda().eval()
+    m_o = FlashBlocksparseAttention(Cfg(), max_seq_length=S - 100).cuda().eval()   # rounded up to 512
+    assert torch.equal(m_t.layout.cpu(), layout) and torch.equal(m_o.blockmask_converted, m_t.blockmask_converted)
+    qkv = torch.randn(B, S, 3, H, D, generator=g).half()
+    out, w = m_t(qkv.cuda())
+    assert w is None
+    sc = D ** -0.5
+    for b in range(B):
+        ref = orc.varlen_attention(qkv[b, :, 0], qkv[b, :, 1], qkv[b, :, 2], _cu([S], "cpu"), _cu([S], "cpu"), sc, False,
+                                   layout=layout.numpy())
+        assert (out[b].float().cpu() - ref["out"]).abs().max() < 2e-3
+    # packed input with and without mask conversion
+    cu = _cu([S] * B, "cuda")
+    packed = qkv.reshape(B * S, 3, H, D).cuda()
+    o1, _ = m_o(packed, cu_seqlens=cu, max_s=S)
+    o2, _ = m_o(packed, cu_seqlens=cu, max_s=S, convert_mask=False)
+    assert torch.equal(o1, out.reshape(B * S, H, D)) and torch.equal(o2, o1)
+    # key padding mask (tensor and .bool_matrix object): shorter sequences use the corner of the layout
+    lens = [300, 512]
+    keep = torch.zeros(B, S, dtype=torch.bool)
+    for b, L in enumerate(lens):
+        keep[b, :L] = True
+
+    class Mask:
+        bool_matrix = keep.cuda()
+
+    o3, _ = m_t(qkv.cuda(), key_padding_mask=keep.cuda())
+    o4, _ = m_t(qkv.cuda(), key_padding_mask=Mask())
+    assert torch.equal(o3, o4)
+    for b, L in enumerate(lens):
+        ref = orc.varlen_attention(qkv[b, :L, 0], qkv[b, :L, 1], qkv[b, :L, 2], _cu([L], "cpu"), _cu([L], "cpu"), sc, False,
+                                   layout=layout[:(L + 15) // 16, :(L + 255) // 256].numpy())
+        assert (o3[b, :L].float().cpu() - ref["out"]).abs().max() < 2e-3
+        assert not o3[b, L:].any()
+    # MHA block: gradient flows to the projections
+    mha = FlashBlocksparseMHA(H * D, H, layout, max_seq_length=S, device="cuda", dtype=torch.float16)
+    x = torch.randn(B, S, H * D, device="cuda", dtype=torch.float16, requires_grad=True)
+    y, _ = mha(x, None, None)
+    y.float().pow(2).mean().backward()
+    assert y.shape == x.shape and torch.isfinite(x.grad).all() and mha.Wqkv.weight.grad.abs().sum() > 0
+    with pytest.raises(TypeError):
+        FlashBlocksparseAttention(object())
