@@ -234,6 +234,26 @@ def main():
             print("%-28s %9.4f ms  %8.1f GB/s of %d (%.1f %% of HBM peak)  [B=%d S=%d dim=%d fp16, %d of %d tokens valid]"
                   % (name, ms, nbytes / ms / 1e6, HBM_PEAK_GBS, 100 * nbytes / ms / 1e6 / HBM_PEAK_GBS, Bp, Sp, dim, nnz, Bp * Sp),
                   file=sys.stderr)
+        # rotary embedding of q and k of a packed qkv, in place (HBM-bound: 2/3 of the tensor read and written)
+        Br, Sr, Hr, Dr = 8, 2048, 12, 64
+        qkv_r = torch.randn(Br, Sr, 3, Hr, Dr, device="cuda", dtype=torch.float16)
+        ang = torch.outer(torch.arange(Sr, device="cuda", dtype=torch.float32),
+                          1.0 / (10000 ** (torch.arange(0, Dr, 2, device="cuda").float() / Dr)))
+        cos_h, sin_h = torch.cos(ang).half().contiguous(), torch.sin(ang).half().contiguous()
+        for _ in range(20):
+            be.rotary(qkv_r, qkv_r, cos_h, sin_h, n_rotated=2)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(50):
+            be.rotary(qkv_r, qkv_r, cos_h, sin_h, n_rotated=2)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / 50
+        nbytes = 2 * 2 * Br * Sr * Hr * Dr * 2   # q and k read and written; v is not touched in place
+        print("%-28s %9.4f ms  %8.1f GB/s of %d (%.1f %% of HBM peak)  [B=%d S=%d H=%d d=%d fp16 packed qkv, in place]"
+              % ("rotary q,k (fa_rotary)", ms, nbytes / ms / 1e6, HBM_PEAK_GBS, 100 * nbytes / ms / 1e6 / HBM_PEAK_GBS,
+                 Br, Sr, Hr, Dr), file=sys.stderr)
     print(json.dumps(res))
 
 

@@ -334,6 +334,32 @@ int fa_scatter_rows(const void* src, void* dst, const int64_t* indices, int64_t 
   return FA_OK;
 }
 
+int fa_rotary(const fa_rotary_args* a) {
+  FA_REQUIRE(a && a->struct_bytes == sizeof(fa_rotary_args), "fa_rotary: struct size mismatch");
+  FA_REQUIRE(a->dtype == FA_FP16 || a->dtype == FA_BF16, "fa_rotary: dtype must be fp16 or bf16");
+  FA_REQUIRE(a->n_rows >= 0 && a->n_parts >= 1 && a->n_rotated >= 0 && a->n_rotated <= a->n_parts && a->n_heads >= 1,
+             "fa_rotary: bad sizes");
+  FA_REQUIRE(a->head_dim >= 8 && a->head_dim % 8 == 0, "fa_rotary: head_dim must be a multiple of 8");
+  if (a->n_rows == 0) return FA_OK;
+  FA_REQUIRE(a->src && a->dst && a->cos_table && a->sin_table, "fa_rotary: null pointer");
+  FA_REQUIRE(a->table_rows >= 1 && (a->positions || a->seqlen >= 1), "fa_rotary: empty table or no positions");
+  FA_REQUIRE(aligned16(a->src) && aligned16(a->dst) && (reinterpret_cast<uintptr_t>(a->cos_table) & 7) == 0 &&
+                 (reinterpret_cast<uintptr_t>(a->sin_table) & 7) == 0,
+             "fa_rotary: pointers must be 16-byte (tensors) / 8-byte (tables) aligned");
+  FA_REQUIRE(stride_ok(a->src_row_stride) && stride_ok(a->src_part_stride) && stride_ok(a->src_head_stride) &&
+                 stride_ok(a->dst_row_stride) && stride_ok(a->dst_part_stride) && stride_ok(a->dst_head_stride),
+             "fa_rotary: strides must be multiples of 8 elements");
+  fa::RotaryParams p;
+  p.src = a->src; p.dst = a->dst; p.cos = a->cos_table; p.sin = a->sin_table; p.positions = a->positions;
+  p.n_rows = a->n_rows;
+  p.src_row_stride = a->src_row_stride; p.src_part_stride = a->src_part_stride; p.src_head_stride = a->src_head_stride;
+  p.dst_row_stride = a->dst_row_stride; p.dst_part_stride = a->dst_part_stride; p.dst_head_stride = a->dst_head_stride;
+  p.n_parts = a->n_parts; p.n_rotated = a->n_rotated; p.n_heads = a->n_heads; p.head_dim = a->head_dim;
+  p.seqlen = a->seqlen; p.table_rows = a->table_rows; p.conjugate = a->conjugate;
+  FA_LAUNCH(fa::launch_rotary(p, a->dtype, reinterpret_cast<hipStream_t>(a->stream)));
+  return FA_OK;
+}
+
 const char* fa_last_error(void) { return g_err; }
 int fa_abi_version(void) { return FA_ABI_VERSION; }
 

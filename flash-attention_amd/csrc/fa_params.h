@@ -139,6 +139,19 @@ inline int tile_grid(bool tile_major, int tiles_per_bh, int BH) {
 // Launchers (defined in fa_fwd.hip / fa_bwd.hip / fa_aux.hip).  Return hipError_t of the launch.
 hipError_t launch_fwd(const FwdParams& p, int dtype, int head_dim, bool causal, bool dropout, bool sparse,
                       hipStream_t stream);
+// fa_rotary: rotate the first n_rotated of n_parts (row, part, head, head_dim) slices, copy the others
+struct RotaryParams {
+  const void* src;
+  void* dst;
+  const void* cos;          // [table_rows, head_dim / 2], tensor dtype
+  const void* sin;
+  const int32_t* positions; // [n_rows] or null: position = row % seqlen
+  int64_t n_rows;
+  int64_t src_row_stride, src_part_stride, src_head_stride;  // elements
+  int64_t dst_row_stride, dst_part_stride, dst_head_stride;
+  int n_parts, n_rotated, n_heads, head_dim, seqlen, table_rows, conjugate;
+};
+hipError_t launch_rotary(const RotaryParams& p, int dtype, hipStream_t stream);
 hipError_t launch_gather_rows(const void* src, void* dst, const int64_t* idx, int64_t n_idx, int64_t n_src,
                               int64_t row_bytes, int64_t src_stride, int64_t dst_stride, int vec, hipStream_t stream);
 hipError_t launch_scatter_rows(const void* src, void* dst, const int64_t* idx, int64_t n_idx, int64_t n_dst,

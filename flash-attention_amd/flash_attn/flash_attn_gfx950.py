@@ -75,10 +75,24 @@ class BwdArgs(ctypes.Structure):
     ]
 
 
+class RotaryArgs(ctypes.Structure):
+    """struct fa_rotary_args, field for field."""
+    _fields_ = [
+        ("struct_bytes", ctypes.c_uint32), ("dtype", ctypes.c_int32),
+        ("src", ctypes.c_void_p), ("dst", ctypes.c_void_p), ("cos_table", ctypes.c_void_p), ("sin_table", ctypes.c_void_p),
+        ("positions", ctypes.c_void_p), ("n_rows", ctypes.c_int64),
+        ("src_row_stride", ctypes.c_int64), ("src_part_stride", ctypes.c_int64), ("src_head_stride", ctypes.c_int64),
+        ("dst_row_stride", ctypes.c_int64), ("dst_part_stride", ctypes.c_int64), ("dst_head_stride", ctypes.c_int64),
+        ("n_parts", ctypes.c_int32), ("n_rotated", ctypes.c_int32), ("n_heads", ctypes.c_int32), ("head_dim", ctypes.c_int32),
+        ("seqlen", ctypes.c_int32), ("table_rows", ctypes.c_int32), ("conjugate", ctypes.c_int32),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
 EXPORTED_SYMBOLS = (
     "fa_fwd", "fa_bwd", "fa_fwd_block", "fa_bwd_block", "fa_fwd_workspace_bytes", "fa_bwd_workspace_bytes",
     "fa_round_seqlens", "fa_philox_offset_increment", "fa_last_error", "fa_abi_version",
-    "fa_gather_rows", "fa_scatter_rows", "fa_scatter_rows_workspace_bytes",
+    "fa_gather_rows", "fa_scatter_rows", "fa_scatter_rows_workspace_bytes", "fa_rotary",
 )
 
 _lib = None
@@ -125,6 +139,8 @@ def load_library():
         lib.fa_scatter_rows.restype = ctypes.c_int
         lib.fa_scatter_rows_workspace_bytes.argtypes = [ctypes.c_int64]
         lib.fa_scatter_rows_workspace_bytes.restype = ctypes.c_size_t
+        lib.fa_rotary.argtypes = [ctypes.POINTER(RotaryArgs)]
+        lib.fa_rotary.restype = ctypes.c_int
         if lib.fa_abi_version() != FA_ABI_VERSION:
             raise RuntimeError("%s has ABI version %d, binding expects %d" % (LIB_NAME, lib.fa_abi_version(), FA_ABI_VERSION))
         _lib = lib
@@ -401,3 +417,41 @@ def scatter_rows(values, indices, first_axis_dim):
     if rc != 0:
         _raise(rc, lib)
     return out
+
+
+def rotary(src, dst, cos, sin, n_rotated, conjugate=False, positions=None):
+    """Rotary embedding of the first `n_rotated` parts of src (batch, seqlen, parts, nheads, headdim) into dst (same
+    shape; may be src), remaining parts copied: the arithmetic of apply_rotary_pos_emb (flash_attn/rotary.py:32-42) for
+    q and k of a packed qkv in one pass (fa_rotary).  cos, sin: (>= seqlen, headdim / 2) tables in src's dtype.
+    positions: optional int32 (batch * seqlen,) table rows to use instead of the position inside the sequence."""
+    _check(src.is_cuda and dst.is_cuda and src.ndim == 5 and src.shape == dst.shape and src.dtype == dst.dtype,
+           "src and dst must be GPU tensors of the same (batch, seqlen, parts, nheads, headdim) shape and dtype")
+    B, S, P, H, D = src.shape
+    for t, name in ((src, "src"), (dst, "dst")):
+        _check(t.stride(4) == 1 and (B <= 1 or t.stride(0) == S * t.stride(1)), "%s rows must be evenly strided" % name)
+    _check(cos.shape == sin.shape and cos.ndim == 2 and cos.shape[1] == D // 2 and cos.dtype == src.dtype
+           and cos.is_contiguous() and sin.is_contiguous() and cos.device == src.device,
+           "cos / sin must be contiguous (rows, headdim / 2) tables in the tensor's dtype")
+    if positions is not None:
+        _check(positions.dtype == torch.int32 and positions.numel() == B * S and positions.is_contiguous()
+               and positions.device == src.device, "positions must be a contiguous int32 tensor with one entry per row")
+    else:
+        _check(cos.shape[0] >= S, "the tables have fewer rows than the sequence has positions")
+    lib = load_library()
+    a = RotaryArgs()
+    a.struct_bytes = ctypes.sizeof(a)
+    a.dtype = _dtype_code(src)
+    a.src, a.dst, a.cos_table, a.sin_table = src.data_ptr(), dst.data_ptr(), cos.data_ptr(), sin.data_ptr()
+    a.positions = positions.data_ptr() if positions is not None else None
+    a.n_rows = B * S
+    a.src_row_stride, a.src_part_stride, a.src_head_stride = src.stride(1), src.stride(2), src.stride(3)
+    a.dst_row_stride, a.dst_part_stride, a.dst_head_stride = dst.stride(1), dst.stride(2), dst.stride(3)
+    in_place = src.data_ptr() == dst.data_ptr() and src.stride() == dst.stride()
+    a.n_parts, a.n_rotated, a.n_heads, a.head_dim = (n_rotated if in_place else P), n_rotated, H, D  # in place: no copy
+    a.seqlen, a.table_rows, a.conjugate = S, cos.shape[0], int(bool(conjugate))
+    a.stream = _stream_handle(src.device)
+    with torch.cuda.device(src.device):
+        rc = lib.fa_rotary(ctypes.byref(a))
+    if rc != 0:
+        _raise(rc, lib)
+    return dst

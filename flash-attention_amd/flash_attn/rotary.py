@@ -1,5 +1,7 @@
 """Rotary position embeddings used by FlashMHA(use_rotary_emb=...), interface-compatible with the reference's
-flash_attn/rotary.py (:22-135).  Pure PyTorch pre-processing of q and k ahead of the attention kernels.
+flash_attn/rotary.py (:22-135).  The general functions are PyTorch elementwise ops as in the reference; for the case
+the attention modules use, q and k of a packed (batch, seqlen, 3, nheads, headdim) GPU tensor, `apply_rotary_emb_qkv_`
+rotates both in place in one pass of a HIP kernel (fa_rotary), with a matching backward.
 
 Convention (rotary.py:22-42,66-87): channel pairs are interleaved, (x[2i], x[2i+1]) is rotated by angle
 pos * 10000^(-2i/dim):   x'[2i] = x[2i] cos - x[2i+1] sin,   x'[2i+1] = x[2i+1] cos + x[2i] sin.
@@ -26,6 +28,34 @@ def apply_rotary_pos_emb(x, cos, sin, seq_dimension: int = -2):
     return x * cos + rotate_half(x) * sin
 
 
+class _ApplyRotaryQKV(torch.autograd.Function):
+    """In-place rotation of the q and k parts of a packed qkv; the backward rotates the incoming gradient by the
+    opposite angle (the transpose of a rotation) and passes the v part through."""
+
+    @staticmethod
+    def forward(ctx, qkv, cos_half, sin_half):
+        from . import flash_attn_gfx950 as backend
+        ctx.save_for_backward(cos_half, sin_half)
+        backend.rotary(qkv, qkv, cos_half, sin_half, n_rotated=2)
+        ctx.mark_dirty(qkv)
+        return qkv
+
+    @staticmethod
+    def backward(ctx, grad):
+        from . import flash_attn_gfx950 as backend
+        cos_half, sin_half = ctx.saved_tensors
+        grad = grad.contiguous()
+        return backend.rotary(grad, torch.empty_like(grad), cos_half, sin_half, n_rotated=2, conjugate=True), None, None
+
+
+def apply_rotary_emb_qkv_(qkv, cos_half, sin_half):
+    """Rotates q = qkv[:, :, 0] and k = qkv[:, :, 1] of a packed (batch, seqlen, 3, nheads, headdim) fp16 / bf16 GPU
+    tensor IN PLACE by the angles whose cosines / sines are cos_half / sin_half ((>= seqlen, headdim / 2), same dtype):
+    the same map as apply_rotary_pos_emb(q, ...), apply_rotary_pos_emb(k, ...) with seq_dimension=-3, products formed in
+    fp32 and rounded once.  Differentiable."""
+    return _ApplyRotaryQKV.apply(qkv, cos_half, sin_half)
+
+
 class RotaryEmbedding(torch.nn.Module):
     """Rotary embedding of RoFormer (Su et al., arXiv:2104.09864) for queries and keys."""
 
@@ -48,6 +78,12 @@ class RotaryEmbedding(torch.nn.Module):
             self._cos_cached = torch.cos(angles).to(x.dtype).repeat_interleave(2, dim=-1)
             self._sin_cached = torch.sin(angles).to(x.dtype).repeat_interleave(2, dim=-1)
         return self._cos_cached, self._sin_cached
+
+    def rotate_qkv_(self, qkv):
+        """q and k of a packed (batch, seqlen, 3, nheads, headdim) GPU tensor rotated in place (one HIP kernel); returns
+        qkv.  Same tables as forward()."""
+        cos, sin = self._update_cos_sin_tables(qkv[:, :, 0], seq_dimension=-3)
+        return apply_rotary_emb_qkv_(qkv, cos[:, ::2].contiguous(), sin[:, ::2].contiguous())
 
     def forward(self, q: torch.Tensor, k: torch.Tensor, seq_dimension=-2) -> Tuple[torch.Tensor, torch.Tensor]:
         assert seq_dimension in [-2, -3]  # (bs, h, s, d) or (bs, s, h, d)

@@ -160,6 +160,32 @@ int fa_scatter_rows(const void* src, void* dst, const int64_t* indices, int64_t 
                     size_t workspace_bytes, void* stream);
 size_t fa_scatter_rows_workspace_bytes(int64_t n_dst_rows);
 
+/* Rotary position embedding of the query and key parts of a packed tensor in one pass: what
+ * RotaryEmbedding.forward / apply_rotary_pos_emb compute with elementwise torch ops (flash_attn/rotary.py:22-42,
+ * 89-100; FlashMHA applies it to q and k before attention, flash_attention.py:109-113).
+ * src / dst: [n_rows, n_parts, n_heads, head_dim] views (strides in elements, innermost stride 1; dst may equal
+ * src).  Parts 0 .. n_rotated-1 are rotated, the remaining parts are copied (packed qkv: n_parts 3, n_rotated 2).
+ * Pair (x[2i], x[2i+1]) of a row at position t becomes (x[2i] c - x[2i+1] s, x[2i+1] c + x[2i] s) with
+ * c = cos_table[t, i], s = sin_table[t, i]; tables are [table_rows, head_dim / 2] in the tensor's dtype;
+ * t = positions[row] if positions != NULL, else row % seqlen.  conjugate != 0 negates s (the backward pass).
+ * head_dim must be a multiple of 8; base pointers and strides must keep 16-byte alignment. */
+typedef struct fa_rotary_args {
+  uint32_t struct_bytes;
+  int32_t dtype;
+  const void* src;
+  void* dst;
+  const void* cos_table;
+  const void* sin_table;
+  const int32_t* positions;
+  int64_t n_rows;
+  int64_t src_row_stride, src_part_stride, src_head_stride;
+  int64_t dst_row_stride, dst_part_stride, dst_head_stride;
+  int32_t n_parts, n_rotated, n_heads, head_dim;
+  int32_t seqlen, table_rows, conjugate;
+  void* stream;
+} fa_rotary_args;
+int fa_rotary(const fa_rotary_args* args);
+
 /* Message for the last non-zero status returned on the calling thread. */
 const char* fa_last_error(void);
 int fa_abi_version(void);

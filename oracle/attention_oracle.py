@@ -276,3 +276,23 @@ def pad_ref(rows, idx, B, S):
     out = np.zeros((B * S, rows.shape[-1]), dtype=rows.dtype)
     out[np.asarray(idx)] = rows
     return out.reshape(B, S, -1)
+
+
+# --------------------------------------------------------------------------------------------------
+# Rotary position embedding (flash_attn/rotary.py:22-42,66-87)
+# --------------------------------------------------------------------------------------------------
+def rotary_ref(x, cos_half, sin_half, positions, conjugate=False):
+    """x (rows, nheads, dim) float array; cos_half, sin_half (table_rows, dim / 2); positions (rows,) ints.
+    Pair (x[2i], x[2i+1]) of row r becomes (x[2i] c - x[2i+1] s, x[2i+1] c + x[2i] s), c = cos_half[positions[r], i]:
+    x * cos + rotate_half(x) * sin with rotate_half(x) = (-x1, x0, -x3, x2, ...) and each table entry repeated twice
+    (rotary.py:22-42, 84-85).  Evaluated in float64."""
+    x = np.asarray(x, dtype=np.float64)
+    c = np.asarray(cos_half, dtype=np.float64)[np.asarray(positions)][:, None, :]
+    s = np.asarray(sin_half, dtype=np.float64)[np.asarray(positions)][:, None, :]
+    if conjugate:
+        s = -s
+    a, b = x[..., 0::2], x[..., 1::2]
+    out = np.empty_like(x)
+    out[..., 0::2] = a * c - b * s
+    out[..., 1::2] = b * c + a * s
+    return out

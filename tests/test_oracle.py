@@ -254,3 +254,25 @@ def test_unpad_pad_roundtrip():
     rows, idx, cu, mx = orc.unpad_ref(x, mask)
     assert cu.tolist() == [0, 3, 10, 11] and mx == 7 and rows.shape == (11, 4)
     assert np.array_equal(orc.pad_ref(rows, idx, 3, 7), x * mask[..., None])
+
+
+def test_rotary_ref_is_a_rotation_and_matches_the_elementwise_definition():
+    """rotary_ref against the definition it cites evaluated literally (x * cos + rotate_half(x) * sin with repeated
+    tables), norm preservation of every pair, angle addition (rotating by t1 then t2 = rotating by t1 + t2), and the
+    conjugate being the inverse."""
+    rng = np.random.default_rng(0)
+    rows, H, dim = 7, 2, 8
+    x = rng.standard_normal((rows, H, dim))
+    inv_freq = 1.0 / (10000 ** (np.arange(0, dim, 2) / dim))
+    ang = np.outer(np.arange(20), inv_freq)
+    cos_h, sin_h = np.cos(ang), np.sin(ang)
+    pos = np.array([0, 3, 5, 1, 19, 7, 2])
+    got = orc.rotary_ref(x, cos_h, sin_h, pos)
+    cos_f, sin_f = np.repeat(cos_h, 2, -1)[pos][:, None], np.repeat(sin_h, 2, -1)[pos][:, None]
+    rot_half = np.stack([-x[..., 1::2], x[..., 0::2]], -1).reshape(x.shape)
+    assert np.allclose(got, x * cos_f + rot_half * sin_f, atol=1e-14)
+    assert np.allclose(got[..., 0::2] ** 2 + got[..., 1::2] ** 2, x[..., 0::2] ** 2 + x[..., 1::2] ** 2)
+    assert np.allclose(orc.rotary_ref(got, cos_h, sin_h, pos, conjugate=True), x, atol=1e-14)
+    twice = orc.rotary_ref(orc.rotary_ref(x, cos_h, sin_h, np.full(rows, 4)), cos_h, sin_h, np.full(rows, 9))
+    assert np.allclose(twice, orc.rotary_ref(x, cos_h, sin_h, np.full(rows, 13)), atol=1e-13)
+    assert np.allclose(orc.rotary_ref(x, cos_h, sin_h, np.zeros(rows, dtype=int)), x)

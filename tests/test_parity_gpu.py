@@ -679,3 +679,54 @@ def test_blocksparse_modules_layout_sources_and_padding():
     assert y.shape == x.shape and torch.isfinite(x.grad).all() and mha.Wqkv.weight.grad.abs().sum() > 0
     with pytest.raises(TypeError):
         FlashBlocksparseAttention(object())
+
+
+# ------------------------------------------------------------------------------------------------
+# rotary embedding kernel (fa_rotary) against the oracle; tolerance: one rounding of the result (the reference's
+# elementwise fp16 ops round three times, rotary.py:32-42)
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [16, 64, 128])
+def test_rotary_kernel_matches_oracle(dtype, D):
+    from flash_attn import flash_attn_gfx950 as be
+    from flash_attn.rotary import RotaryEmbedding, apply_rotary_pos_emb, apply_rotary_emb_qkv_
+    g = torch.Generator().manual_seed(D)
+    B, S, H = 3, 50, 2
+    qkv = torch.randn(B, S, 3, H, D, generator=g).to(dtype)
+    emb = RotaryEmbedding(D)
+    cos_full, sin_full = emb._update_cos_sin_tables(qkv[:, :, 0].cuda(), seq_dimension=-3)   # (S, D) in dtype
+    cos_h, sin_h = cos_full[:, ::2].contiguous(), sin_full[:, ::2].contiguous()
+    ulp = 2.0 ** (-10 if dtype == torch.float16 else -7)
+    pos = np.tile(np.arange(S), B)
+
+    def close(got, want64):  # one rounding to the 16-bit type
+        got = got.double().cpu().numpy()
+        assert np.all(np.abs(got - want64) <= ulp * np.abs(want64) * 0.51 + 1e-7), np.abs(got - want64).max()
+
+    out = be.rotary(qkv.cuda(), torch.empty_like(qkv).cuda(), cos_h, sin_h, n_rotated=2)
+    for part in range(2):
+        want = orc.rotary_ref(qkv[:, :, part].reshape(B * S, H, D).double().numpy(), cos_h.double().cpu().numpy(),
+                              sin_h.double().cpu().numpy(), pos)
+        close(out[:, :, part].reshape(B * S, H, D), want)
+    assert torch.equal(out[:, :, 2].cpu(), qkv[:, :, 2])                                   # v copied untouched
+    # the reference's elementwise formulation agrees within its own three roundings
+    q_t = apply_rotary_pos_emb(qkv[:, :, 0].cuda(), cos_full, sin_full, seq_dimension=-3)
+    assert (q_t.float() - out[:, :, 0].float()).abs().max() <= 3 * ulp * qkv.abs().max() * 1.5
+    # explicit positions, conjugate = inverse, in-place autograd wrapper
+    p32 = torch.randint(0, S, (B * S,), generator=g, dtype=torch.int32)
+    outp = be.rotary(qkv.cuda(), torch.empty_like(qkv).cuda(), cos_h, sin_h, n_rotated=1, positions=p32.cuda())
+    close(outp[:, :, 0].reshape(B * S, H, D), orc.rotary_ref(qkv[:, :, 0].reshape(B * S, H, D).double().numpy(),
+                                                            cos_h.double().cpu().numpy(), sin_h.double().cpu().numpy(), p32.numpy()))
+    assert torch.equal(outp[:, :, 1:].cpu(), qkv[:, :, 1:])
+    back = be.rotary(out, torch.empty_like(out), cos_h, sin_h, n_rotated=2, conjugate=True)
+    assert (back.float().cpu() - qkv.float()).abs().max() <= 4 * ulp * qkv.abs().max()
+    x = qkv.cuda().clone().requires_grad_(True)
+    y = apply_rotary_emb_qkv_(x * 1.0, cos_h, sin_h)
+    assert torch.equal(y, out)
+    go = torch.randn(B, S, 3, H, D, generator=g).to(dtype)
+    y.backward(go.cuda())
+    for part in range(2):
+        want = orc.rotary_ref(go[:, :, part].reshape(B * S, H, D).double().numpy(), cos_h.double().cpu().numpy(),
+                              sin_h.double().cpu().numpy(), pos, conjugate=True)
+        close(x.grad[:, :, part].reshape(B * S, H, D), want)
+    assert torch.equal(x.grad[:, :, 2].cpu(), go[:, :, 2])
