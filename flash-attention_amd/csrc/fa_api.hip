@@ -75,6 +75,29 @@ SparseLayout sparse_layout(const Rounded& r) {
   return s;
 }
 
+// Key-split forward: worth it when the query tiles alone cannot fill the chip and there are many key tiles to share.
+// Returns the number of splits (1 = single pass) and the scratch the partial results need.
+struct SplitPlan {
+  int n_splits;
+  size_t o_bytes, bytes;
+};
+SplitPlan split_plan(int batch, int nheads, int head_dim, int total_q, int max_sq, int max_sk, int sq_r, bool causal,
+                     bool sparse) {
+  SplitPlan sp{1, 0, 0};
+  if (causal || sparse || max_sq <= 0 || max_sq > fa::kFwdBM) return sp;  // one query tile per (batch, head) only
+  const int64_t blocks = (int64_t)batch * nheads * ((max_sq + fa::kFwdBM - 1) / fa::kFwdBM);
+  const int key_tiles = (max_sk + 63) / 64;
+  if (blocks >= 128 || key_tiles < 8) return sp;
+  int64_t n = (768 + blocks - 1) / blocks;  // about three workgroups per compute unit
+  if (n > key_tiles / 4) n = key_tiles / 4; // at least four key tiles per split
+  if (n > 64) n = 64;
+  if (n < 2) return sp;
+  sp.n_splits = (int)n;
+  sp.o_bytes = align16((size_t)n * total_q * nheads * head_dim * 4);
+  sp.bytes = sp.o_bytes + align16((size_t)n * batch * nheads * sq_r * 4);
+  return sp;
+}
+
 int build_maps(const int32_t* blockmask, unsigned char* ws, const SparseLayout& sl, fa::SparseMaps* out,
                hipStream_t stream) {
   FA_LAUNCH(fa::launch_fill_f32(reinterpret_cast<float*>(ws), sl.bytes / 4, 0.f, stream));
@@ -166,7 +189,17 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
   p.rp_keep = 1.f / p_keep;
   p.keep_thr = (uint32_t)std::floor(p_keep * 65535.0);  // fmha_api.cpp:110
   p.pk = make_key(a->philox_seed, a->philox_offset);
+  // short query side, long key side: split the keys over several workgroups if the caller brought the scratch for it
+  const SplitPlan sp = split_plan(a->batch, a->nheads, a->head_dim, a->total_q, a->max_seqlen_q, a->max_seqlen_k, r.sq_r,
+                                  a->is_causal != 0, sparse);
+  const bool split = sp.n_splits > 1 && a->workspace && a->workspace_bytes >= sp.bytes && aligned16(a->workspace);
+  if (split) {
+    p.n_splits = sp.n_splits;
+    p.o_part = reinterpret_cast<float*>(a->workspace);
+    p.lse_part = reinterpret_cast<float*>(reinterpret_cast<unsigned char*>(a->workspace) + sp.o_bytes);
+  }
   FA_LAUNCH(fa::launch_fwd(p, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));
+  if (split) FA_LAUNCH(fa::launch_fwd_combine(p, a->dtype, a->head_dim, stream));
 
   if (a->s_dmask) {
     fa::DumpParams d;
@@ -273,8 +306,11 @@ int fa_bwd(const fa_bwd_args* args) { return bwd_impl(args, false); }
 int fa_bwd_block(const fa_bwd_args* args) { return bwd_impl(args, true); }
 
 size_t fa_fwd_workspace_bytes(const fa_fwd_args* a) {
-  if (!a || !a->blockmask) return 0;
-  return sparse_layout(round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, true)).bytes;
+  if (!a) return 0;
+  if (a->blockmask) return sparse_layout(round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, true)).bytes;
+  const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, false);
+  return split_plan(a->batch, a->nheads, a->head_dim, a->total_q, a->max_seqlen_q, a->max_seqlen_k, r.sq_r,
+                    a->is_causal != 0, false).bytes;
 }
 
 size_t fa_bwd_workspace_bytes(const fa_bwd_args* a) {

@@ -1,5 +1,6 @@
 // Forward launcher: picks the head-dimension specialisation (the role of run_fmha_fp16_sm80,
 // csrc/flash_attn/src/fmha_fprop_fp16_kernel.sm80.cu:84-146).
+#include "fa_common.h"
 #include "fa_params.h"
 
 namespace fa {
@@ -20,6 +21,47 @@ hipError_t launch_fwd(const FwdParams& p, int dtype, int head_dim, bool causal, 
     case 128: return launch_fwd_d<128>(p, dtype, causal, dropout, sparse, stream);
     default: return hipErrorInvalidValue;
   }
+}
+
+// Merges the partial results of a key-split forward: lse = log sum_s exp(lse_s), o = sum_s exp(lse_s - lse) o_s.
+// One thread per (batch, head, query row, 4 output columns).
+template <typename T>
+__global__ void __launch_bounds__(256) fwd_combine_kernel(const FwdParams p, int D) {
+  const int cpr = D / 4;
+  const int64_t total = (int64_t)p.B * p.H * p.max_sq * cpr;
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= total) return;
+  const int ch = (int)(t % cpr);
+  const int row = (int)((t / cpr) % p.max_sq);
+  const int h = (int)((t / cpr / p.max_sq) % p.H);
+  const int b = (int)(t / cpr / p.max_sq / p.H);
+  int q_begin, Lq;
+  if (!seq_extent(p.cu_q, b, p.total_q, p.max_sq, &q_begin, &Lq) || row >= Lq) return;
+  float m = -INFINITY;
+  for (int s = 0; s < p.n_splits; s++) m = fmaxf(m, p.lse_part[(((int64_t)s * p.B + b) * p.H + h) * p.sq_r + row]);
+  float sum = 0.f;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  if (m > -INFINITY) {
+    for (int s = 0; s < p.n_splits; s++) {
+      const float w = __expf(p.lse_part[(((int64_t)s * p.B + b) * p.H + h) * p.sq_r + row] - m);
+      sum += w;
+      const f32x4 o = *reinterpret_cast<const f32x4*>(p.o_part + (((int64_t)s * p.total_q + q_begin + row) * p.H + h) * D + ch * 4);
+      acc = acc + o * w;
+    }
+    acc = acc * (1.f / sum);
+  }
+  if (ch == 0) p.lse[((int64_t)b * p.H + h) * p.sq_r + row] = m > -INFINITY ? m + __logf(sum) : -INFINITY;
+  T* op = reinterpret_cast<T*>(p.o) + (int64_t)(q_begin + row) * p.o_rs + (int64_t)h * p.o_hs + ch * 4;
+  *reinterpret_cast<typename Elem<T>::vec4*>(op) = cvt4<T>(acc);
+}
+
+hipError_t launch_fwd_combine(const FwdParams& p, int dtype, int head_dim, hipStream_t stream) {
+  const int64_t total = (int64_t)p.B * p.H * p.max_sq * (head_dim / 4);
+  if (total == 0) return hipSuccess;
+  const unsigned grid = (unsigned)((total + 255) / 256);
+  if (dtype == 0) hipLaunchKernelGGL(fwd_combine_kernel<_Float16>, dim3(grid), dim3(256), 0, stream, p, head_dim);
+  else hipLaunchKernelGGL(fwd_combine_kernel<__bf16>, dim3(grid), dim3(256), 0, stream, p, head_dim);
+  return hipGetLastError();
 }
 
 }  // namespace fa

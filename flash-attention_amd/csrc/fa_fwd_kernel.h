@@ -48,7 +48,10 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
   // Workgroup -> (batch, head, query tile), XCD-aware (see map_tile): the query tiles of one (batch, head) share
   // one XCD's L2 copy of K and V.
   int bh, rank;
-  if (!map_tile<kCausal>(blockIdx.x, p.nq_tiles, p.B * p.H, &bh, &rank)) return;
+  const int n_splits = p.n_splits > 1 ? p.n_splits : 1;   // key splits per query tile (see FwdParams)
+  if (!map_tile<kCausal>(blockIdx.x, p.nq_tiles * n_splits, p.B * p.H, &bh, &rank)) return;
+  const int split = rank % n_splits;
+  rank /= n_splits;
   const int qt = kCausal ? p.nq_tiles - 1 - rank : rank;  // under a causal mask the last query tiles cost most
   const int b = bh / p.H, h = bh % p.H;
 
@@ -79,7 +82,9 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
 
   int n_end = Lk;
   if (kCausal) n_end = n_end < m0 + BM ? n_end : m0 + BM;
-  const int ntiles = (n_end + BN - 1) / BN;
+  const int ntiles_all = (n_end + BN - 1) / BN;
+  const int tile0 = (int)((int64_t)split * ntiles_all / n_splits);        // this workgroup's share of the key tiles
+  const int ntiles = (int)((int64_t)(split + 1) * ntiles_all / n_splits);
 
   // ---- K/V staging: global -> LDS without passing through registers (waves 0,1 fetch K tiles, waves 2,3 V tiles)
   typename Cfg::Stager stager;
@@ -115,7 +120,7 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
   for (int ks = 0; ks < D / 16; ks++) koff[ks] = frag_off<D, kSwzRow>(c, ks * 2 + hf);
   int buf = 0;
 
-  int it = next_active(0);
+  int it = next_active(tile0);
   if (it < ntiles) stage(it, 0);
   while (it < ntiles) {
     const int n0 = it * BN;
@@ -238,10 +243,27 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
   const bool empty = !(l_tot > 0.f);  // also catches NaN (fmha_fprop_kernel_1xN.h:575,606)
   float inv = empty ? 1.f : fast_rcp(l_tot);
   if (kDropout) inv *= p.rp_keep;
-  if (hf == 0 && qrow < Lq) {
-    const float lse = empty ? -INFINITY : (m_i * cs + fast_log2(l_tot)) * kLn2;
-    p.lse[((int64_t)b * p.H + h) * p.sq_r + qrow] = lse;
+  const float lse_val = empty ? -INFINITY : (m_i * cs + fast_log2(l_tot)) * kLn2;
+  if (p.n_splits > 1) {  // partial result of this key split, fp32, merged by fwd_combine_kernel
+    if (qrow < Lq) {
+      if (hf == 0) p.lse_part[(((int64_t)split * p.B + b) * p.H + h) * p.sq_r + qrow] = lse_val;
+      float* op = p.o_part + (((int64_t)split * p.total_q + q_begin + qrow) * p.H + h) * D;
+#pragma unroll
+      for (int db = 0; db < DV / 32; db++)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          const int d0 = db * 32 + g4 * 8 + hf * 4;
+          if (d0 < D) {
+            f32x4 x;
+#pragma unroll
+            for (int i = 0; i < 4; i++) x[i] = o_acc[db][g4 * 4 + i] * inv;
+            *reinterpret_cast<f32x4*>(op + d0) = x;
+          }
+        }
+    }
+    return;
   }
+  if (hf == 0 && qrow < Lq) p.lse[((int64_t)b * p.H + h) * p.sq_r + qrow] = lse_val;
   __syncthreads();
   constexpr int OS = Cfg::OS;
   T* Os = reinterpret_cast<T*>(lds_raw) + wave * 32 * OS;

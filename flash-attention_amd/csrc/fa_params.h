@@ -45,6 +45,12 @@ struct FwdParams {
   uint32_t keep_thr; // floor(keep * 65535)
   PhiloxKey pk;
   SparseMaps sp;
+  // Key-split forward (few query tiles, many keys): split s of n_splits handles a contiguous share of the key tiles
+  // and writes its normalised fp32 output and its lse to o_part [n_splits, total_q, H, d] / lse_part
+  // [n_splits, B, H, sq_r]; fwd_combine_kernel merges them into o / lse.  n_splits <= 1: single pass.
+  int n_splits;
+  float* o_part;
+  float* lse_part;
 };
 
 struct DumpParams {  // return_softmax path
@@ -139,6 +145,7 @@ inline int tile_grid(bool tile_major, int tiles_per_bh, int BH) {
 // Launchers (defined in fa_fwd.hip / fa_bwd.hip / fa_aux.hip).  Return hipError_t of the launch.
 hipError_t launch_fwd(const FwdParams& p, int dtype, int head_dim, bool causal, bool dropout, bool sparse,
                       hipStream_t stream);
+hipError_t launch_fwd_combine(const FwdParams& p, int dtype, int head_dim, hipStream_t stream);
 // fa_rotary: rotate the first n_rotated of n_parts (row, part, head, head_dim) slices, copy the others
 struct RotaryParams {
   const void* src;

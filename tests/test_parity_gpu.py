@@ -730,3 +730,69 @@ def test_rotary_kernel_matches_oracle(dtype, D):
                               sin_h.double().cpu().numpy(), pos, conjugate=True)
         close(x.grad[:, :, part].reshape(B * S, H, D), want)
     assert torch.equal(x.grad[:, :, 2].cpu(), go[:, :, 2])
+
+
+# ------------------------------------------------------------------------------------------------
+# key-split forward (short query side, long key side: decode / cross-attention shapes)
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("lens_q,lens_k,D,p", [
+    ([1, 1], [2048, 1500], 64, 0.0),        # one query per sequence
+    ([16, 5, 128], [1024, 4000, 513], 64, 0.0),
+    ([100], [3000], 128, 0.0),
+    ([3, 40], [1300, 2100], 32, 0.15),
+])
+def test_key_split_forward(lens_q, lens_k, D, p):
+    """fa_fwd with the scratch fa_fwd_workspace_bytes() asks for takes the key-split path; results must match the
+    oracle, the single-pass kernel (same call without workspace) and, with dropout, use the same mask."""
+    from flash_attn import flash_attn_gfx950 as be
+    lib = be.load_library()
+    H, dtype = 3, torch.float16
+    q, k, v, do = _inputs(lens_q, lens_k, H, D, dtype, seed=sum(lens_k))
+    cu_q, cu_k = _cu(lens_q, "cuda"), _cu(lens_k, "cuda")
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    sq_r, _ = be.round_seqlens(D, max(lens_q), max(lens_k))
+
+    def call(with_ws):
+        o = torch.zeros_like(qd)
+        lse = torch.full((len(lens_q), H, sq_r), float("nan"), device="cuda")
+        a = be.FwdArgs()
+        a.struct_bytes = ctypes.sizeof(a)
+        a.dtype = 0
+        a.q, a.k, a.v, a.o, a.softmax_lse = qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), o.data_ptr(), lse.data_ptr()
+        a.cu_seqlens_q, a.cu_seqlens_k = cu_q.data_ptr(), cu_k.data_ptr()
+        a.q_row_stride = a.k_row_stride = a.v_row_stride = a.o_row_stride = H * D
+        a.q_head_stride = a.k_head_stride = a.v_head_stride = a.o_head_stride = D
+        a.batch, a.nheads, a.head_dim = len(lens_q), H, D
+        a.total_q, a.total_k, a.max_seqlen_q, a.max_seqlen_k = sum(lens_q), sum(lens_k), max(lens_q), max(lens_k)
+        a.p_dropout, a.softmax_scale = p, D ** -0.5
+        a.philox_seed, a.philox_offset = 1234, 8
+        need = lib.fa_fwd_workspace_bytes(ctypes.byref(a))
+        assert need > 0
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda") if with_ws else None
+        a.workspace, a.workspace_bytes = (ws.data_ptr(), need) if with_ws else (None, 0)
+        assert lib.fa_fwd(ctypes.byref(a)) == 0, lib.fa_last_error()
+        torch.cuda.synchronize()
+        return o.cpu(), lse.cpu()
+
+    o_split, lse_split = call(True)
+    o_single, lse_single = call(False)
+    masks = None
+    if p > 0:
+        masks = [torch.tensor(np.stack([orc.dropout_keep_mask(1234, 8, b * H + h, lq, lk, p) for h in range(H)]))
+                 for b, (lq, lk) in enumerate(zip(lens_q, lens_k))]
+    ref = orc.varlen_attention(q, k, v, cu_q.cpu(), cu_k.cpu(), D ** -0.5, False, p_dropout=p, keep_mask=masks)
+    tol = 2e-3
+    assert (o_split.float() - ref["out"]).abs().max() < tol and (o_single.float() - ref["out"]).abs().max() < tol
+    assert (o_split.float() - o_single.float()).abs().max() < 1e-3
+    for b, L in enumerate(lens_q):
+        assert (lse_split[b, :, :L] - ref["lse"][b]).abs().max() < 2e-3
+        assert (lse_split[b, :, :L] - lse_single[b, :, :L]).abs().max() < 1e-4
+    # the interface layer allocates the scratch itself and backpropagates through the result
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    from flash_attn.flash_attn_interface import flash_attn_unpadded_func
+    out = flash_attn_unpadded_func(qg, kg, vg, cu_q, cu_k, max(lens_q), max(lens_k), 0.0)
+    assert (out.float().cpu() - orc.varlen_attention(q, k, v, cu_q.cpu(), cu_k.cpu(), D ** -0.5, False)["out"]).abs().max() < tol
+    out.backward(do.cuda())
+    refb = orc.varlen_attention(q, k, v, cu_q.cpu(), cu_k.cpu(), D ** -0.5, False, dout=do)
+    for name, g in (("dq", qg.grad), ("dk", kg.grad), ("dv", vg.grad)):
+        assert (g.float().cpu() - refb[name]).abs().max() < 5e-3, name
