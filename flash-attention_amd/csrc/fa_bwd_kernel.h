@@ -59,6 +59,8 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
   using vec8 = typename E::vec8;
   using vec4 = typename E::vec4;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, DV = Cfg::DV, CH = Cfg::CH, kBufBytes = Cfg::kBufBytes;
+  constexpr bool kPipe = D == 128;  // software-pipelined LDS fetches (see the main loop)
+  static_assert(BM == 64, "the main loop handles two 32-row slabs per tile");
 
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
 
@@ -170,6 +172,29 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
 
     const bool diag = kCausal && (m0 < n0 + wave * 32 + 32);  // some (q, key) of this wave's slab has key > q
 
+    // LDS fragment fetches.  With kPipe (d = 128: one wave per SIMD, nobody else hides LDS latency) they are issued a
+    // stage ahead of their MFMAs - the row fragments of a 32-row slab before the previous slab's last MFMAs, the
+    // transposed fragments of a 16-row step under the exponentials / the previous step's MFMAs - and scheduling
+    // barriers keep the compiler from sinking them back.  Otherwise they sit next to their use and other waves hide them.
+    auto load_rows = [&](int qb, vec8* aq, vec8* ad) {
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ks++) aq[ks] = *reinterpret_cast<const vec8*>(Ql + qb * 32 * D + foff[ks]);
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ks++) ad[ks] = *reinterpret_cast<const vec8*>(dOl + qb * 32 * D + foff[ks]);
+    };
+    auto load_tr = [&](int qb, int t, u32x4* avs, u32x4* aqs) {
+      const int off = (qb * 32 + 16 * t) * D;
+#pragma unroll
+      for (int db = 0; db < DV / 32; db++) {
+        u32x2 lo = lds_read_tr16(dOl + off + tlo[db]), hi = lds_read_tr16(dOl + off + thi[db]);
+        avs[db] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+        lo = lds_read_tr16(Ql + off + tlo[db]);
+        hi = lds_read_tr16(Ql + off + thi[db]);
+        aqs[db] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+      }
+    };
+    vec8 aq[2][D / 16], ad[2][D / 16];
+    if (kPipe) load_rows(0, aq[0], ad[0]);
 #pragma unroll
     for (int qb = 0; qb < BM / 32; qb++) {
       // ---- S = Q K^T and dP = dO V^T for 32 query rows x this wave's 32 keys
@@ -181,15 +206,16 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
 #pragma unroll
         for (int i = 0; i < 4; i++) { s[4 * j + i] = 0.f; dp[4 * j + i] = nd4[i]; }
       }
+      if (kPipe) __builtin_amdgcn_sched_barrier(0);
+      else load_rows(qb, aq[qb], ad[qb]);
 #pragma unroll
-      for (int ks = 0; ks < D / 16; ks++) {
-        vec8 aq = *reinterpret_cast<const vec8*>(Ql + qb * 32 * D + foff[ks]);
-        s = E::mfma32(aq, kreg[ks], s);
-      }
+      for (int ks = 0; ks < D / 16; ks++) s = E::mfma32(aq[qb][ks], kreg[ks], s);
 #pragma unroll
-      for (int ks = 0; ks < D / 16; ks++) {
-        vec8 ad = *reinterpret_cast<const vec8*>(dOl + qb * 32 * D + foff[ks]);
-        dp = E::mfma32(ad, vreg[ks], dp);
+      for (int ks = 0; ks < D / 16; ks++) dp = E::mfma32(ad[qb][ks], vreg[ks], dp);
+      u32x4 avs[2][DV / 32], aqs[2][DV / 32];
+      if (kPipe) {
+        load_tr(qb, 0, avs[0], aqs[0]);
+        __builtin_amdgcn_sched_barrier(0);
       }
       // ---- P and dS'
       bool rb_on[2] = {true, true};
@@ -232,16 +258,17 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
         for (int i = 0; i < 8; i++) { pf[i] = s[8 * t + i]; df[i] = dp[8 * t + i]; }
         const vec8 pb = cvt8<T>(pf);
         const vec8 db8 = cvt8<T>(df);
+        if (kPipe) {
+          if (t == 0) load_tr(qb, 1, avs[1], aqs[1]);
+          else if (qb + 1 < BM / 32) load_rows(qb + 1, aq[qb + 1], ad[qb + 1]);
+          __builtin_amdgcn_sched_barrier(0);
+        } else {
+          load_tr(qb, t, avs[t], aqs[t]);
+        }
 #pragma unroll
         for (int db = 0; db < DV / 32; db++) {
-          const int off = (qb * 32 + 16 * t) * D;
-          u32x2 lo = lds_read_tr16(dOl + off + tlo[db]), hi = lds_read_tr16(dOl + off + thi[db]);
-          u32x4 av = {lo[0], lo[1], hi[0], hi[1]};
-          acc_dv[db] = E::mfma32(bitcast<vec8>(av), pb, acc_dv[db]);
-          lo = lds_read_tr16(Ql + off + tlo[db]);
-          hi = lds_read_tr16(Ql + off + thi[db]);
-          u32x4 aq = {lo[0], lo[1], hi[0], hi[1]};
-          acc_dk[db] = E::mfma32(bitcast<vec8>(aq), db8, acc_dk[db]);
+          acc_dv[db] = E::mfma32(bitcast<vec8>(avs[t][db]), pb, acc_dv[db]);
+          acc_dk[db] = E::mfma32(bitcast<vec8>(aqs[t][db]), db8, acc_dk[db]);
         }
       }
     }
