@@ -35,7 +35,9 @@ int fail(int code, const char* fmt, ...) {
 
 inline size_t align16(size_t x) { return (x + 15) & ~(size_t)15; }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
-inline bool stride_ok(int64_t s) { return s % 8 == 0; }
+// strides are in elements: multiples of 8 (16-byte vectors), non-negative, and below 2^24 so that the kernels' 32-bit
+// per-lane byte offsets inside a tile (up to 63 rows) cannot overflow
+inline bool stride_ok(int64_t s) { return s % 8 == 0 && s >= 0 && s < ((int64_t)1 << 24); }
 
 struct Rounded {
   int sq_r, sk_r;
@@ -149,7 +151,7 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
   FA_REQUIRE(stride_ok(a->q_row_stride) && stride_ok(a->q_head_stride) && stride_ok(a->k_row_stride) &&
                  stride_ok(a->k_head_stride) && stride_ok(a->v_row_stride) && stride_ok(a->v_head_stride) &&
                  stride_ok(a->o_row_stride) && stride_ok(a->o_head_stride),
-             "row and head strides must be multiples of 8 elements");
+             "row and head strides must be multiples of 8 elements in [0, 2^24)");
   FA_REQUIRE(!(sparse && a->is_causal), "block-sparse attention does not support causal");  // interface.py:21
 
   const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, sparse);
@@ -234,7 +236,7 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
                              a->k_head_stride, a->v_row_stride,  a->v_head_stride, a->o_row_stride,  a->o_head_stride,
                              a->dq_row_stride, a->dq_head_stride, a->dk_row_stride, a->dk_head_stride, a->dv_row_stride,
                              a->dv_head_stride};
-  for (int64_t s : strides) FA_REQUIRE(stride_ok(s), "row and head strides must be multiples of 8 elements");
+  for (int64_t s : strides) FA_REQUIRE(stride_ok(s), "row and head strides must be multiples of 8 elements in [0, 2^24)");
   FA_REQUIRE(!(sparse && a->is_causal), "block-sparse attention does not support causal");
 
   const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, sparse);
