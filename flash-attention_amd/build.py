@@ -20,7 +20,6 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed fp32 VALU forms are switched off on purpose (build flags)
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-munsafe-fp-atomics",  # hardware global_atomic_add_f32 for the dQ accumulator
     "-Wno-unused-result",
 ]
 

@@ -185,7 +185,6 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
   p.max_sq = a->max_seqlen_q; p.max_sk = a->max_seqlen_k;
   p.sq_r = r.sq_r;
   p.nq_tiles = (a->max_seqlen_q + fa::kFwdBM - 1) / fa::kFwdBM;
-  p.total_tiles = p.nq_tiles * a->nheads * a->batch;
   p.scale = a->softmax_scale;
   p.scale_log2 = a->softmax_scale * fa::kLog2e;
   p.rp_keep = 1.f / p_keep;
@@ -281,9 +280,7 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
   p.max_sq = a->max_seqlen_q; p.max_sk = a->max_seqlen_k;
   p.sq_r = r.sq_r; p.lse_stride = a->lse_seq_stride;
   p.nk_tiles = (a->max_seqlen_k + fa::kBwdBN - 1) / fa::kBwdBN;
-  p.total_tiles = p.nk_tiles * a->nheads * a->batch;
   p.nq_tiles = (a->max_seqlen_q + fa::kFwdBM - 1) / fa::kFwdBM;
-  p.total_qtiles = p.nq_tiles * a->nheads * a->batch;
   p.scale = a->softmax_scale;
   p.scale_log2 = a->softmax_scale * fa::kLog2e;
   p.p_keep = p_keep;

@@ -38,7 +38,6 @@ struct FwdParams {
   int max_sq, max_sk;  // caller's bounds on the sequence lengths; longer sequences are truncated to them
   int sq_r;  // rounded max_seqlen_q = innermost extent of lse
   int nq_tiles;
-  int total_tiles;  // nq_tiles * H * B
   float scale;       // softmax_scale
   float scale_log2;  // softmax_scale * log2(e)
   float rp_keep;     // 1 / keep probability
@@ -93,9 +92,7 @@ struct BwdParams {
   int sq_r;        // innermost extent of dsoftmax
   int lse_stride;  // innermost extent of lse
   int nk_tiles;      // key tiles of the dK/dV kernel
-  int total_tiles;   // nk_tiles * H * B
   int nq_tiles;      // query tiles of the dQ kernel
-  int total_qtiles;  // nq_tiles * H * B
   float scale;
   float scale_log2;
   float p_keep;
