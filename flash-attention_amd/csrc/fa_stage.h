@@ -91,22 +91,33 @@ struct TilePairStager {
   }
   FA_DEVICE int swz(int r) const { return second ? tile_swz<D, KIND1>(r) : tile_swz<D, KIND0>(r); }
 
+  // One direct-to-LDS wave instruction: lane l's 16 bytes at (uniform base + per-lane offset) go to lds_dst + 16 * l.
+  // Written as inline assembly on purpose: the compiler makes every ds_read_b64_tr_b16 that follows a direct-to-LDS
+  // load it knows about wait for vmcnt(0) (it cannot tell that they touch different buffers), which would serialise the
+  // prefetch of the next tile with the use of the current one.  The kernels order these loads against their LDS
+  // reads themselves (wait_vmem() + workgroup barrier).  M0 carries the LDS address, as the instruction requires.
+  static FA_DEVICE void dma16(const char* base, uint32_t lane_off, unsigned char* lds_dst) {
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)(lptr_t)lds_dst;
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(lane_off), "s"(base), "s"(lds_addr)
+                 : "memory", "m0");
+  }
+
   // Issues the loads of tile rows [first_row, first_row + ROWS) of both tensors; rows >= n_rows (the tensors' valid
   // extent, > first_row) re-read the last valid row so that LDS never holds anything but real tensor data.
   FA_DEVICE void issue(unsigned char* lds, int first_row, int n_rows) const {
     if (__builtin_expect(first_row + ROWS <= n_rows, 1)) {
       const char* const tb = base + ((int64_t)first_row + row0) * rsb;
 #pragma unroll
-      for (int i = 0; i < NI; i++)
-        __builtin_amdgcn_global_load_lds((gptr_t)(tb + i * RPI * rsb + src_off[i % NOFF]),
-                                         (lptr_t)(lds + dst0 + i * 1024), 16, 0, 0);
+      for (int i = 0; i < NI; i++) dma16(tb + i * RPI * rsb, src_off[i % NOFF], lds + dst0 + i * 1024);
     } else {
+      const char* const tb = base + (int64_t)first_row * rsb;
 #pragma unroll
       for (int i = 0; i < NI; i++) {
         const int r = row0 + i * RPI + rl;
-        const int rc = first_row + r < n_rows ? first_row + r : n_rows - 1;
-        __builtin_amdgcn_global_load_lds((gptr_t)(base + (int64_t)rc * rsb + 16 * (pch ^ swz(r))),
-                                         (lptr_t)(lds + dst0 + i * 1024), 16, 0, 0);
+        const int rc = first_row + r < n_rows ? r : n_rows - 1 - first_row;
+        dma16(tb, (uint32_t)(rc * rsb) + 16u * (uint32_t)(pch ^ swz(r)), lds + dst0 + i * 1024);
       }
     }
   }
@@ -114,5 +125,11 @@ struct TilePairStager {
 
 // s_waitcnt vmcnt(0): every global load this wave has issued, direct-to-LDS ones included, has completed.
 FA_DEVICE void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0f70); }
+// s_waitcnt vmcnt(N): all but the N most recently issued of them have completed (they complete in order).
+template <int N>
+FA_DEVICE void wait_vmem_but() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
 
 }  // namespace fa
