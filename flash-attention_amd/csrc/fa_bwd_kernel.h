@@ -42,12 +42,8 @@ struct BwdCfg {
   // then two buffers of per-row statistics (lse and -Dk)
   typedef TilePairStager<D, BM, kSwzDual, kSwzDual> Stager;
   static constexpr int kBufBytes = Stager::kPairBytes;
-  // Tile buffers: two (the next tile streams in while this one is used) where several workgroups share a CU and hide
-  // each other's load latency; three at d = 128, where one workgroup owns the CU and a tile must be requested two
-  // steps ahead to arrive in time.
-  static constexpr int kStages = D == 128 ? 3 : 2;
   static constexpr int kSlack = D < 32 ? 64 : 0;  // the 32-wide transposed reads run past a 16-wide row
-  static constexpr int kOffStat = kStages * kBufBytes + kSlack;
+  static constexpr int kOffStat = 2 * kBufBytes + kSlack;
   static constexpr int kStatBytes = 2 * BM * 4;   // lse[BM], -Dk[BM]
   static constexpr int kTileBytes = kOffStat + 2 * kStatBytes;
   static constexpr int kEpiBytes = BN * (D + 8) * 2;
@@ -64,7 +60,6 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
   using vec4 = typename E::vec4;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, DV = Cfg::DV, CH = Cfg::CH, kBufBytes = Cfg::kBufBytes;
   constexpr bool kPipe = D == 128;  // software-pipelined LDS fetches (see the main loop)
-  constexpr int kStages = Cfg::kStages;
   static_assert(BM == 64, "the main loop handles two 32-row slabs per tile");
 
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
@@ -115,8 +110,11 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
   // The statistics are only LOADED here, ahead of the tile's direct-to-LDS loads and untouched until the next
   // iteration: any arithmetic on them at this point would make the wave wait for the load (and, memory operations
   // completing in order, for everything issued before it) right away.
+  // Row statistics of a tile (lse and Dk of its BM rows) wait in a register of threads 0 .. 2*BM-1 and are only
+  // converted when the tile is consumed: arithmetic on a loaded value at this point would make the wave wait for the
+  // load - and, memory operations completing in order, for everything issued before it - right away.
   float statpre = 0.f;
-  auto load_stats = [&](int mt) {
+  auto stage = [&](int mt, int buf) {
     const int m0 = mt * BM;
     if (tid < BM) {
       const int row = m0 + tid;
@@ -127,8 +125,8 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
       statpre = 0.f;
       if (row < Lq) statpre = dsbase[row];
     }
+    stager.issue(lds_raw + buf * kBufBytes, m0, Lq);
   };
-  auto stage_tile = [&](int mt, int buf) { stager.issue(lds_raw + buf * kBufBytes, mt * BM, Lq); };
   // lse scaled to base 2, +inf (row off) where the row saw no key; Dk negated: the dP accumulator starts from -Dk
   auto stat_value = [&]() -> float {
     if (tid < BM) return (statpre == -INFINITY) ? INFINITY : statpre * kLog2e;
@@ -165,37 +163,20 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
   }
   int buf = 0;
 
-  // Memory operations complete in order, so the order of issue fixes what a partial wait guarantees: per step the
-  // statistics of the NEXT tile are requested first, then the tile that is kStages - 1 steps ahead.  At the top of a
-  // step everything except the most recent tile request must have landed.
   int mt = next_active(mt_begin);
-  int mt_n1 = mt < mt_end ? next_active(mt + 1) : mt_end;
-  if (mt < mt_end) {
-    load_stats(mt);
-    stage_tile(mt, 0);
-    if (kStages == 3 && mt_n1 < mt_end) stage_tile(mt_n1, 1);
-  }
-  int sbuf = 0;
+  if (mt < mt_end) stage(mt, 0);
   while (mt < mt_end) {
     const int m0 = mt * BM;
-    if (kStages == 3 && mt_n1 < mt_end) wait_vmem_but<Cfg::Stager::NI>();  // all but the tile requested last
-    else wait_vmem();
-    float* const lse_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffStat + sbuf * Cfg::kStatBytes);
+    wait_vmem();  // this thread's share of tile `mt` has arrived (LDS) / is in statpre
+    float* const lse_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffStat + buf * Cfg::kStatBytes);
     float* const dk_l = lse_l + BM;
     if (tid < 2 * BM) lse_l[tid] = stat_value();
-    __syncthreads();  // tile `mt` is complete, and nobody still reads the buffer that is refilled next
-    if (kStages == 3) {
-      const int mt_n2 = mt_n1 < mt_end ? next_active(mt_n1 + 1) : mt_end;
-      if (mt_n1 < mt_end) load_stats(mt_n1);
-      if (mt_n2 < mt_end) stage_tile(mt_n2, (buf + 2) % 3);
-    } else if (mt_n1 < mt_end) {
-      load_stats(mt_n1);
-      stage_tile(mt_n1, buf ^ 1);
-    }
+    __syncthreads();  // tile `mt` is complete, and nobody still reads the other buffer
+    const int mt_next = next_active(mt + 1);
+    if (mt_next < mt_end) stage(mt_next, buf ^ 1);
     const T* const Ql = reinterpret_cast<const T*>(lds_raw + buf * kBufBytes);
     const T* const dOl = Ql + BM * D;
-    buf = (buf + 1) % kStages;
-    sbuf ^= 1;
+    buf ^= 1;
 
     const bool diag = kCausal && (m0 < n0 + wave * 32 + 32);  // some (q, key) of this wave's slab has key > q
 
@@ -299,8 +280,7 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
         }
       }
     }
-    mt = mt_n1;
-    mt_n1 = mt < mt_end ? next_active(mt + 1) : mt_end;
+    mt = mt_next;
   }
 
   // ---- epilogue: scale, transpose dK^T / dV^T through LDS, coalesced stores

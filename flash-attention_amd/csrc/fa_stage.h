@@ -125,11 +125,4 @@ struct TilePairStager {
 
 // s_waitcnt vmcnt(0): every global load this wave has issued, direct-to-LDS ones included, has completed.
 FA_DEVICE void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0f70); }
-// s_waitcnt vmcnt(N): all but the N most recently issued of them have completed (they complete in order).
-template <int N>
-FA_DEVICE void wait_vmem_but() {
-  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-  __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
-}
-
 }  // namespace fa
