@@ -21,6 +21,7 @@ FLAGS = [
     # packed fp32 VALU forms are switched off on purpose (build flags)
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
+    "-Wno-inline-asm",  # fa_stage.h sets M0 inside an asm statement on purpose (direct-to-LDS loads need it)
 ]
 
 
