@@ -1,6 +1,5 @@
-// Small HBM-bound helper kernels around the two attention kernels: fills, the block-sparse activity
-// maps, the backward's rowsum(dO o O) pre-pass, and the probability dump
-// behind return_softmax.
+// Small HBM-bound helper kernels around the attention kernels: fills, the block-sparse activity maps and the
+// probability dump behind return_softmax.
 #include "fa_params.h"
 
 namespace fa {

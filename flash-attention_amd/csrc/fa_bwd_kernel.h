@@ -17,8 +17,9 @@
 //                                       the reference does before these GEMMs, :344,435), A = dO^T / Q^T read from the
 //                                       same row-major LDS tiles with ds_read_b64_tr_b16
 //
-// fa_bwd_dq_kernel    one workgroup owns 128 query rows (wave w: rows 32w..32w+31), keeps Q, dO fragments, lse, Dk and
-//   the dQ^T accumulator in registers and streams 64-key tiles of K and V through LDS; everything transposed so one
+// fa_bwd_dq_kernel    (launched first) one workgroup owns 128 query rows (wave w: rows 32w..32w+31), keeps Q, dO
+//   fragments, lse and the dQ^T accumulator in registers, computes Dk = keep * rowsum(dO o O) of its rows (stored to
+//   softmax_d for the dK/dV kernel) and streams 64-key tiles of K and V through LDS; everything transposed so one
 //   lane owns one query row (as in the forward kernel):
 //     S^T = K Q^T, dP^T = V dO^T        A = K / V rows from LDS, B = Q / dO fragments in registers
 //     dQ^T += K^T dS'^T                 B = dS'^T from the accumulator registers, A = K^T via ds_read_b64_tr_b16
