@@ -275,3 +275,49 @@ def test_blocksparse_module_layout_handling_on_host():
     if importlib.util.find_spec("hydra") is None:
         with pytest.raises(RuntimeError, match="hydra"):
             FlashBlocksparseAttention({"_target_": "some.module.Config"})
+
+
+def test_key_split_workspace_plan(lib):
+    """fa_fwd_workspace_bytes asks for scratch only for dense, non-causal forwards with one query tile, few
+    (batch, head) pairs and many keys; the size is n_splits * (fp32 partial outputs + partial lse)."""
+    from flash_attn import flash_attn_gfx950 as be
+    a = _valid_fwd_args(be)
+    a.batch, a.nheads, a.head_dim = 8, 12, 64
+    a.total_q, a.total_k, a.max_seqlen_q, a.max_seqlen_k = 8, 8 * 2048, 1, 2048
+    need = lib.fa_fwd_workspace_bytes(ctypes.byref(a))
+    # 96 workgroups -> 8 splits of 4 key tiles; partial o: 8 x 8 x 12 x 64 fp32, partial lse: 8 x 8 x 12 x 16 fp32
+    assert need == 8 * 8 * 12 * 64 * 4 + 8 * 8 * 12 * 16 * 4
+    a.is_causal = 1
+    assert lib.fa_fwd_workspace_bytes(ctypes.byref(a)) == 0
+    a.is_causal = 0
+    a.max_seqlen_q, a.total_q = 129, 8 * 129                   # more than one query tile per sequence
+    assert lib.fa_fwd_workspace_bytes(ctypes.byref(a)) == 0
+    a.max_seqlen_q, a.total_q, a.max_seqlen_k = 1, 8, 300      # too few keys to share
+    assert lib.fa_fwd_workspace_bytes(ctypes.byref(a)) == 0
+    a.max_seqlen_k, a.batch, a.total_q = 2048, 64, 64          # enough (batch, head) pairs to fill the chip
+    assert lib.fa_fwd_workspace_bytes(ctypes.byref(a)) == 0
+
+
+def test_rows_and_rotary_argument_checks(lib):
+    """the byte-movement entry points reject bad arguments before any launch (CPU only: nothing valid is executed)"""
+    from flash_attn import flash_attn_gfx950 as be
+    assert lib.fa_scatter_rows_workspace_bytes(1000) == 4000 and lib.fa_scatter_rows_workspace_bytes(0) == 0
+    assert lib.fa_gather_rows(0x1000, 0x2000, 0x3000, 4, 4, 64, 32, 64, None) == -1      # row stride < row width
+    assert b"stride" in lib.fa_last_error()
+    assert lib.fa_gather_rows(None, 0x2000, 0x3000, 4, 4, 64, 64, 64, None) == -1        # null source
+    assert lib.fa_gather_rows(None, None, None, 0, 0, 64, 64, 64, None) == 0             # nothing to do
+    assert lib.fa_scatter_rows(0x1000, 0x2000, 0x3000, 4, 8, 64, 64, 64, None, 0, None) == -2
+    assert b"workspace" in lib.fa_last_error()
+    assert lib.fa_scatter_rows(0x1000, 0x2000, 0x3000, 4, -1, 64, 64, 64, 0x4000, 64, None) == -1
+    r = be.RotaryArgs()
+    r.struct_bytes = ctypes.sizeof(r) - 4
+    assert lib.fa_rotary(ctypes.byref(r)) == -1 and b"struct size" in lib.fa_last_error()
+    r.struct_bytes = ctypes.sizeof(r)
+    r.dtype, r.n_rows, r.n_parts, r.n_rotated, r.n_heads, r.head_dim = 0, 4, 3, 2, 2, 12
+    assert lib.fa_rotary(ctypes.byref(r)) == -1 and b"multiple of 8" in lib.fa_last_error()
+    r.head_dim, r.n_rotated = 64, 4
+    assert lib.fa_rotary(ctypes.byref(r)) == -1 and b"sizes" in lib.fa_last_error()
+    r.n_rotated = 2
+    assert lib.fa_rotary(ctypes.byref(r)) == -1 and b"null" in lib.fa_last_error()
+    r.n_rows = 0
+    assert lib.fa_rotary(ctypes.byref(r)) == 0
