@@ -238,6 +238,18 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
       }
       uint32_t keep = 0xffffu;
       if (kDropout) keep = keep16_col_layout(p.pk, (uint32_t)bh, m0 + qb * 32, key, hf, p.keep_thr);
+      if (kCausal && diag) {  // only slabs that straddle the diagonal: scores above it become -inf (P = 0)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int qrow = m0 + qb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
+          if (key > qrow) s[r] = -INFINITY;
+        }
+      }
+      if (kSparse && !(rb_on[0] && rb_on[1])) {  // an inactive 16-row block inside an active tile
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+          if (!rb_on[r >> 3]) s[r] = -INFINITY;
+      }
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_l + qb * 32 + 8 * j + 4 * hf);
@@ -246,12 +258,7 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           const int r = 4 * j + i;
-          float pe = fast_exp2(__builtin_fmaf(s[r], cs, -lse4[i]));
-          if (kCausal && diag) {
-            const int qrow = m0 + qb * 32 + 8 * j + 4 * hf + i;
-            if (key > qrow) pe = 0.f;
-          }
-          if (kSparse && !rb_on[j >> 1]) pe = 0.f;
+          const float pe = fast_exp2(__builtin_fmaf(s[r], cs, -lse4[i]));
           float dpe = dp[r];  // dP - Dk
           float pm = pe;
           if (kDropout && !((keep >> r) & 1u)) { dpe = nd4[i]; pm = 0.f; }  // dropped: M o dP = 0
