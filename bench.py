@@ -29,9 +29,21 @@ def attention_flops(B, H, N, D, causal=False):
     return f * (0.5 if causal else 1.0)
 
 
+def sparse_layout(torch, N, density=0.25, seed=0, rows_per_draw=1):
+    """Block mask at the interface's granularity (rows of 16 queries, columns of 256 keys): the diagonal band of
+    256 x 256 blocks plus seeded random blocks, `density` of all blocks active in expectation.  One random draw decides
+    rows_per_draw consecutive mask rows (16: the random blocks are 256 x 256 like the band's)."""
+    nrow, ncol = N // 16, N // 256
+    band = (torch.arange(nrow)[:, None] // 16) == torch.arange(ncol)[None, :]
+    extra = (density - 1.0 / ncol) / (1.0 - 1.0 / ncol)
+    draws = torch.rand(nrow // rows_per_draw, ncol, generator=torch.Generator().manual_seed(seed)) < extra
+    return band | draws.repeat_interleave(rows_per_draw, 0)
+
+
 class Workload:
-    def __init__(self, torch, B, H, D, N, dtype, causal=False, p=0.0, lens=None, seed=0):
+    def __init__(self, torch, B, H, D, N, dtype, causal=False, p=0.0, lens=None, seed=0, blockmask=None):
         self.B, self.H, self.D, self.N, self.dtype, self.causal, self.p = B, H, D, N, dtype, causal, p
+        self.blockmask = blockmask  # (N/16, N/256) bool: the block-sparse entry points are timed instead
         g = torch.Generator(device="cuda").manual_seed(seed)
         lens = lens or [N] * B
         self.lens = lens
@@ -46,17 +58,33 @@ class Workload:
         self.dqkv = torch.empty_like(self.qkv)
         self.scale = D ** -0.5
         self.fwd_flops = sum(4.0 * H * L * L * D for L in lens) * (0.5 if causal else 1.0)
+        if blockmask is not None:  # only the active 16 x 256 blocks are counted
+            self.fwd_flops = 4.0 * B * H * D * 16 * 256 * float(blockmask.sum())
+            from flash_attn.flash_blocksparse_attn_interface import convert_blockmask
+            self.blockmask = convert_blockmask(blockmask.cuda(), causal=False)  # the entry points' own column-major form
         self.bytes_fwd = 4 * total * H * D * 2 + 4 * B * H * self.max_s          # q,k,v read + o written, lse
         self.bytes_bwd = 8 * total * H * D * 2 + 2 * 4 * B * H * self.max_s      # q,k,v,o,do read + dq,dk,dv written
 
     def forward(self, be):
         q, k, v = self.qkv[:, 0], self.qkv[:, 1], self.qkv[:, 2]
+        if self.blockmask is not None:
+            self.out, self.lse = be.fwd_block(q, k, v, self.cu, self.cu, self.blockmask, self.max_s, self.max_s, self.p,
+                                              self.scale, self.causal, False, None)
+            return
         self.out, self.lse = be.fwd(q, k, v, self.cu, self.cu, self.max_s, self.max_s, self.p, self.scale, False,
                                     self.causal, False, None)
 
     def backward(self, be, events=None):
         q, k, v = self.qkv[:, 0], self.qkv[:, 1], self.qkv[:, 2]
         dq, dk, dv = self.dqkv[:, 0], self.dqkv[:, 1], self.dqkv[:, 2]
+        if self.blockmask is not None:
+            if events is not None:
+                events[0].record()
+            be.bwd_block(self.dout, q, k, v, self.out, self.lse, dq, dk, dv, self.cu, self.cu, self.blockmask, self.max_s,
+                         self.max_s, self.p, self.scale, self.causal, None)
+            if events is not None:
+                events[1].record()  # whole backward: the sparse entry point has no per-kernel hook
+            return
         be.bwd(self.dout, q, k, v, self.out, self.lse, dq, dk, dv, self.cu, self.cu, self.max_s, self.max_s, self.p,
                self.scale, False, self.causal, None, main_kernel_events=events)
 
@@ -198,6 +226,9 @@ def main():
             ("GPT2 causal bf16 N=4096", dict(B=8, H=12, D=64, N=4096, dtype=torch.bfloat16, causal=True)),
             ("d128 fp16 N=2048", dict(B=16, H=12, D=128, N=2048, dtype=torch.float16)),
             ("d128 fp16 N=2048 causal", dict(B=16, H=12, D=128, N=2048, dtype=torch.float16, causal=True)),
+            ("blocksparse 25% 16x256", dict(B=4, H=16, D=64, N=4096, dtype=torch.float16, blockmask=sparse_layout(torch, 4096))),
+            ("blocksparse 25% 256x256", dict(B=4, H=16, D=64, N=4096, dtype=torch.float16,
+                                             blockmask=sparse_layout(torch, 4096, rows_per_draw=16))),
         ]
         print("%-28s %9s %9s %9s %9s %8s %10s" % ("config", "fwd ms", "bwd ms", "fwd TF", "f+b TF", "% peak", "f+b GB/s"),
               file=sys.stderr)

@@ -18,7 +18,8 @@ LIB_PATH = os.path.join(HERE, "flash_attn", "libflash_attn_gfx950.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
-    # packed fp32 VALU forms are switched off on purpose (build flags)
+    # packed fp32 VALU forms (v_pk_*_f32) are switched off on purpose: some of their forms have produced silently
+    # wrong results on this hardware; ordinary float code must not be compiled into them
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
     "-Wno-inline-asm",  # fa_stage.h sets M0 inside an asm statement on purpose (direct-to-LDS loads need it)

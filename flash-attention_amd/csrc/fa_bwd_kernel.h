@@ -108,15 +108,20 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
   typename Cfg::Stager stager;
   stager.init(wave, lane, reinterpret_cast<const T*>(p.q) + (int64_t)q_begin * p.q_rs + (int64_t)h * p.q_hs, p.q_rs,
               reinterpret_cast<const T*>(p.dout) + (int64_t)q_begin * p.do_rs + (int64_t)h * p.do_hs, p.do_rs);
-  // The statistics are only LOADED here, ahead of the tile's direct-to-LDS loads and untouched until the next
-  // iteration: any arithmetic on them at this point would make the wave wait for the load (and, memory operations
-  // completing in order, for everything issued before it) right away.
   // Row statistics of a tile (lse and Dk of its BM rows) wait in a register of threads 0 .. 2*BM-1 and are only
   // converted when the tile is consumed: arithmetic on a loaded value at this point would make the wave wait for the
   // load - and, memory operations completing in order, for everything issued before it - right away.
+  // Sparse: the activity bytes of the tile's four 16-row blocks for this key block travel the same way (lane l holds
+  // that of row block l & 3).
   float statpre = 0.f;
+  int actpre = 1;
   auto stage = [&](int mt, int buf) {
     const int m0 = mt * BM;
+    if (kSparse) {
+      int rb = (m0 >> 4) + (lane & 3);
+      rb = rb < p.sp.nrb ? rb : p.sp.nrb - 1;
+      actpre = p.sp.act16[rb * p.sp.ncb + (n0 >> 8)];
+    }
     if (tid < BM) {
       const int row = m0 + tid;
       statpre = INFINITY;  // rows past the end are switched off (P = 0)
@@ -172,6 +177,8 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
     float* const lse_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffStat + buf * Cfg::kStatBytes);
     float* const dk_l = lse_l + BM;
     if (tid < 2 * BM) lse_l[tid] = stat_value();
+    uint64_t rows_on = ~0ull;  // bit j (j < 4): 16-row block j of this tile attends this key block
+    if (kSparse) rows_on = __ballot(actpre != 0);
     __syncthreads();  // tile `mt` is complete, and nobody still reads the other buffer
     const int mt_next = next_active(mt + 1);
     if (mt_next < mt_end) stage(mt_next, buf ^ 1);
@@ -206,6 +213,15 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
     if (kPipe) load_rows(0, aq[0], ad[0]);
 #pragma unroll
     for (int qb = 0; qb < BM / 32; qb++) {
+      bool rb_on[2] = {true, true};
+      if (kSparse) {
+        rb_on[0] = (rows_on >> (2 * qb)) & 1;
+        rb_on[1] = (rows_on >> (2 * qb + 1)) & 1;
+        if (!(rb_on[0] || rb_on[1])) {  // no row of this slab attends the key block: nothing to add to dK, dV
+          if (kPipe && qb + 1 < BM / 32) load_rows(qb + 1, aq[qb + 1], ad[qb + 1]);
+          continue;
+        }
+      }
       // ---- S = Q K^T and dP = dO V^T for 32 query rows x this wave's 32 keys
       // dP starts from -Dk of its query row (fmha_dgrad_kernel_1xN_loop.h:361-371), so the MFMA delivers dP - Dk
       f32x16 s, dp;
@@ -227,17 +243,8 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
         __builtin_amdgcn_sched_barrier(0);
       }
       // ---- P and dS'
-      bool rb_on[2] = {true, true};
-      if (kSparse) {
-#pragma unroll
-        for (int u = 0; u < 2; u++) {
-          int rb = (m0 + qb * 32 + u * 16) >> 4;
-          rb = rb < p.sp.nrb ? rb : p.sp.nrb - 1;
-          rb_on[u] = p.sp.act16[rb * p.sp.ncb + (n0 >> 8)] != 0;
-        }
-      }
-      uint32_t keep = 0xffffu;
-      if (kDropout) keep = keep16_col_layout(p.pk, (uint32_t)bh, m0 + qb * 32, key, hf, p.keep_thr);
+      KeepFields keep;
+      if (kDropout) keep = keep_fields_col_layout(p.pk, (uint32_t)bh, m0 + qb * 32, key, hf);
       if (kCausal && diag) {  // only slabs that straddle the diagonal: scores above it become -inf (P = 0)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
@@ -261,7 +268,7 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
           const float pe = fast_exp2(__builtin_fmaf(s[r], cs, -lse4[i]));
           float dpe = dp[r];  // dP - Dk
           float pm = pe;
-          if (kDropout && !((keep >> r) & 1u)) { dpe = nd4[i]; pm = 0.f; }  // dropped: M o dP = 0
+          if (kDropout && !keep.keep_col(r, p.keep_thr)) { dpe = nd4[i]; pm = 0.f; }  // dropped: M o dP = 0
           s[r] = pm;          // P o M, feeds dV
           dp[r] = pe * dpe;   // dS' = P o (M o dP - Dk), feeds dK
         }
@@ -450,8 +457,16 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
   }
   int buf = 0;
 
+  // Sparse: this lane's 16-row block's activity byte for a tile, fetched one tile ahead and compared when consumed
+  const uint8_t* act_row = nullptr;
+  if (kSparse) act_row = p.sp.act16 + (int64_t)((qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1) * p.sp.ncb;
+  int act_cur = 1, act_next = 1;
+
   int it = next_active(0);
-  if (it < ntiles) stage(it, 0);
+  if (it < ntiles) {
+    stage(it, 0);
+    if (kSparse) act_cur = act_row[(it * BN) >> 8];
+  }
   while (it < ntiles) {
     const int n0 = it * BN;
     // Opaque redefinition of the accumulators (keeps the register allocator from copying them around the loop)
@@ -460,7 +475,10 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
     wait_vmem();      // this wave's share of tile `it` is in LDS
     __syncthreads();  // so is everyone else's, and nobody still reads the other buffer
     const int it_next = next_active(it + 1);
-    if (it_next < ntiles) stage(it_next, buf ^ 1);
+    if (it_next < ntiles) {
+      stage(it_next, buf ^ 1);
+      if (kSparse) act_next = act_row[(it_next * BN) >> 8];
+    }
     const T* const Ks = reinterpret_cast<const T*>(lds_raw + buf * kBufBytes);
     const T* const Vs = Ks + BN * D;
     buf ^= 1;
@@ -469,8 +487,8 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
     if (kCausal && n0 > mw + 31) wave_work = false;
     bool row_on = true;
     if (kSparse) {
-      const int rb = (qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1;
-      row_on = p.sp.act16[rb * p.sp.ncb + (n0 >> 8)] != 0;
+      row_on = act_cur != 0;
+      act_cur = act_next;
       if (__ballot(row_on) == 0) wave_work = false;
     }
     if (wave_work) {
@@ -501,13 +519,13 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
             if (dead) s[r] = -INFINITY;
           }
         }
-        uint32_t keep = 0xffffu;
-        if (kDropout) keep = keep16_row_layout(p.pk, (uint32_t)bh, qrow, n0 + kb * 32, hf, p.keep_thr);
+        KeepFields keep;
+        if (kDropout) keep = keep_fields_row_layout(p.pk, (uint32_t)bh, qrow, n0 + kb * 32, hf);
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           const float pe = fast_exp2(__builtin_fmaf(s[r], cs, -lse2));  // 0 for dead scores and switched-off rows
           float dpe = kInitNegD ? dp[r] : dp[r] - dkv;  // dP - Dk
-          if (kDropout && !((keep >> r) & 1u)) dpe = -dkv;
+          if (kDropout && !keep.keep_row(r, p.keep_thr)) dpe = -dkv;
           s[r] = pe * dpe;  // dS'
         }
 #pragma unroll

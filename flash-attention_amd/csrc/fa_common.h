@@ -145,14 +145,17 @@ struct PhiloxKey {
   uint32_t c3;      // offset_lo
 };
 
+// a ^ b ^ c in one instruction (v_bitop3_b32 with the parity truth table)
+FA_DEVICE uint32_t xor3(uint32_t a, uint32_t b, uint32_t c) { return __builtin_amdgcn_bitop3_b32(a, b, c, 0x96); }
+
 FA_DEVICE u32x4 philox4x32_7(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1) {
 #pragma unroll
   for (int i = 0; i < 7; i++) {
     uint64_t p0 = (uint64_t)0xD2511F53u * c0;
     uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
-    uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    uint32_t n0 = xor3((uint32_t)(p1 >> 32), c1, k0);
     uint32_t n1 = (uint32_t)p1;
-    uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    uint32_t n2 = xor3((uint32_t)(p0 >> 32), c3, k1);
     uint32_t n3 = (uint32_t)p0;
     c0 = n0; c1 = n1; c2 = n2; c3 = n3;
     k0 += 0x9E3779B9u;
@@ -178,38 +181,81 @@ FA_DEVICE uint32_t dropout_keep_bits16(const PhiloxKey& pk, uint32_t bh, uint32_
   return bits;
 }
 
-// Broadcast lane (4*(lane/4) + j)'s value to the 4 lanes of its quad.
-template <int J>
-FA_DEVICE uint32_t quad_bcast(uint32_t x) {
-  return (uint32_t)__builtin_amdgcn_mov_dpp((int)x, J | (J << 2) | (J << 4) | (J << 6), 0xf, 0xf, true);
+// dest lane i of every quad reads lane P_i of its quad (CTRL = P0 | P1 << 2 | P2 << 4 | P3 << 6)
+template <int CTRL>
+FA_DEVICE uint32_t quad_perm(uint32_t x) {
+  return (uint32_t)__builtin_amdgcn_mov_dpp((int)x, CTRL, 0xf, 0xf, true);
 }
+constexpr int kQuadXor1 = 0xB1, kQuadXor2 = 0x4E;  // lane ^ 1, lane ^ 2
 
-// Keep bits of the 16 score elements one lane owns in a 32x32 MFMA accumulator tile; bit r <=> register r is kept.
+// The 16 random 16-bit fields that decide the 16 score elements one lane owns in a 32x32 MFMA accumulator tile.
 // "Row layout" (S^T = K Q^T tiles: lane -> query row `qrow`, register r -> key key0 + 8*(r/4) + 4*hf + r%4) and
 // "column layout" (S = Q K^T tiles: lane -> key `key`, register r -> query row q0 + 8*(r/4) + 4*hf + r%4).
-// The four lanes of a quad own the four rows (columns) of the same four micro-blocks; lane t of the quad draws the
-// Philox numbers of micro-block t and the quad exchanges the resulting 16-bit masks with DPP broadcasts.
-FA_DEVICE uint32_t keep16_row_layout(const PhiloxKey& pk, uint32_t bh, int qrow, int key0, int hf, uint32_t thr) {
-  const int t = qrow & 3;
-  const uint32_t mine = dropout_keep_bits16(pk, bh, (uint32_t)qrow >> 2, ((uint32_t)key0 >> 2) + 2 * t + hf, thr);
-  uint32_t r = ((quad_bcast<0>(mine) >> (4 * t)) & 0xfu);
-  r |= ((quad_bcast<1>(mine) >> (4 * t)) & 0xfu) << 4;
-  r |= ((quad_bcast<2>(mine) >> (4 * t)) & 0xfu) << 8;
-  r |= ((quad_bcast<3>(mine) >> (4 * t)) & 0xfu) << 12;
-  return r;
+// The four lanes of a quad own the four rows (columns) of the same four micro-blocks.  Lane t of the quad draws the
+// two Philox outputs of micro-block t (8 words = 4 rows of 2 words) and the quad then transposes - every lane needs
+// row (column) lane%4 of all four micro-blocks - in two DPP butterfly stages.  The raw fields travel: nothing is
+// compared, packed into bit masks and unpacked again on the way; the consumer compares a half-word with the threshold.
+struct KeepFields {
+  uint32_t w[8];
+  // row layout: w[2 tt + h] holds row lane%4 of micro-block tt = r / 4, columns 2h (low half) and 2h + 1 (high half)
+  FA_DEVICE bool keep_row(int r, uint32_t thr) const { return ((w[r >> 1] >> (16 * (r & 1))) & 0xffffu) <= thr; }
+  // column layout: w[4 pi + rho] holds row rho = r % 4, column lane%4 of micro-blocks 2 pi (low half), 2 pi + 1 (high)
+  FA_DEVICE bool keep_col(int r, uint32_t thr) const {
+    return ((w[4 * (r >> 3) + (r & 3)] >> (16 * ((r >> 2) & 1))) & 0xffffu) <= thr;
+  }
+};
+
+FA_DEVICE void philox_micro_block(const PhiloxKey& pk, uint32_t bh, uint32_t Q4, uint32_t K4, uint32_t (&a)[8]) {
+  const u32x4 r0 = philox4x32_7((K4 << 1) | 0u, Q4, bh, pk.c3, pk.k0, pk.k1);
+  const u32x4 r1 = philox4x32_7((K4 << 1) | 1u, Q4, bh, pk.c3, pk.k0, pk.k1);
+#pragma unroll
+  for (int i = 0; i < 4; i++) { a[i] = r0[i]; a[4 + i] = r1[i]; }  // row rho of the micro-block: a[2 rho], a[2 rho + 1]
 }
 
-FA_DEVICE uint32_t keep16_col_layout(const PhiloxKey& pk, uint32_t bh, int q0, int key, int hf, uint32_t thr) {
+FA_DEVICE KeepFields keep_fields_row_layout(const PhiloxKey& pk, uint32_t bh, int qrow, int key0, int hf) {
+  const int t = qrow & 3;
+  uint32_t a[8];
+  philox_micro_block(pk, bh, (uint32_t)qrow >> 2, ((uint32_t)key0 >> 2) + 2 * t + hf, a);
+  // 4 x 4 transpose over (lane, row): swap bit 0 of both, then bit 1
+  const bool t0 = (t & 1) != 0, t1 = (t & 2) != 0;
+  uint32_t c[8];
+  KeepFields e;
+#pragma unroll
+  for (int rho = 0; rho < 4; rho++)
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const uint32_t nb = quad_perm<kQuadXor1>(a[2 * (rho ^ 1) + h]);
+      c[2 * rho + h] = (((rho & 1) != 0) == t0) ? a[2 * rho + h] : nb;
+    }
+#pragma unroll
+  for (int rho = 0; rho < 4; rho++)
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const uint32_t nb = quad_perm<kQuadXor2>(c[2 * (rho ^ 2) + h]);
+      e.w[2 * rho + h] = (((rho & 2) != 0) == t1) ? c[2 * rho + h] : nb;
+    }
+  return e;
+}
+
+FA_DEVICE KeepFields keep_fields_col_layout(const PhiloxKey& pk, uint32_t bh, int q0, int key, int hf) {
   const int t = key & 3;
-  const uint32_t mine = dropout_keep_bits16(pk, bh, ((uint32_t)q0 >> 2) + 2 * t + hf, (uint32_t)key >> 2, thr);
-  const uint32_t b[4] = {quad_bcast<0>(mine) >> t, quad_bcast<1>(mine) >> t, quad_bcast<2>(mine) >> t,
-                         quad_bcast<3>(mine) >> t};
-  uint32_t r = 0;
+  uint32_t a[8];
+  philox_micro_block(pk, bh, ((uint32_t)q0 >> 2) + 2 * t + hf, (uint32_t)key >> 2, a);
+  // Column c of a micro-block is half (c & 1) of its words of parity c >> 1.  Stage 1 swaps lane bit 1 against the
+  // word parity; stage 2 swaps lane bit 0 against the half, by a byte permute whose selector depends on the lane:
+  // even lanes keep their low half and take the neighbour's low half as high half, odd lanes the reverse.
+  const bool t1 = (t & 2) != 0;
+  const uint32_t sel = (t & 1) ? 0x03020706u : 0x05040100u;
+  KeepFields g;
 #pragma unroll
-  for (int j = 0; j < 4; j++)
+  for (int pi = 0; pi < 2; pi++)
 #pragma unroll
-    for (int i = 0; i < 4; i++) r |= ((b[j] >> (4 * i)) & 1u) << (4 * j + i);
-  return r;
+    for (int rho = 0; rho < 4; rho++) {
+      const uint32_t nb2 = quad_perm<kQuadXor2>(a[2 * rho + (pi ^ 1)]);
+      const uint32_t cw = ((pi != 0) == t1) ? a[2 * rho + pi] : nb2;  // from lane (lane & 1) | pi << 1, parity lane / 2
+      g.w[4 * pi + rho] = __builtin_amdgcn_perm(quad_perm<kQuadXor1>(cw), cw, sel);
+    }
+  return g;
 }
 
 }  // namespace fa

@@ -120,8 +120,17 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
   for (int ks = 0; ks < D / 16; ks++) koff[ks] = frag_off<D, kSwzRow>(c, ks * 2 + hf);
   int buf = 0;
 
+  // Sparse: this lane's 16-row block's activity byte for a tile, fetched one tile ahead (its latency hides behind the
+  // current tile) and only compared when it is consumed (vector memory completes in order).
+  const uint8_t* act_row = nullptr;
+  if (kSparse) act_row = p.sp.act16 + (int64_t)((qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1) * p.sp.ncb;
+  int act_cur = 1, act_next = 1;
+
   int it = next_active(tile0);
-  if (it < ntiles) stage(it, 0);
+  if (it < ntiles) {
+    stage(it, 0);
+    if (kSparse) act_cur = act_row[(it * BN) >> 8];
+  }
   while (it < ntiles) {
     const int n0 = it * BN;
     // Opaque redefinition of the accumulators at the top of every iteration: without it the register allocator
@@ -131,7 +140,10 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
     wait_vmem();                         // this wave's share of tile `it` is in LDS
     __syncthreads();                     // so is everyone else's, and nobody still reads the other buffer
     const int it_next = next_active(it + 1);
-    if (it_next < ntiles) stage(it_next, buf ^ 1);
+    if (it_next < ntiles) {
+      stage(it_next, buf ^ 1);
+      if (kSparse) act_next = act_row[(it_next * BN) >> 8];
+    }
     const T* Ks = reinterpret_cast<const T*>(lds_raw + buf * kBufBytes);
     const T* Vs = Ks + BN * D;
     buf ^= 1;
@@ -140,8 +152,8 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
     if (kCausal && n0 > mw + 31) wave_work = false;  // every key of this tile is above the wave's diagonal
     bool row_on = true;
     if (kSparse) {
-      const int rb = (qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1;
-      row_on = p.sp.act16[rb * p.sp.ncb + (n0 >> 8)] != 0;
+      row_on = act_cur != 0;
+      act_cur = act_next;
       if (__ballot(row_on) == 0) wave_work = false;
     }
 
@@ -207,10 +219,10 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
       if (kDropout) {
 #pragma unroll
         for (int kb = 0; kb < BN / 32; kb++) {
-          const uint32_t keep = keep16_row_layout(p.pk, (uint32_t)bh, qrow, n0 + kb * 32, hf, p.keep_thr);
+          const KeepFields keep = keep_fields_row_layout(p.pk, (uint32_t)bh, qrow, n0 + kb * 32, hf);
 #pragma unroll
           for (int r = 0; r < 16; r++)
-            if (!((keep >> r) & 1u)) s[kb][r] = 0.f;
+            if (!keep.keep_row(r, p.keep_thr)) s[kb][r] = 0.f;
         }
       }
 

@@ -249,6 +249,7 @@ def test_error_behaviour_on_device():
 # dropout: exact mask, exact algebra with that mask, keep rate, RNG semantics
 # ------------------------------------------------------------------------------------------------
 def _gen_state():
+    torch.cuda.init()  # the default generators only exist once the runtime is up
     g = torch.cuda.default_generators[torch.cuda.current_device()]
     return g.initial_seed(), g.get_offset()
 
