@@ -60,8 +60,8 @@ Rounded round_seqlens(int head_dim, int max_sq, int max_sk, bool blocksparse) {
 }
 
 struct SparseLayout {
-  int nrb, ncb, nqt, nqt2;
-  size_t off16, offq, offk, bytes;
+  int nrb, ncb, nqt, ncw, nrw;
+  size_t offr, offq, offc, bytes;
 };
 
 SparseLayout sparse_layout(const Rounded& r) {
@@ -69,11 +69,12 @@ SparseLayout sparse_layout(const Rounded& r) {
   s.nrb = r.sq_r / 16;
   s.ncb = r.sk_r / 256;
   s.nqt = (r.sq_r + fa::kFwdBM - 1) / fa::kFwdBM;
-  s.nqt2 = (r.sq_r + fa::kBwdBM - 1) / fa::kBwdBM;
-  s.off16 = 0;
-  s.offq = s.off16 + align16((size_t)s.nrb * s.ncb);
-  s.offk = s.offq + align16((size_t)s.nqt * s.ncb);
-  s.bytes = s.offk + align16((size_t)s.ncb * s.nqt2);
+  s.ncw = (s.ncb + 63) / 64;
+  s.nrw = (s.nrb + 63) / 64;
+  s.offr = 0;
+  s.offq = s.offr + align16((size_t)s.nrb * s.ncw * 8);
+  s.offc = s.offq + align16((size_t)s.nqt * s.ncw * 8);
+  s.bytes = s.offc + align16((size_t)s.ncb * s.nrw * 8);
   return s;
 }
 
@@ -103,15 +104,18 @@ SplitPlan split_plan(int batch, int nheads, int head_dim, int total_q, int max_s
 int build_maps(const int32_t* blockmask, unsigned char* ws, const SparseLayout& sl, fa::SparseMaps* out,
                hipStream_t stream) {
   FA_LAUNCH(fa::launch_fill_f32(reinterpret_cast<float*>(ws), sl.bytes / 4, 0.f, stream));
-  FA_LAUNCH(fa::launch_build_sparse_maps(blockmask, ws + sl.off16, ws + sl.offq, ws + sl.offk, sl.nrb, sl.ncb,
-                                         fa::kFwdBM, sl.nqt, fa::kBwdBM, sl.nqt2, stream));
-  out->act16 = ws + sl.off16;
-  out->actq = ws + sl.offq;
-  out->actk = ws + sl.offk;
+  FA_LAUNCH(fa::launch_build_sparse_maps(blockmask, reinterpret_cast<uint64_t*>(ws + sl.offr),
+                                         reinterpret_cast<uint64_t*>(ws + sl.offq),
+                                         reinterpret_cast<uint64_t*>(ws + sl.offc), sl.nrb, sl.ncb, fa::kFwdBM, sl.nqt,
+                                         sl.ncw, sl.nrw, stream));
+  out->rbits = reinterpret_cast<const uint64_t*>(ws + sl.offr);
+  out->qbits = reinterpret_cast<const uint64_t*>(ws + sl.offq);
+  out->cbits = reinterpret_cast<const uint64_t*>(ws + sl.offc);
   out->nrb = sl.nrb;
   out->ncb = sl.ncb;
   out->nqt = sl.nqt;
-  out->nqt2 = sl.nqt2;
+  out->ncw = sl.ncw;
+  out->nrw = sl.nrw;
   return FA_OK;
 }
 

@@ -27,8 +27,8 @@ __global__ void zero_rows_kernel(uint16_t* base, int64_t rs, int64_t hs, int tot
 
 // blockmask: [ncb][nrb] int32, entries 4*rowblock + flags for the active 16-row blocks of each 256-key
 // column block, -1 padded (flash_blocksparse_attn_interface.py:8-40; read as fmha_blockmask.h:41-53 does).
-__global__ void sparse_maps_kernel(const int32_t* blockmask, uint8_t* act16, uint8_t* actq, uint8_t* actk, int nrb,
-                                   int ncb, int rpq, int nqt, int rpq2, int nqt2) {
+__global__ void sparse_maps_kernel(const int32_t* blockmask, uint32_t* rbits, uint32_t* qbits, uint32_t* cbits, int nrb,
+                                   int ncb, int rpq, int nqt, int ncw, int nrw) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= nrb * ncb) return;
   const int cb = i / nrb;
@@ -36,9 +36,10 @@ __global__ void sparse_maps_kernel(const int32_t* blockmask, uint8_t* act16, uin
   if (e < 0) return;
   const int rb = e >> 2;
   if (rb >= nrb) return;
-  act16[rb * ncb + cb] = 1;
-  if (rb / rpq < nqt) actq[(rb / rpq) * ncb + cb] = 1;
-  if (rb / rpq2 < nqt2) actk[cb * nqt2 + rb / rpq2] = 1;
+  // the 64-bit words are addressed as pairs of 32-bit words (bit b of a word: half b / 32, bit b % 32)
+  atomicOr(rbits + ((int64_t)rb * ncw * 2 + (cb >> 5)), 1u << (cb & 31));
+  if (rb / rpq < nqt) atomicOr(qbits + ((int64_t)(rb / rpq) * ncw * 2 + (cb >> 5)), 1u << (cb & 31));
+  atomicOr(cbits + ((int64_t)cb * nrw * 2 + (rb >> 5)), 1u << (rb & 31));
 }
 
 // One thread per (query row, key) element of S_dmask.  Slow scalar dot products: this path exists for tests
@@ -60,7 +61,7 @@ __global__ void __launch_bounds__(256) dump_probs_kernel(const DumpParams p) {
   if (p.causal && key > qrow) live = false;
   if (live && p.sparse) {
     const int rb = qrow >> 4, cb = key >> 8;
-    live = rb < p.sp.nrb && cb < p.sp.ncb && p.sp.act16[rb * p.sp.ncb + cb] != 0;
+    live = rb < p.sp.nrb && cb < p.sp.ncb && ((p.sp.rbits[(int64_t)rb * p.sp.ncw + (cb >> 6)] >> (cb & 63)) & 1) != 0;
   }
   if (live) {
     const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)(q_begin + qrow) * p.q_rs + (int64_t)h * p.q_hs;
@@ -100,12 +101,12 @@ hipError_t launch_zero_rows(void* base, int64_t row_stride, int64_t head_stride,
   return hipGetLastError();
 }
 
-hipError_t launch_build_sparse_maps(const int32_t* blockmask, uint8_t* act16, uint8_t* actq, uint8_t* actk, int nrb,
-                                    int ncb, int rows_per_qt, int nqt, int rows_per_qt2, int nqt2,
-                                    hipStream_t stream) {
+hipError_t launch_build_sparse_maps(const int32_t* blockmask, uint64_t* rbits, uint64_t* qbits, uint64_t* cbits, int nrb,
+                                    int ncb, int rows_per_qt, int nqt, int ncw, int nrw, hipStream_t stream) {
   const int n = nrb * ncb;
-  hipLaunchKernelGGL(sparse_maps_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, blockmask, act16, actq, actk,
-                     nrb, ncb, rows_per_qt / 16, nqt, rows_per_qt2 / 16, nqt2);
+  hipLaunchKernelGGL(sparse_maps_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, blockmask,
+                     reinterpret_cast<uint32_t*>(rbits), reinterpret_cast<uint32_t*>(qbits),
+                     reinterpret_cast<uint32_t*>(cbits), nrb, ncb, rows_per_qt / 16, nqt, ncw, nrw);
   return hipGetLastError();
 }
 

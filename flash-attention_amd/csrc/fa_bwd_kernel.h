@@ -111,17 +111,9 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
   // Row statistics of a tile (lse and Dk of its BM rows) wait in a register of threads 0 .. 2*BM-1 and are only
   // converted when the tile is consumed: arithmetic on a loaded value at this point would make the wave wait for the
   // load - and, memory operations completing in order, for everything issued before it - right away.
-  // Sparse: the activity bytes of the tile's four 16-row blocks for this key block travel the same way (lane l holds
-  // that of row block l & 3).
   float statpre = 0.f;
-  int actpre = 1;
   auto stage = [&](int mt, int buf) {
     const int m0 = mt * BM;
-    if (kSparse) {
-      int rb = (m0 >> 4) + (lane & 3);
-      rb = rb < p.sp.nrb ? rb : p.sp.nrb - 1;
-      actpre = p.sp.act16[rb * p.sp.ncb + (n0 >> 8)];
-    }
     if (tid < BM) {
       const int row = m0 + tid;
       statpre = INFINITY;  // rows past the end are switched off (P = 0)
@@ -139,9 +131,20 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
     return -statpre;
   };
 
+  // Sparse: the activity bits of 64 consecutive 16-row blocks (16 query tiles) for this key block sit in a register
+  // pair; a query tile is visited iff one of its four row blocks attends the key block.
+  uint64_t col_bits = 0;
+  int bits_word = -1;
+  auto tile_rows_on = [&](int mt) -> uint32_t {  // bit j: 16-row block j of query tile mt attends this key block
+    if ((mt >> 4) != bits_word) {
+      bits_word = __builtin_amdgcn_readfirstlane(mt >> 4);
+      col_bits = uniform64(p.sp.cbits[(int64_t)(n0 >> 8) * p.sp.nrw + bits_word]);
+    }
+    return (uint32_t)(col_bits >> (4 * (mt & 15))) & 0xfu;
+  };
   auto tile_active = [&](int mt) -> bool {
     if (!kSparse) return true;
-    return p.sp.actk[(n0 >> 8) * p.sp.nqt2 + mt] != 0;
+    return tile_rows_on(mt) != 0;
   };
   auto next_active = [&](int mt) -> int {
     while (mt < mt_end && !tile_active(mt)) mt++;
@@ -177,8 +180,8 @@ __global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_k
     float* const lse_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffStat + buf * Cfg::kStatBytes);
     float* const dk_l = lse_l + BM;
     if (tid < 2 * BM) lse_l[tid] = stat_value();
-    uint64_t rows_on = ~0ull;  // bit j (j < 4): 16-row block j of this tile attends this key block
-    if (kSparse) rows_on = __ballot(actpre != 0);
+    uint32_t rows_on = 0xfu;  // bit j: 16-row block j of this tile attends this key block
+    if (kSparse) rows_on = tile_rows_on(mt);
     __syncthreads();  // tile `mt` is complete, and nobody still reads the other buffer
     const int mt_next = next_active(mt + 1);
     if (mt_next < mt_end) stage(mt_next, buf ^ 1);
@@ -427,12 +430,25 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
               reinterpret_cast<const T*>(p.v) + (int64_t)k_begin * p.v_rs + (int64_t)h * p.v_hs, p.v_rs);
   auto stage = [&](int it, int buf) { stager.issue(lds_raw + buf * kBufBytes, it * BN, Lk); };
 
+  // Sparse: the tile's and this lane's row block's activity bits of 64 consecutive key blocks sit in registers
+  uint64_t tile_bits = 0, row_bits = 0;
+  int bits_word = -1;
+  const int qt_u = __builtin_amdgcn_readfirstlane(qt);
   auto tile_active = [&](int it) -> bool {
     if (!kSparse) return true;
-    return p.sp.actq[qt * p.sp.ncb + ((it * BN) >> 8)] != 0;
+    const int cb = __builtin_amdgcn_readfirstlane((it * BN) >> 8);
+    if ((cb >> 6) != bits_word) {
+      bits_word = cb >> 6;
+      tile_bits = uniform64(p.sp.qbits[(int64_t)qt_u * p.sp.ncw + bits_word]);
+      const int rb = (qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1;
+      row_bits = p.sp.rbits[(int64_t)rb * p.sp.ncw + bits_word];
+    }
+    return (tile_bits >> (cb & 63)) & 1;
   };
+  bool row_on_next = true;  // this lane's row block attends the tile the last next_active() found
   auto next_active = [&](int it) -> int {
     while (it < ntiles && !tile_active(it)) it++;
+    if (kSparse && it < ntiles) row_on_next = (row_bits >> (((it * BN) >> 8) & 63)) & 1;
     return it;
   };
 
@@ -457,16 +473,9 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
   }
   int buf = 0;
 
-  // Sparse: this lane's 16-row block's activity byte for a tile, fetched one tile ahead and compared when consumed
-  const uint8_t* act_row = nullptr;
-  if (kSparse) act_row = p.sp.act16 + (int64_t)((qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1) * p.sp.ncb;
-  int act_cur = 1, act_next = 1;
-
   int it = next_active(0);
-  if (it < ntiles) {
-    stage(it, 0);
-    if (kSparse) act_cur = act_row[(it * BN) >> 8];
-  }
+  bool row_on_cur = row_on_next;
+  if (it < ntiles) stage(it, 0);
   while (it < ntiles) {
     const int n0 = it * BN;
     // Opaque redefinition of the accumulators (keeps the register allocator from copying them around the loop)
@@ -475,10 +484,7 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
     wait_vmem();      // this wave's share of tile `it` is in LDS
     __syncthreads();  // so is everyone else's, and nobody still reads the other buffer
     const int it_next = next_active(it + 1);
-    if (it_next < ntiles) {
-      stage(it_next, buf ^ 1);
-      if (kSparse) act_next = act_row[(it_next * BN) >> 8];
-    }
+    if (it_next < ntiles) stage(it_next, buf ^ 1);
     const T* const Ks = reinterpret_cast<const T*>(lds_raw + buf * kBufBytes);
     const T* const Vs = Ks + BN * D;
     buf ^= 1;
@@ -487,8 +493,8 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
     if (kCausal && n0 > mw + 31) wave_work = false;
     bool row_on = true;
     if (kSparse) {
-      row_on = act_cur != 0;
-      act_cur = act_next;
+      row_on = row_on_cur;
+      row_on_cur = row_on_next;  // next_active(it + 1) above has set it
       if (__ballot(row_on) == 0) wave_work = false;
     }
     if (wave_work) {

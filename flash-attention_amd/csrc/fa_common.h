@@ -99,6 +99,13 @@ FA_DEVICE float sum8_acc(bf16x8 v, float acc) {
 // Threshold (log2 units) of the forward kernel's lazy accumulator rescale.
 constexpr float kRescaleLog2 = 8.f;
 
+// A wave-uniform 64-bit value moved to scalar registers (the compiler cannot always prove uniformity of a load)
+FA_DEVICE uint64_t uniform64(uint64_t x) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)x);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(x >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+
 FA_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 FA_DEVICE float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 FA_DEVICE float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }

@@ -37,7 +37,7 @@ struct FwdCfg {
 };
 
 template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse>
-__global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
+__global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2) fa_fwd_kernel(const FwdParams p) {
   using Cfg = FwdCfg<T, D, BN>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
@@ -92,14 +92,26 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
               reinterpret_cast<const T*>(p.v) + (int64_t)k_begin * p.v_rs + (int64_t)h * p.v_hs, p.v_rs);
   auto stage = [&](int it, int buf) { stager.issue(lds_raw + buf * kBufBytes, it * BN, Lk); };
 
-  // Sparse: tile `it` is computed iff its 256-key block is active for any 16-row block of this query tile.
+  // Sparse: tile `it` is computed iff its 256-key block is active for any 16-row block of this query tile.  The tile's
+  // and this lane's row block's activity bits of 64 consecutive key blocks (16384 keys) sit in registers.
+  uint64_t tile_bits = 0, row_bits = 0;
+  int bits_word = -1;
+  const int qt_u = __builtin_amdgcn_readfirstlane(qt);
   auto tile_active = [&](int it) -> bool {
     if (!kSparse) return true;
-    const int cb = (it * BN) >> 8;
-    return p.sp.actq[qt * p.sp.ncb + cb] != 0;
+    const int cb = __builtin_amdgcn_readfirstlane((it * BN) >> 8);
+    if ((cb >> 6) != bits_word) {
+      bits_word = cb >> 6;
+      tile_bits = uniform64(p.sp.qbits[(int64_t)qt_u * p.sp.ncw + bits_word]);
+      const int rb = (qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1;
+      row_bits = p.sp.rbits[(int64_t)rb * p.sp.ncw + bits_word];
+    }
+    return (tile_bits >> (cb & 63)) & 1;
   };
+  bool row_on_next = true;  // this lane's row block attends the tile the last next_active() found
   auto next_active = [&](int it) -> int {
     while (it < ntiles && !tile_active(it)) it++;
+    if (kSparse && it < ntiles) row_on_next = (row_bits >> (((it * BN) >> 8) & 63)) & 1;
     return it;
   };
 
@@ -120,17 +132,9 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
   for (int ks = 0; ks < D / 16; ks++) koff[ks] = frag_off<D, kSwzRow>(c, ks * 2 + hf);
   int buf = 0;
 
-  // Sparse: this lane's 16-row block's activity byte for a tile, fetched one tile ahead (its latency hides behind the
-  // current tile) and only compared when it is consumed (vector memory completes in order).
-  const uint8_t* act_row = nullptr;
-  if (kSparse) act_row = p.sp.act16 + (int64_t)((qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1) * p.sp.ncb;
-  int act_cur = 1, act_next = 1;
-
   int it = next_active(tile0);
-  if (it < ntiles) {
-    stage(it, 0);
-    if (kSparse) act_cur = act_row[(it * BN) >> 8];
-  }
+  bool row_on_cur = row_on_next;
+  if (it < ntiles) stage(it, 0);
   while (it < ntiles) {
     const int n0 = it * BN;
     // Opaque redefinition of the accumulators at the top of every iteration: without it the register allocator
@@ -140,10 +144,7 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
     wait_vmem();                         // this wave's share of tile `it` is in LDS
     __syncthreads();                     // so is everyone else's, and nobody still reads the other buffer
     const int it_next = next_active(it + 1);
-    if (it_next < ntiles) {
-      stage(it_next, buf ^ 1);
-      if (kSparse) act_next = act_row[(it_next * BN) >> 8];
-    }
+    if (it_next < ntiles) stage(it_next, buf ^ 1);
     const T* Ks = reinterpret_cast<const T*>(lds_raw + buf * kBufBytes);
     const T* Vs = Ks + BN * D;
     buf ^= 1;
@@ -152,8 +153,8 @@ __global__ void __launch_bounds__(256, 2) fa_fwd_kernel(const FwdParams p) {
     if (kCausal && n0 > mw + 31) wave_work = false;  // every key of this tile is above the wave's diagonal
     bool row_on = true;
     if (kSparse) {
-      row_on = act_cur != 0;
-      act_cur = act_next;
+      row_on = row_on_cur;
+      row_on_cur = row_on_next;  // next_active(it + 1) above has set it
       if (__ballot(row_on) == 0) wave_work = false;
     }
 

@@ -9,19 +9,19 @@
 
 namespace fa {
 
-// Block-sparse activity maps, built on the device from the reference's converted block list
-// (flash_blocksparse_attn_interface.py:8-40) by build_sparse_maps():
-//   act16[rb * ncb + cb]  != 0  <=> the 16-row x 256-key block (rb, cb) is computed
-//   actq [qt * ncb + cb]  != 0  <=> any 16-row block of forward query tile qt is active in cb
-//   actk [cb * nqt2 + qt2] != 0 <=> any 16-row block of backward query tile qt2 is active in cb
+// Block-sparse activity, built on the device from the reference's converted block list
+// (flash_blocksparse_attn_interface.py:8-40) by launch_build_sparse_maps(): the 16-row x 256-key block (rb, cb) is
+// computed iff its bit is set.  Bit sets (bit j of 64-bit word w <-> block 64 w + j), so that a kernel holds what it
+// needs in a register pair and re-reads memory only every 64 blocks.
 struct SparseMaps {
-  const uint8_t* act16;
-  const uint8_t* actq;
-  const uint8_t* actk;
+  const uint64_t* rbits;  // [nrb][ncw]: 16-row block -> its active 256-key column blocks
+  const uint64_t* qbits;  // [nqt][ncw]: forward query tile -> column blocks active for any of its row blocks
+  const uint64_t* cbits;  // [ncb][nrw]: column block -> its active 16-row blocks
   int nrb;   // 16-row blocks  (= max_seqlen_q_rounded / 16)
   int ncb;   // 256-key blocks (= max_seqlen_k_rounded / 256)
   int nqt;   // forward query tiles
-  int nqt2;  // backward query tiles
+  int ncw;   // 64-bit words per row of rbits / qbits
+  int nrw;   // 64-bit words per row of cbits
 };
 
 struct FwdParams {
@@ -165,8 +165,8 @@ hipError_t launch_dump_probs(const DumpParams& p, int dtype, hipStream_t stream)
 // which: 0 = dQ kernel, 1 = dK/dV kernel
 hipError_t launch_bwd(const BwdParams& p, int which, int dtype, int head_dim, bool causal, bool dropout, bool sparse,
                       hipStream_t stream);
-hipError_t launch_build_sparse_maps(const int32_t* blockmask, uint8_t* act16, uint8_t* actq, uint8_t* actk, int nrb,
-                                    int ncb, int rows_per_qt, int nqt, int rows_per_qt2, int nqt2, hipStream_t stream);
+hipError_t launch_build_sparse_maps(const int32_t* blockmask, uint64_t* rbits, uint64_t* qbits, uint64_t* cbits, int nrb,
+                                    int ncb, int rows_per_qt, int nqt, int ncw, int nrw, hipStream_t stream);
 hipError_t launch_fill_f32(float* p, size_t n, float value, hipStream_t stream);
 // Zero a strided [total, H, D] tensor of 16-bit elements.
 hipError_t launch_zero_rows(void* base, int64_t row_stride, int64_t head_stride, int total, int H, int D,

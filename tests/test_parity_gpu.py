@@ -367,6 +367,31 @@ def test_blocksparse_parity(D, N, p):
     assert S[0, :, :lens[0], :lens[0]].cpu()[:, ~full].abs().max() == 0
 
 
+def test_blocksparse_more_than_64_key_blocks():
+    """The kernels keep the activity bits of 64 key blocks (16384 keys) in registers and reload them beyond: a key side of
+    66 blocks with active blocks on both sides of the boundary, through the raw entry points (separate q and k lengths)."""
+    from flash_attn import flash_attn_gfx950 as be
+    from flash_attn.flash_blocksparse_attn_interface import convert_blockmask
+    H, D, lens_q, lens_k = 2, 32, [200, 120], [16700, 16500]
+    sq_r, sk_r = be.round_seqlens(D, max(lens_q), max(lens_k), True)
+    layout = torch.rand(sq_r // 16, sk_r // 256, generator=torch.Generator().manual_seed(3)) < 0.1
+    layout[:, 63:66] = torch.rand(sq_r // 16, 3, generator=torch.Generator().manual_seed(4)) < 0.5
+    layout[5] = False
+    layout[5, 65] = True        # a row block whose only keys lie beyond the boundary
+    q, k, v, do = _inputs(lens_q, lens_k, H, D, torch.float16, 9)
+    cu_q, cu_k = _cu(lens_q, "cpu"), _cu(lens_k, "cpu")
+    qc, kc, vc, doc = (x.cuda() for x in (q, k, v, do))
+    bm = convert_blockmask(layout.cuda(), causal=False)
+    out, lse = be.fwd_block(qc, kc, vc, cu_q.cuda(), cu_k.cuda(), bm, max(lens_q), max(lens_k), 0.0, D ** -0.5, False, False, None)
+    dq, dk, dv = torch.empty_like(qc), torch.empty_like(kc), torch.empty_like(vc)
+    be.bwd_block(doc, qc, kc, vc, out, lse, dq, dk, dv, cu_q.cuda(), cu_k.cuda(), bm, max(lens_q), max(lens_k), 0.0, D ** -0.5,
+                 False, None)
+    torch.cuda.synchronize()
+    ref = orc.varlen_attention(q, k, v, cu_q, cu_k, None, False, layout=layout.numpy(), dout=do)
+    half = half_attention(qc, kc, vc, cu_q.tolist(), cu_k.tolist(), D ** -0.5, False, layout=layout.numpy(), dout=doc)
+    check_against_oracle({"out": out, "dq": dq, "dk": dk, "dv": dv}, ref, half, torch.float16, what="blocksparse 66 key blocks")
+
+
 def test_blocksparse_full_layout_equals_dense():
     from flash_attn.flash_blocksparse_attn_interface import flash_blocksparse_attn_func
     from flash_attn.flash_attn_interface import flash_attn_unpadded_qkvpacked_func
