@@ -124,6 +124,17 @@ template <bool kTileMajor>
 FA_DEVICE bool map_tile(int block, int tiles_per_bh, int BH, int* bh, int* rank) {
   if (kTileMajor) {
     const int bhp = (BH + 7) & ~7;
+    // A grid small enough to be resident all at once (up to 4 workgroups on each of the 256 compute units) is dealt
+    // out in one go, compute unit c getting ids c, c + 256, ...: then every odd group of 256 ids is walked backwards
+    // (in steps of 8, so that id % 8 is kept), and a compute unit that got one of the dearest tiles of a group gets
+    // one of the cheapest of the next.  Larger grids are scheduled as workgroups retire; plain dearest-first is best.
+    const int grp = block >> 8;
+    if ((grp & 1) && bhp * tiles_per_bh <= 1024) {
+      const int left = bhp * tiles_per_bh - (grp << 8);
+      const int size8 = (left < 256 ? left : 256) >> 3;
+      const int pos = block & 255;
+      block = (grp << 8) + ((size8 - 1 - (pos >> 3)) << 3) + (pos & 7);
+    }
     *rank = block / bhp;
     *bh = block - *rank * bhp;
     return *bh < BH && *rank < tiles_per_bh;
