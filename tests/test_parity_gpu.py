@@ -364,6 +364,31 @@ def test_dropout_backward_reuses_the_forward_mask_without_probs():
     check_against_oracle(ours, ref, half, torch.float16, what="dropout production path")
 
 
+def test_element_offsets_beyond_int32():
+    """A packed qkv tensor of 2.2e9 elements (4.4 GB): the last sequences live at element offsets above 2^31, which the
+    kernels must address with 64-bit arithmetic.  Forward and backward of the first and the last sequence are compared
+    with the oracle; the others only have to be finite."""
+    H, D, N, B = 16, 128, 1024, 350
+    assert B * N * 3 * H * D > 2 ** 31
+    g = torch.Generator(device="cuda").manual_seed(5)
+    qkv = torch.randn(B * N, 3, H, D, device="cuda", dtype=torch.float16, generator=g).requires_grad_()
+    do = torch.randn(B * N, H, D, device="cuda", dtype=torch.float16, generator=g)
+    cu = torch.arange(0, (B + 1) * N, N, dtype=torch.int32, device="cuda")
+    from flash_attn import flash_attn_interface as fi
+    out = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0, None, True)
+    out.backward(do)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all()) and bool(torch.isfinite(qkv.grad).all())
+    cu1 = _cu([N], "cpu")
+    for b in (0, B - 1):
+        sl = slice(b * N, (b + 1) * N)
+        q, k, v = (qkv[sl, i].detach().cpu() for i in range(3))
+        ref = orc.varlen_attention(q, k, v, cu1, cu1, None, True, dout=do[sl].cpu())
+        half = half_attention(q.cuda(), k.cuda(), v.cuda(), [0, N], [0, N], D ** -0.5, True, dout=do[sl])
+        ours = {"out": out[sl].detach(), "dq": qkv.grad[sl, 0], "dk": qkv.grad[sl, 1], "dv": qkv.grad[sl, 2]}
+        check_against_oracle(ours, ref, half, torch.float16, what="sequence %d of %d" % (b, B))
+
+
 def test_parity_random_shapes_sweep():
     """Twenty-four seeded random cases over what the parametrised tests hold fixed: batch size, ragged query and key
     lengths (self- and cross-attention, empty key sides excluded), heads, head dim, dtype, causal, packing, scale."""
