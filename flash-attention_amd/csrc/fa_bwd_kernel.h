@@ -489,7 +489,7 @@ __global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
     const T* const Vs = Ks + BN * D;
     buf ^= 1;
 
-    bool wave_work = true;
+    bool wave_work = mw < Lq;  // a wave whose 32 rows all lie past the sequence's end only helps with the staging
     if (kCausal && n0 > mw + 31) wave_work = false;
     bool row_on = true;
     if (kSparse) {

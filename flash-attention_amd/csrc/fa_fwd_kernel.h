@@ -149,7 +149,7 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
     const T* Vs = Ks + BN * D;
     buf ^= 1;
 
-    bool wave_work = true;
+    bool wave_work = mw < Lq;  // a wave whose 32 rows all lie past the sequence's end only helps with the staging
     if (kCausal && n0 > mw + 31) wave_work = false;  // every key of this tile is above the wave's diagonal
     bool row_on = true;
     if (kSparse) {
