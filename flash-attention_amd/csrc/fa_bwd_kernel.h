@@ -54,7 +54,7 @@ struct BwdCfg {
 };
 
 template <typename T, int D, bool kCausal, bool kDropout, bool kSparse>
-__global__ void __launch_bounds__(256, (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 3 : (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
   using Cfg = BwdCfg<T, D>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
@@ -359,7 +359,7 @@ struct DqCfg {
 };
 
 template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse>
-__global__ void __launch_bounds__(256, 2) fa_bwd_dq_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq_kernel(const BwdParams p) {
   using Cfg = DqCfg<T, D, BN>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
