@@ -54,7 +54,7 @@ struct BwdCfg {
 };
 
 template <typename T, int D, bool kCausal, bool kDropout, bool kSparse>
-__global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 3 : (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
   using Cfg = BwdCfg<T, D>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
