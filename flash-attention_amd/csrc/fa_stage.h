@@ -113,11 +113,15 @@ struct TilePairStager {
       for (int i = 0; i < NI; i++) dma16(tb + i * RPI * rsb, src_off[i % NOFF], lds + dst0 + i * 1024);
     } else {
       const char* const tb = base + (int64_t)first_row * rsb;
+      // The opaque copies keep this rarely taken path's per-lane arithmetic inside it: hoisted out of the caller's main
+      // loop (it is loop invariant) it would occupy, or spill, a dozen registers for the whole kernel.
+      int rlv = rl, pchv = pch;
+      asm volatile("" : "+v"(rlv), "+v"(pchv));
 #pragma unroll
       for (int i = 0; i < NI; i++) {
-        const int r = row0 + i * RPI + rl;
+        const int r = row0 + i * RPI + rlv;
         const int rc = first_row + r < n_rows ? r : n_rows - 1 - first_row;
-        dma16(tb, (uint32_t)(rc * rsb) + 16u * (uint32_t)(pch ^ swz(r)), lds + dst0 + i * 1024);
+        dma16(tb, (uint32_t)(rc * rsb) + 16u * (uint32_t)(pchv ^ swz(r)), lds + dst0 + i * 1024);
       }
     }
   }
