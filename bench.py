@@ -209,8 +209,8 @@ def main():
                      "frac": round(bwd_kernel_tflops / MFMA_PEAK_TFLOPS, 4),
                      "avg_launch_ms": round(t["bwd_main_kernel_ms"], 4),
                      # HBM bytes per launch from rocprofv3 FETCH_SIZE x2.00 + WRITE_SIZE x1.00 (scale factors from a
-                     # 256 MiB copy): 99 980 KiB read + 49 152 KiB written
-                     "traffic": 152.7e6},
+                     # 256 MiB copy): 101 461 KiB read + 50 688 KiB written
+                     "traffic": 155.8e6},
     }
     if not a.no_cpu:
         res["cpu_baseline"] = cpu_baseline(torch, B, H, D, N, a.cpu_budget)
