@@ -142,13 +142,16 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
     }
     return (uint32_t)(col_bits >> (4 * (mt & 15))) & 0xfu;
   };
-  auto tile_active = [&](int mt) -> bool {
-    if (!kSparse) return true;
-    return tile_rows_on(mt) != 0;
-  };
+  // First query tile >= mt with a set bit (mt_end if none), found with a count-trailing-zeros on the loaded word
   auto next_active = [&](int mt) -> int {
-    while (mt < mt_end && !tile_active(mt)) mt++;
-    return mt;
+    if (!kSparse) return mt;
+    while (mt < mt_end) {
+      tile_rows_on(mt);  // loads the word of mt if needed
+      const uint64_t rest = col_bits >> (4 * (mt & 15));  // bits 0..3: this tile's row blocks
+      if (rest & 0xf) break;
+      mt = rest ? mt + ((int)__builtin_ctzll(rest) >> 2) : (mt | 15) + 1;
+    }
+    return mt < mt_end ? mt : mt_end;
   };
 
   f32x16 acc_dk[DV / 32], acc_dv[DV / 32];
@@ -434,21 +437,27 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
   uint64_t tile_bits = 0, row_bits = 0;
   int bits_word = -1;
   const int qt_u = __builtin_amdgcn_readfirstlane(qt);
-  auto tile_active = [&](int it) -> bool {
-    if (!kSparse) return true;
-    const int cb = __builtin_amdgcn_readfirstlane((it * BN) >> 8);
-    if ((cb >> 6) != bits_word) {
-      bits_word = cb >> 6;
-      tile_bits = uniform64(p.sp.qbits[(int64_t)qt_u * p.sp.ncw + bits_word]);
-      const int rb = (qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1;
-      row_bits = p.sp.rbits[(int64_t)rb * p.sp.ncw + bits_word];
-    }
-    return (tile_bits >> (cb & 63)) & 1;
-  };
+  // First tile >= it whose 256-key block is active (ntiles if none): the bits of the loaded word are searched with a
+  // count-trailing-zeros, not tile by tile.
   bool row_on_next = true;  // this lane's row block attends the tile the last next_active() found
   auto next_active = [&](int it) -> int {
-    while (it < ntiles && !tile_active(it)) it++;
-    if (kSparse && it < ntiles) row_on_next = (row_bits >> (((it * BN) >> 8) & 63)) & 1;
+    if (!kSparse) return it;
+    constexpr int kTilesPerBlock = 256 / BN;
+    while (it < ntiles) {
+      const int cb = __builtin_amdgcn_readfirstlane((it * BN) >> 8);
+      if ((cb >> 6) != bits_word) {
+        bits_word = cb >> 6;
+        tile_bits = uniform64(p.sp.qbits[(int64_t)qt_u * p.sp.ncw + bits_word]);
+        const int rb = (qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1;
+        row_bits = p.sp.rbits[(int64_t)rb * p.sp.ncw + bits_word];
+      }
+      const uint64_t rest = tile_bits >> (cb & 63);  // bit 0: this tile's block
+      if (rest & 1) break;
+      // first tile of the next active block of this word, or of the next word
+      it = (rest ? cb + (int)__builtin_ctzll(rest) : (cb | 63) + 1) * kTilesPerBlock;
+    }
+    if (it > ntiles) it = ntiles;
+    if (it < ntiles) row_on_next = (row_bits >> (((it * BN) >> 8) & 63)) & 1;
     return it;
   };
 

@@ -97,21 +97,27 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
   uint64_t tile_bits = 0, row_bits = 0;
   int bits_word = -1;
   const int qt_u = __builtin_amdgcn_readfirstlane(qt);
-  auto tile_active = [&](int it) -> bool {
-    if (!kSparse) return true;
-    const int cb = __builtin_amdgcn_readfirstlane((it * BN) >> 8);
-    if ((cb >> 6) != bits_word) {
-      bits_word = cb >> 6;
-      tile_bits = uniform64(p.sp.qbits[(int64_t)qt_u * p.sp.ncw + bits_word]);
-      const int rb = (qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1;
-      row_bits = p.sp.rbits[(int64_t)rb * p.sp.ncw + bits_word];
-    }
-    return (tile_bits >> (cb & 63)) & 1;
-  };
+  // First tile >= it whose 256-key block is active (ntiles if none): the bits of the loaded word are searched with a
+  // count-trailing-zeros, not tile by tile.
   bool row_on_next = true;  // this lane's row block attends the tile the last next_active() found
   auto next_active = [&](int it) -> int {
-    while (it < ntiles && !tile_active(it)) it++;
-    if (kSparse && it < ntiles) row_on_next = (row_bits >> (((it * BN) >> 8) & 63)) & 1;
+    if (!kSparse) return it;
+    constexpr int kTilesPerBlock = 256 / BN;
+    while (it < ntiles) {
+      const int cb = __builtin_amdgcn_readfirstlane((it * BN) >> 8);
+      if ((cb >> 6) != bits_word) {
+        bits_word = cb >> 6;
+        tile_bits = uniform64(p.sp.qbits[(int64_t)qt_u * p.sp.ncw + bits_word]);
+        const int rb = (qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1;
+        row_bits = p.sp.rbits[(int64_t)rb * p.sp.ncw + bits_word];
+      }
+      const uint64_t rest = tile_bits >> (cb & 63);  // bit 0: this tile's block
+      if (rest & 1) break;
+      // first tile of the next active block of this word, or of the next word
+      it = (rest ? cb + (int)__builtin_ctzll(rest) : (cb | 63) + 1) * kTilesPerBlock;
+    }
+    if (it > ntiles) it = ntiles;
+    if (it < ntiles) row_on_next = (row_bits >> (((it * BN) >> 8) & 63)) & 1;
     return it;
   };
 
