@@ -219,6 +219,9 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
     if (kPipe) load_rows(0, aq[0], ad[0]);
 #pragma unroll
     for (int qb = 0; qb < BM / 32; qb++) {
+      // dropout: the two slabs' Philox streams are not to be interleaved by the scheduler (it would, for the sake of
+      // instruction-level parallelism, and need 70 more registers: one wave per SIMD fewer)
+      if (kDropout && !kPipe) __builtin_amdgcn_sched_barrier(0);
       bool rb_on[2] = {true, true};
       if (kSparse) {
         rb_on[0] = (rows_on >> (2 * qb)) & 1;
