@@ -1,0 +1,57 @@
+"""Build-time guard of the register budgets the kernels' speed depends on (CPU only: hipcc cross-compiles for gfx950).
+
+The d = 64 kernels are tuned to the register counts at which one more wave fits a SIMD (128 VGPRs: four waves, 168: three).
+One extra live register in a main loop silently costs a wave per SIMD or turns into scratch traffic, so the counts the
+compiler reports (-Rpass-analysis=kernel-resource-usage) are pinned here for the variants the headline workloads run.
+"""
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "flash-attention_amd"))
+import build as fa_build  # noqa: E402
+
+
+def _resources(src):
+    cmd = [fa_build.HIPCC] + fa_build.FLAGS + ["-Rpass-analysis=kernel-resource-usage", "-c",
+                                               os.path.join(fa_build.CSRC, src), "-o", os.devnull]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout[-2000:]
+    out, name = {}, None
+    for line in r.stdout.splitlines():
+        m = re.search(r"Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+            out[name] = {}
+            continue
+        m = re.search(r"remark:\s+([A-Za-z ]+?)(?: \[[^\]]*\])?: (\d+)", line)
+        if m and name:
+            out[name][m.group(1).strip()] = int(m.group(2))
+    return out
+
+
+def _pick(res, *parts):
+    hits = [v for k, v in res.items() if all(p in k for p in parts)]
+    assert len(hits) == 1, (parts, [k for k in res if parts[0] in k])
+    return hits[0]
+
+
+@pytest.mark.timeout(600)
+def test_d64_kernels_keep_their_waves_per_simd():
+    fwd = _resources("fa_fwd_d64.hip")
+    bwd = _resources("fa_bwd_d64.hip")
+    # <f16, 64, ..., causal, dropout, sparse> mangled as ...IDF16_Li64E...Lb{0,1}E x3
+    plain, causal, dropout = "Lb0ELb0ELb0E", "Lb1ELb0ELb0E", "Lb0ELb1ELb0E"
+    for flags, want in ((plain, 4), (causal, 4), (dropout, 3)):
+        k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags)
+        assert k["Occupancy"] >= want and k["VGPRs Spill"] == 0, ("forward", flags, k)
+    for flags, want in ((plain, 3), (causal, 3), (dropout, 3)):
+        k = _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", flags)
+        assert k["Occupancy"] >= want and k["VGPRs Spill"] == 0, ("dq", flags, k)
+    for flags, want, spill in ((plain, 3, 2), (causal, 3, 2), (dropout, 2, 0)):
+        k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", flags)
+        assert k["Occupancy"] >= want and k["VGPRs Spill"] <= spill, ("dkdv", flags, k)
