@@ -14,6 +14,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "flash_attn", "libflash_attn_gfx950.so")
+# a caller of the C ABI without Python or torch (examples/c_abi_caller.cpp), run by the GPU tests
+EXAMPLE_SRC = os.path.join(HERE, "examples", "c_abi_caller.cpp")
+EXAMPLE_BIN = os.path.join(OBJ_DIR, "c_abi_caller")
+INCLUDE_DIR = os.path.join(os.path.dirname(HERE), "include")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -52,6 +56,11 @@ def build(jobs=8, verbose=False):
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stdout)
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-I", INCLUDE_DIR, EXAMPLE_SRC, "-L", os.path.dirname(LIB_PATH),
+           "-lflash_attn_gfx950", "-Wl,-rpath,$ORIGIN/../flash_attn", "-o", EXAMPLE_BIN]
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("building %s failed:\n%s" % (EXAMPLE_SRC, r.stdout))
     return LIB_PATH
 
 

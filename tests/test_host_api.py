@@ -321,3 +321,20 @@ def test_rows_and_rotary_argument_checks(lib):
     assert lib.fa_rotary(ctypes.byref(r)) == -1 and b"null" in lib.fa_last_error()
     r.n_rows = 0
     assert lib.fa_rotary(ctypes.byref(r)) == 0
+
+
+def test_header_is_plain_c(tmp_path):
+    """include/flash_attn_gfx950.h must be usable from C (the boundary a cgo / JNI / ctypes binding sees): it compiles as
+    C99 with warnings as errors, and every declared entry point can be named."""
+    import subprocess
+    from flash_attn import flash_attn_gfx950 as be
+    src = tmp_path / "use_header.c"
+    names = [n for n in be.EXPORTED_SYMBOLS]
+    src.write_text('#include "flash_attn_gfx950.h"\n'
+                   "typedef void (*entry_t)(void);\n"
+                   "entry_t entry_points[] = {" + ", ".join("(entry_t)%s" % n for n in names) + "};\n"
+                   "int sizes[] = {(int)sizeof(fa_fwd_args), (int)sizeof(fa_bwd_args), (int)sizeof(fa_rotary_args)};\n")
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only",
+                        "-I", os.path.join(ROOT, "include"), str(src)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert r.returncode == 0, r.stdout
+

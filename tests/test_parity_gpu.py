@@ -948,3 +948,16 @@ def test_forward_and_backward_replay_from_a_hip_graph():
         for b, L in enumerate(lens):
             assert torch.equal(got[1][b, :, :L], lse_e[b, :, :L]), rep
         assert torch.equal(got[2], dqkv), rep
+
+
+def test_c_abi_caller_without_python_or_torch():
+    """examples/c_abi_caller.cpp (built by build.py): hipMalloc'ed buffers, the header's structs, one forward and backward of
+    a ragged causal batch, checked inside the program against the closed form in double precision."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "flash-attention_amd", "build", "c_abi_caller")
+    assert os.path.exists(exe), "run `python flash-attention_amd/build.py` first"
+    r = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    print(r.stdout)
+    assert r.returncode == 0 and "PASS" in r.stdout, r.stdout
+
