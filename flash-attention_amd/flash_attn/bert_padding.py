@@ -13,6 +13,9 @@ import torch.nn.functional as F
 from . import flash_attn_gfx950 as _backend
 
 
+# The device of the INPUT decides, never the availability of the library: a GPU tensor always goes to the HIP kernels
+# (and raises if the library is not built); only tensors that live in host memory, which no GPU kernel could read,
+# are indexed by torch.
 def _gather(input, indices):
     if input.is_cuda:
         return _backend.gather_rows(input, indices)

@@ -83,7 +83,7 @@ class FlashMHA(nn.Module):
         qkv = self.Wqkv(x).reshape(b, s, 3, self.num_heads, self.head_dim)
         if self.use_rotary_emb == "1d" and qkv.is_cuda and qkv.dtype in (torch.float16, torch.bfloat16):
             qkv = self.rotary_emb.rotate_qkv_(qkv)  # q and k rotated in place by one kernel
-        elif self.use_rotary_emb:
+        elif self.use_rotary_emb:  # "2d" (no fused kernel for it): the reference's elementwise formulation, on the GPU
             query, key, value = qkv.unbind(dim=2)
             query, key = self.rotary_emb(query, key, seq_dimension=-3)
             qkv = torch.stack([query, key, value], dim=2)
