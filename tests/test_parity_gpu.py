@@ -480,6 +480,45 @@ def test_blocksparse_more_than_64_key_blocks():
     check_against_oracle({"out": out, "dq": dq, "dk": dk, "dv": dv}, ref, half, torch.float16, what="blocksparse 66 key blocks")
 
 
+def test_blocksparse_random_layouts_sweep():
+    """Ten seeded random block-sparse cases: densities from 5 % to 90 % (with and without the diagonal band), ragged
+    lengths up to 2100 (several activity words per key block on the backward side), every head dim, both dtypes, dropout."""
+    from flash_attn.flash_blocksparse_attn_interface import flash_blocksparse_attn_func
+    from flash_attn import flash_attn_gfx950 as be
+    rng = np.random.default_rng(31)
+    for case in range(10):
+        D = int(rng.choice([16, 32, 64, 128]))
+        dtype = torch.float16 if rng.integers(2) else torch.bfloat16
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 3))
+        N = int(rng.choice([100, 300, 520, 1100, 2100]))
+        lens = [N] + [int(x) for x in rng.integers(max(1, N // 3), N + 1, B - 1)]
+        dens = float(rng.choice([0.05, 0.2, 0.5, 0.9]))
+        p = float(rng.choice([0.0, 0.0, 0.2]))
+        sq_r, sk_r = be.round_seqlens(D, N, N, True)
+        layout = torch.rand(sq_r // 16, sk_r // 256, generator=torch.Generator().manual_seed(case)) < dens
+        if rng.integers(2):
+            layout |= (torch.arange(sq_r // 16)[:, None] // 16) == torch.arange(sk_r // 256)[None, :]
+        what = "case %d: D=%d %s B=%d H=%d lens=%s density %.2f p=%.1f" % (case, D, dtype, B, H, lens, dens, p)
+        print(what, flush=True)
+        q, k, v, do = _inputs(lens, lens, H, D, dtype, 3000 + case)
+        cu = _cu(lens, "cpu")
+        qkv = torch.stack([q, k, v], 1).cuda().requires_grad_()
+        torch.manual_seed(case)
+        seed, offset = _gen_state()
+        ctx = flash_blocksparse_attn_func(qkv, cu.cuda(), layout.cuda(), p, N)
+        ctx.backward(do.cuda())
+        torch.cuda.synchronize()
+        masks = None
+        if p > 0:
+            masks = [torch.tensor(np.stack([orc.dropout_keep_mask(seed, offset, b * H + h, L, L, p) for h in range(H)]))
+                     for b, L in enumerate(lens)]
+        ref = orc.varlen_attention(q, k, v, cu, cu, None, False, p_dropout=p, keep_mask=masks, layout=layout.numpy(), dout=do)
+        half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu.tolist(), cu.tolist(), D ** -0.5, False, masks, p,
+                              layout=layout.numpy(), dout=do.cuda())
+        ours = {"out": ctx.detach(), "dq": qkv.grad[:, 0], "dk": qkv.grad[:, 1], "dv": qkv.grad[:, 2]}
+        check_against_oracle(ours, ref, half, dtype, what=what)
+
+
 def test_blocksparse_full_layout_equals_dense():
     from flash_attn.flash_blocksparse_attn_interface import flash_blocksparse_attn_func
     from flash_attn.flash_attn_interface import flash_attn_unpadded_qkvpacked_func
