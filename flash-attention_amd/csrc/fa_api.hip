@@ -249,7 +249,9 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
   const float p_keep = 1.f - a->p_dropout;
 
   const SparseLayout sl = sparse_layout(r);
-  const size_t need = sparse ? sl.bytes : 0;  // the dense backward needs no scratch: no dq_tmp (fmha_api.cpp:403-404)
+  // the dense backward needs no scratch: no dq_tmp (fmha_api.cpp:403-404); it uses some, if offered, to split the keys of
+  // a lone query tile over several workgroups (see below)
+  const size_t need = sparse ? sl.bytes : 0;
   if (need > 0 && (!a->workspace || a->workspace_bytes < need))
     return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need, a->workspace_bytes);
   FA_REQUIRE(need == 0 || aligned16(a->workspace), "workspace must be 16-byte aligned");
@@ -292,7 +294,16 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
   p.keep_thr = (uint32_t)std::floor(p_keep * 65535.0);
   p.pk = make_key(a->philox_seed, a->philox_offset);
 
+  // short query side, long key side: the dQ kernel would walk all keys with one workgroup per (batch, head)
+  const SplitPlan sp = split_plan(a->batch, a->nheads, a->head_dim, a->total_q, a->max_seqlen_q, a->max_seqlen_k, r.sq_r,
+                                  a->is_causal != 0, sparse);
+  const bool split = sp.n_splits > 1 && a->workspace && a->workspace_bytes >= sp.o_bytes && aligned16(a->workspace);
+  if (split) {
+    p.n_splits = sp.n_splits;
+    p.dq_part = reinterpret_cast<float*>(a->workspace);
+  }
   FA_LAUNCH(fa::launch_bwd(p, 0, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));  // dQ, softmax_d
+  if (split) FA_LAUNCH(fa::launch_dq_combine(p, a->dtype, a->head_dim, stream));
   if (a->ev_main_start) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(a->ev_main_start), stream));
   FA_LAUNCH(fa::launch_bwd(p, 1, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));  // dK, dV
   if (a->ev_main_stop) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(a->ev_main_stop), stream));
@@ -318,9 +329,11 @@ size_t fa_fwd_workspace_bytes(const fa_fwd_args* a) {
 
 size_t fa_bwd_workspace_bytes(const fa_bwd_args* a) {
   if (!a) return 0;
-  size_t n = 0;
-  if (a->blockmask) n += sparse_layout(round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, true)).bytes;
-  return n;
+  if (a->blockmask) return sparse_layout(round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, true)).bytes;
+  // optional: partial dQ of the key-split dQ kernel (same plan as the forward's; o_bytes is n_splits fp32 copies of dq)
+  const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, false);
+  return split_plan(a->batch, a->nheads, a->head_dim, a->total_q, a->max_seqlen_q, a->max_seqlen_k, r.sq_r,
+                    a->is_causal != 0, false).o_bytes;
 }
 
 void fa_round_seqlens(int32_t head_dim, int32_t max_seqlen_q, int32_t max_seqlen_k, int32_t blocksparse,

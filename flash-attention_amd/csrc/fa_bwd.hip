@@ -23,4 +23,34 @@ hipError_t launch_bwd(const BwdParams& p, int which, int dtype, int head_dim, bo
   }
 }
 
+// Adds up the partial dQ of a key-split backward (BwdParams::dq_part) and writes dq in the tensor dtype.
+// One thread per (batch, head, query row, 4 columns).
+template <typename T>
+__global__ void __launch_bounds__(256) dq_combine_kernel(const BwdParams p, int D) {
+  const int cpr = D / 4;
+  const int64_t total = (int64_t)p.B * p.H * p.max_sq * cpr;
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= total) return;
+  const int ch = (int)(t % cpr);
+  const int row = (int)((t / cpr) % p.max_sq);
+  const int h = (int)((t / cpr / p.max_sq) % p.H);
+  const int b = (int)(t / cpr / p.max_sq / p.H);
+  int q_begin, Lq;
+  if (!seq_extent(p.cu_q, b, p.total_q, p.max_sq, &q_begin, &Lq) || row >= Lq) return;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < p.n_splits; s++)
+    acc = acc + *reinterpret_cast<const f32x4*>(p.dq_part + (((int64_t)s * p.total_q + q_begin + row) * p.H + h) * D + ch * 4);
+  T* op = reinterpret_cast<T*>(p.dq) + (int64_t)(q_begin + row) * p.dq_rs + (int64_t)h * p.dq_hs + ch * 4;
+  *reinterpret_cast<typename Elem<T>::vec4*>(op) = cvt4<T>(acc);
+}
+
+hipError_t launch_dq_combine(const BwdParams& p, int dtype, int head_dim, hipStream_t stream) {
+  const int64_t total = (int64_t)p.B * p.H * p.max_sq * (head_dim / 4);
+  if (total == 0) return hipSuccess;
+  const unsigned grid = (unsigned)((total + 255) / 256);
+  if (dtype == 0) hipLaunchKernelGGL(dq_combine_kernel<_Float16>, dim3(grid), dim3(256), 0, stream, p, head_dim);
+  else hipLaunchKernelGGL(dq_combine_kernel<__bf16>, dim3(grid), dim3(256), 0, stream, p, head_dim);
+  return hipGetLastError();
+}
+
 }  // namespace fa

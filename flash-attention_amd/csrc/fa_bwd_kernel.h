@@ -374,7 +374,10 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
 
   int bh, rank;
-  if (!map_tile<kCausal>(blockIdx.x, p.nq_tiles, p.B * p.H, &bh, &rank)) return;
+  const int n_splits = p.n_splits > 1 ? p.n_splits : 1;  // key splits per query tile (see BwdParams)
+  if (!map_tile<kCausal>(blockIdx.x, p.nq_tiles * n_splits, p.B * p.H, &bh, &rank)) return;
+  const int split = rank % n_splits;
+  rank /= n_splits;
   const int qt = kCausal ? p.nq_tiles - 1 - rank : rank;
   const int b = bh / p.H, h = bh % p.H;
 
@@ -416,7 +419,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
       const float x = p.lse[((int64_t)b * p.H + h) * p.lse_stride + qrow];
       lse2 = (x == -INFINITY) ? INFINITY : x * kLog2e;
       dkv = dsum;
-      if (hf == 0) p.dsoftmax[((int64_t)b * p.H + h) * p.sq_r + qrow] = dsum;
+      if (hf == 0 && split == 0) p.dsoftmax[((int64_t)b * p.H + h) * p.sq_r + qrow] = dsum;
     }
   }
   // For d <= 64 the dP^T accumulator starts from -Dk of this lane's query row (16 registers that save 16 subtractions
@@ -427,7 +430,9 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
   for (int r = 0; r < 16; r++) negd[r] = kInitNegD ? -dkv : 0.f;
   int n_end = Lk;
   if (kCausal) n_end = n_end < m0 + BM ? n_end : m0 + BM;
-  const int ntiles = (n_end + BN - 1) / BN;
+  const int ntiles_all = (n_end + BN - 1) / BN;
+  const int tile0 = (int)((int64_t)split * ntiles_all / n_splits);  // this workgroup's share of the key tiles
+  const int ntiles = (int)((int64_t)(split + 1) * ntiles_all / n_splits);
 
   // ---- K/V staging: global -> LDS without passing through registers (waves 0,1 fetch K tiles, waves 2,3 V tiles).
   // Keys past the end re-read the last key: their P is masked to 0 below, so they add 0 * finite to dQ.
@@ -485,7 +490,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
   }
   int buf = 0;
 
-  int it = next_active(0);
+  int it = next_active(tile0);
   bool row_on_cur = row_on_next;
   if (it < ntiles) stage(it, 0);
   while (it < ntiles) {
@@ -567,6 +572,24 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
 
   // ---- epilogue: dQ = dQ^T acc * scale / keep, transposed through LDS, coalesced stores
   const float f = p.scale * p.rp_keep;
+  if (p.n_splits > 1) {  // partial sum of this key split, fp32, added up by dq_combine_kernel
+    if (qrow < Lq) {
+      float* op = p.dq_part + (((int64_t)split * p.total_q + q_begin + qrow) * p.H + h) * D;
+#pragma unroll
+      for (int db = 0; db < DV / 32; db++)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          const int d0 = db * 32 + g4 * 8 + hf * 4;
+          if (d0 < D) {
+            f32x4 x;
+#pragma unroll
+            for (int i = 0; i < 4; i++) x[i] = acc[db][g4 * 4 + i] * f;
+            *reinterpret_cast<f32x4*>(op + d0) = x;
+          }
+        }
+    }
+    return;
+  }
   __syncthreads();
   constexpr int OS = Cfg::OS;
   T* Os = reinterpret_cast<T*>(lds_raw) + wave * 32 * OS;

@@ -100,6 +100,10 @@ struct BwdParams {
   uint32_t keep_thr;
   PhiloxKey pk;
   SparseMaps sp;
+  // Key-split dQ (one query tile, many keys; see FwdParams): split s of n_splits walks its share of the key tiles and
+  // writes its scaled fp32 partial dQ to dq_part [n_splits, total_q, H, d]; dq_combine_kernel sums them into dq.
+  int n_splits;
+  float* dq_part;
 };
 
 // Sequence extent of batch entry b, clamped so that a cu_seqlens array that disagrees with the declared
@@ -154,6 +158,7 @@ inline int tile_grid(bool tile_major, int tiles_per_bh, int BH) {
 hipError_t launch_fwd(const FwdParams& p, int dtype, int head_dim, bool causal, bool dropout, bool sparse,
                       hipStream_t stream);
 hipError_t launch_fwd_combine(const FwdParams& p, int dtype, int head_dim, hipStream_t stream);
+hipError_t launch_dq_combine(const BwdParams& p, int dtype, int head_dim, hipStream_t stream);
 // fa_rotary: rotate the first n_rotated of n_parts (row, part, head, head_dim) slices, copy the others
 struct RotaryParams {
   const void* src;

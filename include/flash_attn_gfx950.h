@@ -127,13 +127,14 @@ int fa_fwd_block(const fa_fwd_args* args);
 /* replaces flash_attn_cuda.bwd_block -> mha_bwd_block, csrc/flash_attn/fmha_api.cpp:575-718 */
 int fa_bwd_block(const fa_bwd_args* args);
 
-/* Scratch the caller provides.  The dense backward needs none and the dense forward needs none to be correct
+/* Scratch the caller provides.  The dense forward and backward need none to be correct
  * (there is no o_tmp / dq_tmp, fmha_api.cpp:247,403-404).  The block-sparse paths need room for their block activity
  * maps (an error without it).  For a dense, non-causal forward with few query rows and many keys (max_seqlen_q <= 128,
  * batch * nheads < 128, max_seqlen_k >= 512: decoding and cross-attention shapes) fa_fwd_workspace_bytes() returns the size of the
  * partial results of a key-split pass: if `workspace` holds that much, fa_fwd shares the keys of each query tile
- * among several workgroups and merges their results; if not, it runs the single pass.  Only shapes, is_causal and
- * blockmask != NULL are read. */
+ * among several workgroups and merges their results; if not, it runs the single pass.  fa_bwd_workspace_bytes() does the
+ * same for the dQ kernel of such shapes (fp32 partial dQ per key split).  Only shapes, is_causal and blockmask != NULL
+ * are read. */
 size_t fa_fwd_workspace_bytes(const fa_fwd_args* args);
 size_t fa_bwd_workspace_bytes(const fa_bwd_args* args);
 

@@ -1005,3 +1005,64 @@ def test_c_abi_caller_without_python_or_torch():
     print(r.stdout)
     assert r.returncode == 0 and "PASS" in r.stdout, r.stdout
 
+
+
+@pytest.mark.parametrize("lens_q,lens_k,D,p", [
+    ([1, 1], [2048, 1500], 64, 0.0),
+    ([16, 5, 128], [1024, 4000, 513], 64, 0.0),
+    ([100], [3000], 128, 0.0),
+    ([3, 40], [1300, 2100], 32, 0.15),
+])
+def test_key_split_backward(lens_q, lens_k, D, p):
+    """fa_bwd with the scratch fa_bwd_workspace_bytes() asks for splits the keys of the dQ kernel's lone query tile over
+    several workgroups (fp32 partial dQ, summed by a second launch); dq must match the oracle and the unsplit kernel
+    (same call without workspace), dk and dv must be bitwise those of the unsplit call."""
+    from flash_attn import flash_attn_gfx950 as be
+    lib = be.load_library()
+    H, dtype = 3, torch.float16
+    q, k, v, do = _inputs(lens_q, lens_k, H, D, dtype, seed=sum(lens_k) + 1)
+    cu_q, cu_k = _cu(lens_q, "cuda"), _cu(lens_k, "cuda")
+    qd, kd, vd, dod = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    torch.manual_seed(99)
+    seed, offset = _gen_state()  # the pair the forward below reads from the default generator (and then advances)
+    out, lse = be.fwd(qd, kd, vd, cu_q, cu_k, max(lens_q), max(lens_k), p, D ** -0.5, False, False, False, None)
+    sq_r, _ = be.round_seqlens(D, max(lens_q), max(lens_k))
+
+    def call(with_ws):
+        dq, dk, dv = torch.zeros_like(qd), torch.zeros_like(kd), torch.zeros_like(vd)
+        sd = torch.zeros(len(lens_q), H, sq_r, device="cuda")
+        a = be.BwdArgs()
+        a.struct_bytes = ctypes.sizeof(a)
+        a.dtype = 0
+        a.dout, a.q, a.k, a.v, a.out, a.softmax_lse = (dod.data_ptr(), qd.data_ptr(), kd.data_ptr(), vd.data_ptr(),
+                                                       out.data_ptr(), lse.data_ptr())
+        a.dq, a.dk, a.dv, a.softmax_d = dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), sd.data_ptr()
+        a.cu_seqlens_q, a.cu_seqlens_k = cu_q.data_ptr(), cu_k.data_ptr()
+        for name in ("do", "q", "k", "v", "o", "dq", "dk", "dv"):
+            setattr(a, name + "_row_stride", H * D)
+            setattr(a, name + "_head_stride", D)
+        a.lse_seq_stride = lse.shape[2]
+        a.batch, a.nheads, a.head_dim = len(lens_q), H, D
+        a.total_q, a.total_k, a.max_seqlen_q, a.max_seqlen_k = sum(lens_q), sum(lens_k), max(lens_q), max(lens_k)
+        a.p_dropout, a.softmax_scale = p, D ** -0.5
+        a.philox_seed, a.philox_offset = seed, offset
+        need = lib.fa_bwd_workspace_bytes(ctypes.byref(a))
+        assert need > 0
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda") if with_ws else None
+        a.workspace, a.workspace_bytes = (ws.data_ptr(), need) if with_ws else (None, 0)
+        assert lib.fa_bwd(ctypes.byref(a)) == 0, lib.fa_last_error()
+        torch.cuda.synchronize()
+        return dq.cpu(), dk.cpu(), dv.cpu(), sd.cpu()
+
+    dq_s, dk_s, dv_s, sd_s = call(True)
+    dq_1, dk_1, dv_1, sd_1 = call(False)
+    assert torch.equal(dk_s, dk_1) and torch.equal(dv_s, dv_1) and torch.equal(sd_s, sd_1)
+    masks = None
+    if p > 0:
+        masks = [torch.tensor(np.stack([orc.dropout_keep_mask(seed, offset, b * H + h, lq, lk, p) for h in range(H)]))
+                 for b, (lq, lk) in enumerate(zip(lens_q, lens_k))]
+    ref = orc.varlen_attention(q, k, v, cu_q.cpu(), cu_k.cpu(), D ** -0.5, False, p_dropout=p, keep_mask=masks, dout=do)
+    half = half_attention(qd, kd, vd, cu_q.tolist(), cu_k.tolist(), D ** -0.5, False, masks, p, dout=dod)
+    for got in (dq_s, dq_1):
+        check_against_oracle({"dq": got}, ref, half, dtype, names=("dq",), what="key-split backward")
+    assert (dq_s.float() - dq_1.float()).abs().max() <= 2.0 ** -10 * max(1.0, ref["dq"].abs().max().item())
