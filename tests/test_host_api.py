@@ -296,6 +296,17 @@ def test_key_split_workspace_plan(lib):
     assert lib.fa_fwd_workspace_bytes(ctypes.byref(a)) == 0
     a.max_seqlen_k, a.batch, a.total_q = 2048, 64, 64          # enough (batch, head) pairs to fill the chip
     assert lib.fa_fwd_workspace_bytes(ctypes.byref(a)) == 0
+    # the backward asks for the fp32 partial dQ of the same plan (8 splits x 8 rows x 12 heads x 64), and for nothing
+    # where the forward asks for nothing
+    g = be.BwdArgs()
+    g.struct_bytes = ctypes.sizeof(g)
+    g.batch, g.nheads, g.head_dim = 8, 12, 64
+    g.total_q, g.total_k, g.max_seqlen_q, g.max_seqlen_k = 8, 8 * 2048, 1, 2048
+    assert lib.fa_bwd_workspace_bytes(ctypes.byref(g)) == 8 * 8 * 12 * 64 * 4
+    g.is_causal = 1
+    assert lib.fa_bwd_workspace_bytes(ctypes.byref(g)) == 0
+    g.is_causal, g.max_seqlen_q, g.total_q = 0, 2048, 8 * 2048
+    assert lib.fa_bwd_workspace_bytes(ctypes.byref(g)) == 0
 
 
 def test_rows_and_rotary_argument_checks(lib):
