@@ -44,23 +44,21 @@ __global__ void __launch_bounds__(256) invert_index_kernel(const int64_t* __rest
   if (d >= 0 && d < n_dst) inv[d] = (int32_t)i;
 }
 
-__global__ void __launch_bounds__(256) fill_i32_kernel(int32_t* p, int64_t n, int32_t v) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < n) p[i] = v;
-}
-
-// dst[r, :] = inv[r] >= 0 ? src[inv[r], :] : 0 for every r < n_dst
+// dst[r, :] = src[s, :] if some idx[s] == r, else 0, for every r < n_dst.  inv is NOT initialised before
+// invert_index_kernel writes the entries that have a source: an entry is trusted only if it points back (idx[inv[r]] == r),
+// which stale scratch contents can satisfy only by naming the right source row, the indices being unique.
 template <int V>
 __global__ void __launch_bounds__(256) scatter_rows_kernel(const unsigned char* __restrict__ src, unsigned char* __restrict__ dst,
-                                                           const int32_t* __restrict__ inv, int64_t n_dst, int64_t cpr,
-                                                           int64_t src_stride, int64_t dst_stride) {
+                                                           const int32_t* __restrict__ inv, const int64_t* __restrict__ idx,
+                                                           int64_t n_idx, int64_t n_dst, int64_t cpr, int64_t src_stride,
+                                                           int64_t dst_stride) {
   typedef typename Chunk<V>::type C;
   const int64_t total = n_dst * cpr;
   for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (int64_t)gridDim.x * 256) {
     const int64_t row = t / cpr, ch = t - row * cpr;
-    const int32_t s = inv[row];
+    const int64_t s = inv[row];
     C v = C{};
-    if (s >= 0) v = *reinterpret_cast<const C*>(src + (int64_t)s * src_stride + ch * V);
+    if (s >= 0 && s < n_idx && idx[s] == row) v = *reinterpret_cast<const C*>(src + s * src_stride + ch * V);
     *reinterpret_cast<C*>(dst + row * dst_stride + ch * V) = v;
   }
 }
@@ -98,13 +96,12 @@ hipError_t launch_scatter_rows(const void* src, void* dst, const int64_t* idx, i
                                int64_t row_bytes, int64_t src_stride, int64_t dst_stride, int vec, int32_t* inv,
                                hipStream_t stream) {
   if (n_dst == 0 || row_bytes == 0) return hipSuccess;
-  hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)((n_dst + 255) / 256)), dim3(256), 0, stream, inv, n_dst, -1);
   if (n_idx > 0)
     hipLaunchKernelGGL(invert_index_kernel, dim3((unsigned)((n_idx + 255) / 256)), dim3(256), 0, stream, idx, n_idx, n_dst, inv);
   const int64_t cpr = row_bytes / vec;
   const unsigned grid = grid_for(n_dst * cpr);
   FA_DISPATCH_V(vec, scatter_rows_kernel, reinterpret_cast<const unsigned char*>(src), reinterpret_cast<unsigned char*>(dst),
-                inv, n_dst, cpr, src_stride, dst_stride)
+                inv, idx, n_idx, n_dst, cpr, src_stride, dst_stride)
   return hipGetLastError();
 }
 

@@ -749,18 +749,24 @@ def test_rows_raw_c_abi_unsorted_strided_and_errors():
     n_dst = 64
     out_base = torch.full((n_dst, 2 * dim), 5.0, dtype=torch.float16, device="cuda")
     out = out_base[:, dim:]
-    ws = torch.empty(n_dst, dtype=torch.int32, device="cuda")
     vals = torch.randn(31, dim, generator=g).half().cuda()
     sidx = torch.randperm(n_dst, generator=g)[:31]
     sidx_bad = sidx.clone()
     sidx_bad[0] = n_dst                                   # ignored
-    rc = lib.fa_scatter_rows(vals.data_ptr(), out.data_ptr(), sidx_bad.cuda().data_ptr(), 31, n_dst, dim * 2, dim * 2,
-                             out.stride(0) * 2, ws.data_ptr(), n_dst * 4, None)
-    assert rc == 0, lib.fa_last_error()
-    torch.cuda.synchronize()
     want = torch.zeros(n_dst, dim, dtype=torch.float16)
     want[sidx[1:]] = vals.cpu()[1:]
-    assert torch.equal(out.cpu(), want)
+    # the workspace arrives with whatever the last user left in it: plausible source rows, the entries of an earlier
+    # call with other indices, values far out of range
+    stale = [torch.arange(n_dst) % 31, torch.randperm(n_dst, generator=g) % 31, torch.full((n_dst,), 2 ** 31 - 1),
+             torch.full((n_dst,), -2 ** 31), torch.zeros(n_dst)]
+    for fill in stale:
+        ws = fill.to(torch.int32).cuda()
+        out.fill_(5.0)
+        rc = lib.fa_scatter_rows(vals.data_ptr(), out.data_ptr(), sidx_bad.cuda().data_ptr(), 31, n_dst, dim * 2, dim * 2,
+                                 out.stride(0) * 2, ws.data_ptr(), n_dst * 4, None)
+        assert rc == 0, lib.fa_last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(out.cpu(), want)
     assert torch.equal(out_base[:, :dim].cpu(), torch.full((n_dst, dim), 5.0, dtype=torch.float16))  # neighbours untouched
     # empty and error cases
     assert lib.fa_gather_rows(None, None, None, 0, 0, 16, 16, 16, None) == 0
