@@ -156,7 +156,6 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
                  stride_ok(a->k_head_stride) && stride_ok(a->v_row_stride) && stride_ok(a->v_head_stride) &&
                  stride_ok(a->o_row_stride) && stride_ok(a->o_head_stride),
              "row and head strides must be multiples of 8 elements in [0, 2^24)");
-  FA_REQUIRE(!(sparse && a->is_causal), "block-sparse attention does not support causal");  // interface.py:21
 
   const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, sparse);
   hipStream_t stream = reinterpret_cast<hipStream_t>(a->stream);
@@ -240,7 +239,6 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
                              a->dq_row_stride, a->dq_head_stride, a->dk_row_stride, a->dk_head_stride, a->dv_row_stride,
                              a->dv_head_stride};
   for (int64_t s : strides) FA_REQUIRE(stride_ok(s), "row and head strides must be multiples of 8 elements in [0, 2^24)");
-  FA_REQUIRE(!(sparse && a->is_causal), "block-sparse attention does not support causal");
 
   const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, sparse);
   FA_REQUIRE(a->lse_seq_stride >= a->max_seqlen_q, "softmax_lse is shorter than max_seqlen_q");

@@ -14,12 +14,17 @@ from . import flash_attn_gfx950 as _backend
 def convert_blockmask(blockmask, causal):
     """0/1 layout (row, col) -> int32 (col, row).  Row c of the result lists the nonzero row-block indices of column
     c in ascending order, padded with -1.  Each index is multiplied by 4; bit 0 marks the first nonzero of its
-    layout row, bit 1 the last nonzero of its layout row."""
-    assert not causal
+    layout row, bit 1 the last nonzero of its layout row.
+
+    causal=True (the reference asserts against it, :21; the kernels here apply the element-wise causal mask on top of the
+    block list): blocks that lie wholly above the diagonal are dropped from the lists first, so that the first/last
+    marks describe the blocks that are actually computed."""
     nz = blockmask != 0
     nrow, ncol = nz.shape
     dev = nz.device
     cols = torch.arange(ncol, device=dev)
+    if causal:  # block (r, c) holds a key <= query iff its first key 256 c is <= its last row 16 r + 15
+        nz = nz & (256 * cols[None, :] <= 16 * torch.arange(nrow, device=dev)[:, None] + 15)
     big = ncol + 1
     first_col = torch.where(nz, cols, torch.full_like(cols, big)).min(dim=1).values   # (nrow,)
     last_col = torch.where(nz, cols, torch.full_like(cols, -1)).max(dim=1).values

@@ -122,7 +122,9 @@ int fa_fwd(const fa_fwd_args* args);
 /* replaces flash_attn_cuda.bwd -> mha_bwd, csrc/flash_attn/fmha_api.cpp:302-449 */
 int fa_bwd(const fa_bwd_args* args);
 /* replaces flash_attn_cuda.fwd_block -> mha_fwd_block, csrc/flash_attn/fmha_api.cpp:451-573
- * (args->blockmask must be non-NULL) */
+ * (args->blockmask must be non-NULL).  is_causal may be set together with a blockmask, here and in fa_bwd_block: a score
+ * counts iff its block is listed AND key <= query; blocks that lie wholly above the diagonal may be listed or not.  The
+ * reference's kernels take the flag too, but its Python refuses it (flash_blocksparse_attn_interface.py:21). */
 int fa_fwd_block(const fa_fwd_args* args);
 /* replaces flash_attn_cuda.bwd_block -> mha_bwd_block, csrc/flash_attn/fmha_api.cpp:575-718 */
 int fa_bwd_block(const fa_bwd_args* args);

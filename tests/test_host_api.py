@@ -90,15 +90,16 @@ def test_null_pointers_and_alignment_are_errors_not_crashes(lib):
     assert lib.fa_fwd(None) == -1
 
 
-def test_block_sparse_needs_workspace_and_rejects_causal(lib):
+def test_block_sparse_needs_workspace_also_when_causal(lib):
     from flash_attn import flash_attn_gfx950 as be
     a = _valid_fwd_args(be)
     for f in ("q", "k", "v", "o", "softmax_lse", "cu_seqlens_q", "cu_seqlens_k", "blockmask"):
         setattr(a, f, 0x1000)
     assert lib.fa_fwd_workspace_bytes(ctypes.byref(a)) > 0
     assert lib.fa_fwd_block(ctypes.byref(a)) == -2 and b"workspace" in lib.fa_last_error()
-    a.is_causal = 1
-    assert lib.fa_fwd_block(ctypes.byref(a)) == -1 and b"causal" in lib.fa_last_error()
+    a.is_causal = 1  # accepted together with a blockmask: the same workspace rule applies
+    assert lib.fa_fwd_workspace_bytes(ctypes.byref(a)) > 0
+    assert lib.fa_fwd_block(ctypes.byref(a)) == -2 and b"workspace" in lib.fa_last_error()
 
 
 def test_workspace_sizes(lib):
@@ -193,8 +194,16 @@ def test_convert_blockmask_matches_spec():
             got = convert_blockmask(m, causal=False)
             assert got.dtype == torch.int32 and tuple(got.shape) == (shape[1], shape[0])
             assert np.array_equal(got.numpy(), orc.convert_blockmask_ref(m.numpy()))
-    with pytest.raises(AssertionError):
-        convert_blockmask(torch.ones(2, 2), causal=True)  # flash_blocksparse_attn_interface.py:21
+    # causal (the reference asserts against it, flash_blocksparse_attn_interface.py:21): the list of the layout with
+    # the blocks that hold no key <= query taken out, found here element by element
+    for shape in ((3, 2), (16, 1), (40, 3), (64, 4)):
+        m = torch.rand(shape, generator=g) < 0.7
+        seen = np.zeros(shape, dtype=bool)
+        for r in range(shape[0]):
+            for c in range(shape[1]):
+                seen[r, c] = any(k <= q for q in range(16 * r, 16 * r + 16) for k in (256 * c, 256 * c + 255))
+        want = orc.convert_blockmask_ref(m.numpy() & seen)
+        assert np.array_equal(convert_blockmask(m, causal=True).numpy(), want)
 
 
 def test_unpad_pad_match_spec_and_backprop():

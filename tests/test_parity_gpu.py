@@ -530,6 +530,59 @@ def test_blocksparse_full_layout_equals_dense():
     b = flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0)
     torch.cuda.synchronize()
     assert torch.equal(a, b)
+    a = flash_blocksparse_attn_func(qkv, cu, layout, 0.0, N, causal=True)
+    b = flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0, causal=True)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
+def test_blocksparse_causal_sweep():
+    """Causal on top of a block layout (the reference's Python refuses the pair, flash_blocksparse_attn_interface.py:21;
+    its kernels take both): a score counts iff its block is listed and key <= query.  Eight seeded cases over head dim,
+    dtype, ragged lengths, density and dropout; rows whose listed blocks all lie above the diagonal give zeros; the
+    returned probabilities vanish above the diagonal and outside the layout."""
+    from flash_attn.flash_blocksparse_attn_interface import flash_blocksparse_attn_func
+    from flash_attn import flash_attn_gfx950 as be
+    rng = np.random.default_rng(77)
+    for case in range(8):
+        D = int(rng.choice([16, 32, 64, 128]))
+        dtype = torch.float16 if rng.integers(2) else torch.bfloat16
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 3))
+        N = int(rng.choice([100, 300, 520, 1100, 2100]))
+        lens = [N] + [int(x) for x in rng.integers(max(1, N // 3), N + 1, B - 1)]
+        dens = float(rng.choice([0.1, 0.3, 0.6, 1.0]))
+        p = float(rng.choice([0.0, 0.0, 0.2]))
+        sq_r, sk_r = be.round_seqlens(D, N, N, True)
+        layout = torch.rand(sq_r // 16, sk_r // 256, generator=torch.Generator().manual_seed(50 + case)) < dens
+        if rng.integers(2):
+            layout |= (torch.arange(sq_r // 16)[:, None] // 16) == torch.arange(sk_r // 256)[None, :]
+        if sk_r > 256 and sq_r // 16 > 2:
+            layout[2] = False
+            layout[2, 1] = True     # rows 32..47 list only keys 256..511: nothing visible under the causal mask
+        what = "case %d: D=%d %s B=%d H=%d lens=%s density %.2f p=%.1f" % (case, D, dtype, B, H, lens, dens, p)
+        print(what, flush=True)
+        q, k, v, do = _inputs(lens, lens, H, D, dtype, 4000 + case)
+        cu = _cu(lens, "cpu")
+        qkv = torch.stack([q, k, v], 1).cuda().requires_grad_()
+        torch.manual_seed(case)
+        seed, offset = _gen_state()
+        ctx, S, lse = flash_blocksparse_attn_func(qkv, cu.cuda(), layout.cuda(), p, N, None, True, True)
+        ctx.backward(do.cuda())
+        torch.cuda.synchronize()
+        masks = None
+        if p > 0:
+            masks = [torch.tensor(np.stack([orc.dropout_keep_mask(seed, offset, b * H + h, L, L, p) for h in range(H)]))
+                     for b, L in enumerate(lens)]
+        ref = orc.varlen_attention(q, k, v, cu, cu, None, True, p_dropout=p, keep_mask=masks, layout=layout.numpy(), dout=do)
+        half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu.tolist(), cu.tolist(), D ** -0.5, True, masks, p,
+                              layout=layout.numpy(), dout=do.cuda())
+        ours = {"out": ctx.detach(), "dq": qkv.grad[:, 0], "dk": qkv.grad[:, 1], "dv": qkv.grad[:, 2]}
+        check_against_oracle(ours, ref, half, dtype, what=what)
+        seen = orc.expand_block_layout(layout.numpy(), N, N) & (torch.arange(N)[None, :] <= torch.arange(N)[:, None])
+        assert S[0, :, :N, :N].cpu()[:, ~seen].abs().max() == 0, what
+        if sk_r > 256 and sq_r // 16 > 2:
+            assert ctx[32:48].abs().max() == 0 and torch.isinf(lse[0, :, 32:48]).all(), what
+            assert qkv.grad[32:48, 0].abs().max() == 0, what
 
 
 # ------------------------------------------------------------------------------------------------
@@ -830,6 +883,13 @@ def test_blocksparse_modules_layout_sources_and_padding():
                                    layout=layout[:(L + 15) // 16, :(L + 255) // 256].numpy())
         assert (o3[b, :L].float().cpu() - ref["out"]).abs().max() < 2e-3
         assert not o3[b, L:].any()
+    # causal=True through the module: padded, and packed with the module's stored (non-causal) conversion
+    oc, _ = m_t(qkv.cuda(), causal=True)
+    oc2, _ = m_o(packed, cu_seqlens=cu, max_s=S, causal=True, convert_mask=False)
+    assert torch.equal(oc2, oc.reshape(B * S, H, D))
+    ref = orc.varlen_attention(qkv[0, :, 0], qkv[0, :, 1], qkv[0, :, 2], _cu([S], "cpu"), _cu([S], "cpu"), sc, True,
+                               layout=layout.numpy())
+    assert (oc[0].float().cpu() - ref["out"]).abs().max() < 2e-3
     # MHA block: gradient flows to the projections
     mha = FlashBlocksparseMHA(H * D, H, layout, max_seq_length=S, device="cuda", dtype=torch.float16)
     x = torch.randn(B, S, H * D, device="cuda", dtype=torch.float16, requires_grad=True)
