@@ -159,7 +159,7 @@ uint64_t fa_philox_offset_increment(void);
  *                  (IndexPutFirstAxis.forward :38-48, IndexFirstAxis.backward :21-30).  dst is written exactly once
  *                  and needs no prior zero fill; indices must be unique (duplicates: one of the rows wins); indices
  *                  outside [0, n_dst_rows) are ignored.  `workspace`: fa_scatter_rows_workspace_bytes(n_dst_rows)
- *                  bytes of device scratch (the inverse index). */
+ *                  bytes of device scratch (the inverse index; its contents on entry do not matter). */
 int fa_gather_rows(const void* src, void* dst, const int64_t* indices, int64_t n_indices, int64_t n_src_rows,
                    int64_t row_bytes, int64_t src_row_stride, int64_t dst_row_stride, void* stream);
 int fa_scatter_rows(const void* src, void* dst, const int64_t* indices, int64_t n_indices, int64_t n_dst_rows,
