@@ -13,6 +13,7 @@ It restates, in plain fp32/fp64 PyTorch and NumPy on the host, the algorithm of 
   dropout_keep_mask        this engine's mapping from (seed, offset, b, h, q, key) to keep/drop
   convert_blockmask_ref    specification of flash_attn/flash_blocksparse_attn_interface.py:8-40
   unpad_ref / pad_ref      specification of flash_attn/bert_padding.py:60-95
+  rotary_ref               rotation of flash_attn/rotary.py:22-42 (x * cos + rotate_half(x) * sin) in fp64
 
 How each function is pinned (the reference has no tests, golden vectors or fixtures of its own):
   attention_ref / varlen_attention forward: against torch.nn.functional.scaled_dot_product_attention (library
@@ -24,6 +25,9 @@ How each function is pinned (the reference has no tests, golden vectors or fixtu
       the reference uses (tests/golden/philox_kat.json).
   dropout_keep_mask: it is the definition; tests compare the kernels' S_dmask signs to it bit for bit.
   convert_blockmask_ref: brute force over all small masks against an independent per-element definition.
+  unpad_ref / pad_ref: round trip pad(unpad(x)) == x * mask, cu_seqlens against the cumulative sum of the lengths.
+  rotary_ref: the cited definition evaluated literally; it is a rotation (norm kept, conjugate inverts it, angles add,
+      position 0 is the identity).
 PARITY UNPINNED (only running the CUDA reference could pin them; nothing in this pipeline can): the reference's
   fragment-permuted S_dmask layout and running-max scaling (gmem_tile.h:289-405), its thread-indexed Philox stream
   assignment (so masks are compared with this engine's own definition, not NVIDIA's), and bit-level fp16 rounding /
