@@ -1,7 +1,8 @@
 // Micro-benchmarks of the gfx950 compute unit that the attention kernels' design is argued from:
 //   1. sustained MFMA rate (v_mfma_f32_32x32x16_f16) and the shader clock it settles at, with constant and with
 //      random operands (the part is power limited: toggling operands lower the clock),
-//   2. cost of VALU / transcendental instructions issued between MFMAs (they do not run underneath an MFMA),
+//   2. cost of VALU / transcendental instructions issued between MFMAs (they do not run underneath an MFMA, whether
+//      they come from the same wave or from another wave of the SIMD), and what the accumulators' register file costs,
 //   3. issue cost of the VALU instructions the softmax uses, on their own,
 //   4. LDS read bandwidth of ds_read_b128 row fragments and ds_read_b64_tr_b16 transposed fragments for padded row
 //      strides and for the unpadded, chunk-swizzled tile layouts of fa_stage.h.
@@ -59,8 +60,12 @@ struct ClockProbe {
 };
 
 // ---- 1 + 2: 8 MFMAs per trip over 4 independent accumulators; operands rotate over 8 A and 8 B fragments taken from
-// `src`; NV independent fp32 FMAs and NE exp2 follow every MFMA
-template <int NV, int NE>
+// `src`; NV independent fp32 FMAs and NE exp2 follow every MFMA.
+// FORM 0: the compiler's choice for this kernel, accumulators in AccVGPRs (it has the whole register file);
+// FORM 1: accumulators in ordinary VGPRs, the form the attention kernels' MFMAs have (their results feed the VALU).
+// SPLIT: workgroups with an even id only issue the MFMAs, those with an odd id only the VALU work; at two workgroups per
+// compute unit every SIMD then holds one wave of each kind.
+template <int NV, int NE, int FORM = 0, bool SPLIT = false>
 __global__ void __launch_bounds__(256) mfma_mix_kernel(const f16x8* __restrict__ src, float* out, int iters) {
   ClockProbe probe;
   probe.start();
@@ -78,11 +83,18 @@ __global__ void __launch_bounds__(256) mfma_mix_kernel(const f16x8* __restrict__
   for (int it = 0; it < iters; it++) {
 #pragma unroll
     for (int u = 0; u < 8; u++) {
-      acc[u & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[u], Bv[(u * 3 + 1) & 7], acc[u & 3], 0, 0, 0);
+      if (!SPLIT || (blockIdx.x & 1) == 0) {
+        if (FORM == 1)
+          asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc[u & 3]) : "v"(A[u]), "v"(Bv[(u * 3 + 1) & 7]));
+        else
+          acc[u & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[u], Bv[(u * 3 + 1) & 7], acc[u & 3], 0, 0, 0);
+      }
+      if (!SPLIT || (blockIdx.x & 1) == 1) {
 #pragma unroll
-      for (int v = 0; v < NV; v++) xs[v & 7] = __builtin_fmaf(xs[v & 7], 0.999f, 0.37f);
+        for (int v = 0; v < NV; v++) xs[v & 7] = __builtin_fmaf(xs[v & 7], 0.999f, 0.37f);
 #pragma unroll
-      for (int v = 0; v < NE; v++) xs[(v + 4) & 7] = __builtin_amdgcn_exp2f(xs[(v + 4) & 7] * 0.03f);
+        for (int v = 0; v < NE; v++) xs[(v + 4) & 7] = __builtin_amdgcn_exp2f(xs[(v + 4) & 7] * 0.03f);
+      }
     }
     if ((it & 63) == 63)
       for (int n = 0; n < 4; n++) acc[n] = acc[n] * 0.001f;  // keep the accumulators bounded
@@ -95,14 +107,15 @@ __global__ void __launch_bounds__(256) mfma_mix_kernel(const f16x8* __restrict__
   probe.stop();
 }
 
-template <int NV, int NE>
+template <int NV, int NE, int FORM = 0, bool SPLIT = false>
 static void run_mix(const char* name, int waves_per_simd) {
   const int iters = 2000, blocks = 256 * waves_per_simd;
   double ghz;
-  const float ms = time_ms([&] { mfma_mix_kernel<NV, NE><<<blocks, 256>>>(g_src, g_out, iters); }, &ghz);
-  const double flops = (double)blocks * 4 * iters * 8 * 32768.0;
+  const float ms = time_ms([&] { mfma_mix_kernel<NV, NE, FORM, SPLIT><<<blocks, 256>>>(g_src, g_out, iters); }, &ghz);
+  const int mfma_waves = SPLIT ? waves_per_simd / 2 : waves_per_simd;  // waves per SIMD that issue MFMAs
+  const double flops = (double)blocks / waves_per_simd * mfma_waves * 4 * iters * 8 * 32768.0;
   printf("  %-34s %d wave(s)/SIMD: %7.1f TFLOP/s, clock %.2f GHz, %5.1f cycles per MFMA slot\n", name, waves_per_simd,
-         flops / ms / 1e9, ghz, ms * 1e-3 * ghz * 1e9 / ((double)iters * 8 * waves_per_simd));
+         flops / ms / 1e9, ghz, ms * 1e-3 * ghz * 1e9 / ((double)iters * 8 * mfma_waves));
 }
 
 static void fill_src(int mode) {  // 0: uniform random in [-2, 2), 1: zeros
@@ -234,6 +247,11 @@ int main() {
   run_mix<0, 2>("MFMA + 2 v_exp_f32 (+2 v_mul)", 2);
   run_mix<8, 2>("MFMA + 8 v_fma_f32 + 2 v_exp_f32", 2);
   run_mix<8, 2>("MFMA + 8 v_fma_f32 + 2 v_exp_f32", 3);
+  printf("2b. accumulators in VGPRs (as in the attention kernels) instead of AccVGPRs; MFMA and VALU work in separate waves\n");
+  run_mix<0, 0, 1>("VGPR acc: MFMA only", 2);
+  run_mix<8, 0, 1>("VGPR acc: MFMA + 8 v_fma_f32", 2);
+  run_mix<8, 2, 1>("VGPR acc: MFMA + 8 fma + 2 exp", 2);
+  run_mix<8, 0, 0, true>("MFMA wave | 8 v_fma_f32 wave", 2);
 
   printf("3. issue cost of VALU instructions on their own, 2 waves per SIMD\n");
   run_op<0>("v_fma_f32");
