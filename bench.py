@@ -155,6 +155,23 @@ def cpu_baseline(torch, B, H, D, N, budget_s=20.0):
                       % (reps, B, H, D, N, spent)}
 
 
+def device_peak(torch):
+    """Dense fp16 MFMA rate from what the device reports: compute units x 4096 flop/clock x the maximum shader clock
+    (v_mfma_f32_32x32x16_f16 = 32768 flop in 32 cycles on each of a compute unit's 4 SIMDs)."""
+    import ctypes
+    props = torch.cuda.get_device_properties(0)
+    cus = int(props.multi_processor_count)
+    mhz = 0.0
+    try:  # hipDeviceAttributeClockRate = 5: peak clock in kHz (torch's device properties do not carry it)
+        khz = ctypes.c_int(0)
+        if ctypes.CDLL("libamdhip64.so").hipDeviceGetAttribute(ctypes.byref(khz), 5, 0) == 0:
+            mhz = khz.value / 1e3
+    except OSError:
+        pass
+    return {"name": props.name, "compute_units": cus, "max_clock_mhz": round(mhz, 1),
+            "tflops": round(cus * 4096 * mhz * 1e6 / 1e12, 1) if mhz else None}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -201,6 +218,7 @@ def main():
         "config": {"workload": "headline: fp16 packed qkv [16384,3,12,64], B=8 H=12 d=64 N=2048 equal lengths, "
                                "non-causal, dropout 0, fwd+bwd with dout~N(0,1)"},
         "pct_of_mfma_peak": round(100.0 * value / MFMA_PEAK_TFLOPS, 2),
+        "device_peak": device_peak(torch),
         "fwd_ms": round(t["fwd_ms"], 4), "bwd_ms": round(t["bwd_ms"], 4),
         "fwd_tflops": round(fwd_flops / (t["fwd_ms"] * 1e-3) / 1e12, 1),
         "bwd_tflops": round(2.5 * fwd_flops / (t["bwd_ms"] * 1e-3) / 1e12, 1),
