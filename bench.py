@@ -259,7 +259,7 @@ def main():
                 name, tt["fwd_ms"], tt["bwd_ms"], wl.fwd_flops / (tt["fwd_ms"] * 1e-3) / 1e12, fb,
                 100 * fb / MFMA_PEAK_TFLOPS, gbs), file=sys.stderr)
         # unpad / pad (row gather and scatter, HBM-bound): BERT-large-like padded batch, 75 % of the tokens valid
-        from flash_attn.bert_padding import pad_input, unpad_input
+        from flash_attn.bert_padding import unpad_input
         Bp, Sp, dim = 64, 512, 1024
         gen = torch.Generator().manual_seed(0)
         lens_p = torch.randint(Sp // 2, Sp + 1, (Bp,), generator=gen)

@@ -7,7 +7,6 @@ shared library next to the Python package that loads it.
 import argparse
 import os
 import subprocess
-import sys
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
