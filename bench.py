@@ -131,6 +131,46 @@ def time_steps(torch, be, w, steps, warmup, settle_s=0.2):
             "bwd_main_kernel_ms": bwd_main_ms}
 
 
+def torch_attention_ms(torch, w, iters=8):
+    """Forward + backward of standard attention written with PyTorch ops in the workload's own dtype on the GPU - the
+    comparison point of every speed-up the reference publishes (attention_ref, benchmarks/benchmark_flash_attention.py:
+    14-36, 60-66: scores, key-padding and causal masks as -inf, softmax, dropout, attn @ v on a padded batch)."""
+    B, H, D, N = w.B, w.H, w.D, w.max_s
+    qkv = torch.zeros(B, N, 3, H, D, device="cuda", dtype=w.dtype)
+    dout = torch.zeros(B, N, H, D, device="cuda", dtype=w.dtype)
+    keep = torch.zeros(B, N, dtype=torch.bool, device="cuda")
+    cu = w.cu.tolist()
+    for b, L in enumerate(w.lens):
+        qkv[b, :L] = w.qkv[cu[b]:cu[b + 1]]
+        dout[b, :L] = w.dout[cu[b]:cu[b + 1]]
+        keep[b, :L] = True
+    qkv.requires_grad_()
+    ragged = min(w.lens) < N
+    causal_mask = torch.triu(torch.ones(N, N, dtype=torch.bool, device="cuda"), 1) if w.causal else None
+
+    def step():
+        q, k, v = qkv.unbind(dim=2)
+        scores = torch.einsum("bthd,bshd->bhts", q * w.scale, k)
+        if ragged:
+            scores = scores.masked_fill(~keep[:, None, None, :], float("-inf"))
+        if causal_mask is not None:
+            scores = scores.masked_fill(causal_mask, float("-inf"))
+        attn = torch.nn.functional.dropout(torch.softmax(scores, dim=-1), w.p)
+        out = torch.einsum("bhts,bshd->bthd", attn, v)
+        qkv.grad = None
+        out.backward(dout)
+
+    for _ in range(3):
+        step()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
 def cpu_baseline(torch, B, H, D, N, budget_s=20.0):
     """The oracle's standard attention (attention_ref: fp32, PyTorch ops on the host cores), forward + backward through
     autograd, on a bounded sample of the headline workload: whole batches of (B, N) are repeated until about
@@ -230,6 +270,11 @@ def main():
                      # 256 MiB copy): 101 461 KiB read + 50 688 KiB written
                      "traffic": 155.8e6},
     }
+    pt_ms = torch_attention_ms(torch, w)
+    res["pytorch_attention_same_gpu"] = {
+        "ms_per_step": round(pt_ms, 3), "speedup": round(pt_ms / (t["fwd_ms"] + t["bwd_ms"]), 2),
+        "what": "standard attention with PyTorch fp16 ops, fwd+bwd, same inputs, same GPU: the comparison point of the "
+                "reference's published speed-ups (about 2x on A100 for this shape without mask or dropout)"}
     if not a.no_cpu:
         res["cpu_baseline"] = cpu_baseline(torch, B, H, D, N, a.cpu_budget)
     else:
@@ -248,16 +293,21 @@ def main():
             ("blocksparse 25% 256x256", dict(B=4, H=16, D=64, N=4096, dtype=torch.float16,
                                              blockmask=sparse_layout(torch, 4096, rows_per_draw=16))),
         ]
-        print("%-28s %9s %9s %9s %9s %8s %10s" % ("config", "fwd ms", "bwd ms", "fwd TF", "f+b TF", "% peak", "f+b GB/s"),
-              file=sys.stderr)
+        print("%-28s %9s %9s %9s %9s %8s %10s %11s %8s" % ("config", "fwd ms", "bwd ms", "fwd TF", "f+b TF", "% peak", "f+b GB/s",
+                                                          "PyTorch ms", "speedup"), file=sys.stderr)
         for name, kw in cfgs:
             wl = Workload(torch, **kw)
             tt = time_steps(torch, be, wl, max(10, a.steps // 2), 5, a.settle)
             fb = 3.5 * wl.fwd_flops / ((tt["fwd_ms"] + tt["bwd_ms"]) * 1e-3) / 1e12
             gbs = (wl.bytes_fwd + wl.bytes_bwd) / ((tt["fwd_ms"] + tt["bwd_ms"]) * 1e-3) / 1e9
-            print("%-28s %9.4f %9.4f %9.1f %9.1f %8.2f %10.1f" % (
+            # PyTorch standard attention on the same GPU (no counterpart for a block layout)
+            pt = torch_attention_ms(torch, wl, 4) if wl.blockmask is None else None
+            print("%-28s %9.4f %9.4f %9.1f %9.1f %8.2f %10.1f %11s %8s" % (
                 name, tt["fwd_ms"], tt["bwd_ms"], wl.fwd_flops / (tt["fwd_ms"] * 1e-3) / 1e12, fb,
-                100 * fb / MFMA_PEAK_TFLOPS, gbs), file=sys.stderr)
+                100 * fb / MFMA_PEAK_TFLOPS, gbs, "%.3f" % pt if pt else "-",
+                "%.1fx" % (pt / (tt["fwd_ms"] + tt["bwd_ms"])) if pt else "-"), file=sys.stderr)
+            del wl
+            torch.cuda.empty_cache()
         # unpad / pad (row gather and scatter, HBM-bound): BERT-large-like padded batch, 75 % of the tokens valid
         from flash_attn.bert_padding import unpad_input
         Bp, Sp, dim = 64, 512, 1024
