@@ -131,7 +131,7 @@ def time_steps(torch, be, w, steps, warmup, settle_s=0.2):
             "bwd_main_kernel_ms": bwd_main_ms}
 
 
-def torch_attention_ms(torch, w, iters=8):
+def torch_attention_ms(torch, w, iters=8, want_memory=False):
     """Forward + backward of standard attention written with PyTorch ops in the workload's own dtype on the GPU - the
     comparison point of every speed-up the reference publishes (attention_ref, benchmarks/benchmark_flash_attention.py:
     14-36, 60-66: scores, key-padding and causal masks as -inf, softmax, dropout, attn @ v on a padded batch)."""
@@ -168,7 +168,38 @@ def torch_attention_ms(torch, w, iters=8):
         step()
     e1.record()
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) / iters
+    ms = e0.elapsed_time(e1) / iters
+    if not want_memory:
+        return ms
+    # peak device memory of one step beyond what is allocated before it (inputs, dout, the previous gradient)
+    qkv.grad = None
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    step()
+    torch.cuda.synchronize()
+    return ms, torch.cuda.max_memory_allocated() - base
+
+
+def fused_step_memory(torch, w):
+    """Peak device memory of one forward + backward through the public autograd function beyond what is allocated
+    before it (out, softmax_lse, dqkv; no N x N tensor)."""
+    from flash_attn.flash_attn_interface import flash_attn_unpadded_qkvpacked_func
+    qkv = w.qkv.detach().clone().requires_grad_()
+
+    def step():
+        qkv.grad = None
+        out = flash_attn_unpadded_qkvpacked_func(qkv, w.cu, w.max_s, w.p, causal=w.causal)
+        out.backward(w.dout)
+
+    step()
+    qkv.grad = None
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    step()
+    torch.cuda.synchronize()
+    return torch.cuda.max_memory_allocated() - base
 
 
 def cpu_baseline(torch, B, H, D, N, budget_s=20.0):
@@ -270,11 +301,15 @@ def main():
                      # 256 MiB copy): 101 461 KiB read + 50 688 KiB written
                      "traffic": 155.8e6},
     }
-    pt_ms = torch_attention_ms(torch, w)
+    pt_ms, pt_mem = torch_attention_ms(torch, w, want_memory=True)
+    our_mem = fused_step_memory(torch, w)
     res["pytorch_attention_same_gpu"] = {
         "ms_per_step": round(pt_ms, 3), "speedup": round(pt_ms / (t["fwd_ms"] + t["bwd_ms"]), 2),
+        "step_memory_mb": round(pt_mem / 2 ** 20, 1), "fused_step_memory_mb": round(our_mem / 2 ** 20, 1),
+        "memory_reduction": round(pt_mem / our_mem, 1),
         "what": "standard attention with PyTorch fp16 ops, fwd+bwd, same inputs, same GPU: the comparison point of the "
-                "reference's published speed-ups (about 2x on A100 for this shape without mask or dropout)"}
+                "reference's published speed-ups (about 2x on A100 for this shape without mask or dropout) and memory "
+                "savings (about 10x at N=2048); step memory = peak device memory of one fwd+bwd beyond its inputs"}
     if not a.no_cpu:
         res["cpu_baseline"] = cpu_baseline(torch, B, H, D, N, a.cpu_budget)
     else:
