@@ -319,6 +319,9 @@ def main():
         cfgs = [
             ("BERT varlen p=0.1 fp16", dict(B=8, H=12, D=64, N=512, dtype=torch.float16, p=0.1,
                                             lens=torch.randint(256, 513, (8,), generator=torch.Generator().manual_seed(0)).tolist())),
+            # the configuration of the reference's own script (benchmarks/benchmark_flash_attention.py:39-70)
+            ("reference script B64 H16 p=0.1", dict(B=64, H=16, D=64, N=1024, dtype=torch.float16, p=0.1,
+                                                    lens=torch.randint(1004, 1024, (64,), generator=torch.Generator().manual_seed(0)).tolist())),
             ("GPT2 causal bf16 N=1024", dict(B=8, H=12, D=64, N=1024, dtype=torch.bfloat16, causal=True)),
             ("GPT2 causal bf16 N=2048", dict(B=8, H=12, D=64, N=2048, dtype=torch.bfloat16, causal=True)),
             ("GPT2 causal bf16 N=4096", dict(B=8, H=12, D=64, N=4096, dtype=torch.bfloat16, causal=True)),
@@ -328,7 +331,7 @@ def main():
             ("blocksparse 25% 256x256", dict(B=4, H=16, D=64, N=4096, dtype=torch.float16,
                                              blockmask=sparse_layout(torch, 4096, rows_per_draw=16))),
         ]
-        print("%-28s %9s %9s %9s %9s %8s %10s %11s %8s" % ("config", "fwd ms", "bwd ms", "fwd TF", "f+b TF", "% peak", "f+b GB/s",
+        print("%-31s %9s %9s %9s %9s %8s %10s %11s %8s" % ("config", "fwd ms", "bwd ms", "fwd TF", "f+b TF", "% peak", "f+b GB/s",
                                                           "PyTorch ms", "speedup"), file=sys.stderr)
         for name, kw in cfgs:
             wl = Workload(torch, **kw)
@@ -337,7 +340,7 @@ def main():
             gbs = (wl.bytes_fwd + wl.bytes_bwd) / ((tt["fwd_ms"] + tt["bwd_ms"]) * 1e-3) / 1e9
             # PyTorch standard attention on the same GPU (no counterpart for a block layout)
             pt = torch_attention_ms(torch, wl, 4) if wl.blockmask is None else None
-            print("%-28s %9.4f %9.4f %9.1f %9.1f %8.2f %10.1f %11s %8s" % (
+            print("%-31s %9.4f %9.4f %9.1f %9.1f %8.2f %10.1f %11s %8s" % (
                 name, tt["fwd_ms"], tt["bwd_ms"], wl.fwd_flops / (tt["fwd_ms"] * 1e-3) / 1e12, fb,
                 100 * fb / MFMA_PEAK_TFLOPS, gbs, "%.3f" % pt if pt else "-",
                 "%.1fx" % (pt / (tt["fwd_ms"] + tt["bwd_ms"])) if pt else "-"), file=sys.stderr)
