@@ -394,6 +394,65 @@ def test_element_offsets_beyond_int32():
         check_against_oracle(ours, ref, half, torch.float16, what="sequence %d of %d" % (b, B))
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_sequence_of_64k_tokens(causal):
+    """One sequence of 65536 tokens (the longest the reference advertises, README.md:68): 512 query tiles and 1024 key
+    tiles per head, far more than any other test walks.  The N x N closed form does not fit the oracle's way of working,
+    so it is evaluated in fp32 on the GPU in row chunks (exact lse and out for every row), and the gradients are checked
+    on sampled rows (dq) and sampled key columns (dk, dv) from the explicit formulas dV = P^T dO, dS = P o (dP - D),
+    dQ = scale dS K, dK = scale dS^T Q.  Tolerances: a few fp16 roundings of values of order one."""
+    from flash_attn import flash_attn_gfx950 as be
+    N, H, D = 65536, 2, 64
+    scale = D ** -0.5
+    g = torch.Generator(device="cuda").manual_seed(11)
+    qkv = torch.randn(N, 3, H, D, device="cuda", dtype=torch.float16, generator=g)
+    do = torch.randn(N, H, D, device="cuda", dtype=torch.float16, generator=g)
+    cu = torch.tensor([0, N], dtype=torch.int32, device="cuda")
+    out, lse = be.fwd(qkv[:, 0], qkv[:, 1], qkv[:, 2], cu, cu, N, N, 0.0, scale, False, causal, False, None)
+    grad = torch.empty_like(qkv)
+    be.bwd(do, qkv[:, 0], qkv[:, 1], qkv[:, 2], out, lse, grad[:, 0], grad[:, 1], grad[:, 2], cu, cu, N, N, 0.0, scale,
+           False, causal, None)
+    torch.cuda.synchronize()
+    q, k, v = (qkv[:, i].float().transpose(0, 1) for i in range(3))             # (H, N, D)
+    dof = do.float().transpose(0, 1)
+    pos = torch.arange(N, device="cuda")
+    lse_ref = torch.empty(H, N, device="cuda")
+    out_ref = torch.empty(H, N, D, device="cuda")
+    for r0 in range(0, N, 4096):
+        sc = torch.einsum("hqd,hkd->hqk", q[:, r0:r0 + 4096], k) * scale
+        if causal:
+            sc = sc.masked_fill(pos[None, None, :] > pos[None, r0:r0 + 4096, None], float("-inf"))
+        lse_ref[:, r0:r0 + 4096] = torch.logsumexp(sc, -1)
+        out_ref[:, r0:r0 + 4096] = torch.einsum("hqk,hkd->hqd", torch.exp(sc - lse_ref[:, r0:r0 + 4096, None]), v)
+        del sc
+    assert (lse[0, :, :N] - lse_ref).abs().max() < 1e-3
+    assert (out.float().transpose(0, 1) - out_ref).abs().max() < 2e-3
+    dsum = (dof * out_ref).sum(-1)                                             # D_i = rowsum(dO o O)
+    gsel = torch.Generator().manual_seed(3)
+    rows = torch.cat([torch.tensor([0, 1, 127, 128, N - 1]), torch.randint(0, N, (251,), generator=gsel)]).cuda()
+    cols = torch.cat([torch.tensor([0, 63, 64, N - 2, N - 1]), torch.randint(0, N, (251,), generator=gsel)]).cuda()
+    # sampled query rows against every key
+    sc = torch.einsum("hqd,hkd->hqk", q[:, rows], k) * scale
+    if causal:
+        sc = sc.masked_fill(pos[None, None, :] > rows[None, :, None], float("-inf"))
+    pr = torch.exp(sc - lse_ref[:, rows, None])
+    ds = pr * (torch.einsum("hqd,hkd->hqk", dof[:, rows], v) - dsum[:, rows, None])
+    dq_ref = scale * torch.einsum("hqk,hkd->hqd", ds, k)
+    assert (grad[rows, 0].float().transpose(0, 1) - dq_ref).abs().max() < 4e-3
+    del sc, pr, ds
+    # every query row against sampled key columns
+    sc = torch.einsum("hqd,hkd->hqk", q, k[:, cols]) * scale
+    if causal:
+        sc = sc.masked_fill(cols[None, None, :] > pos[None, :, None], float("-inf"))
+    pr = torch.exp(sc - lse_ref[:, :, None])
+    dv_ref = torch.einsum("hqk,hqd->hkd", pr, dof)
+    ds = pr * (torch.einsum("hqd,hkd->hqk", dof, v[:, cols]) - dsum[:, :, None])
+    dk_ref = scale * torch.einsum("hqk,hqd->hkd", ds, q)
+    tol = lambda ref: 4e-3 + 2.0 ** -10 * ref.abs().max().item()
+    assert (grad[cols, 2].float().transpose(0, 1) - dv_ref).abs().max() < tol(dv_ref)
+    assert (grad[cols, 1].float().transpose(0, 1) - dk_ref).abs().max() < tol(dk_ref)
+
+
 def test_parity_random_shapes_sweep():
     """Twenty-four seeded random cases over what the parametrised tests hold fixed: batch size, ragged query and key
     lengths (self- and cross-attention, empty key sides excluded), heads, head dim, dtype, causal, packing, scale."""
