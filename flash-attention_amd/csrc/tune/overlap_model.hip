@@ -11,7 +11,8 @@
 //              exponentials, one MFMA per N VALU instructions (scheduling-group barriers), i.e. the matrix pipe and the
 //              VALU of ONE wave always have independent work,
 // next to the MFMAs alone and the VALU work alone, and the chain with the K and V fragments fetched from LDS every step
-// as a kernel must (8 ds_read_b128 + 16 ds_read_b64 per wave and step, no staging traffic).  Every line reports time and, from the cycle counter read against
+// as a kernel must (8 ds_read_b128 + 16 ds_read_b64 per wave and step, no staging traffic), once for 32 query rows per
+// wave and once for 64 (two row blocks share every fragment read; the time is quoted per 32 rows).  Every line reports time and, from the cycle counter read against
 // the 100 MHz wall clock inside the kernel, the shader clock: when the interleaved forms need fewer cycles but the clock
 // falls by as much, the loop is power limited, not issue limited.
 // Build and run from the repository root with the kernels' flags:
@@ -30,7 +31,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 struct PFrag { f16x8 v[4]; };  // the converted probabilities of a step: B operands of its four PV MFMA pairs
 __device__ long long g_clk[2];
 
-enum { kMfmaOnly, kValuOnly, kChain, kAhead, kAheadPV, kChainLds };
+enum { kMfmaOnly, kValuOnly, kChain, kAhead, kAheadPV, kChainLds, kChainLds2 };
 
 __device__ __forceinline__ void s_mfma(f32x16* s, const f16x8* K, const f16x8* Q) {
 #pragma unroll
@@ -103,8 +104,15 @@ __global__ void __launch_bounds__(256, WAVES) step_kernel(const f16x8* __restric
   PFrag pa, pb;
   for (int j = 0; j < 4; j++) pa.v[j] = K[j];
   if (FORM == kAhead || FORM == kAheadPV) s_mfma(sa, K, Q);
-  __shared__ __attribute__((aligned(16))) unsigned char lds[FORM == kChainLds ? 32768 : 16];
-  if (FORM == kChainLds) {
+  constexpr bool kLds = FORM == kChainLds || FORM == kChainLds2;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[kLds ? 32768 : 16];
+  f16x8 Q2[4];   // second row block of kChainLds2
+  f32x16 o2[2];
+  float m2 = 0.5f, l2 = 0.f;
+  for (int i = 0; i < 4; i++) Q2[i] = src[(lane * 4 + i + 3072 + tid) & 4095];
+  for (int n = 0; n < 2; n++)
+    for (int i = 0; i < 16; i++) o2[n][i] = 0;
+  if (kLds) {
     for (int i = tid; i < 2048; i += 256) reinterpret_cast<f16x8*>(lds)[i] = src[(i * 7 + blockIdx.x) & 4095];
     __syncthreads();
   }
@@ -113,6 +121,7 @@ __global__ void __launch_bounds__(256, WAVES) step_kernel(const f16x8* __restric
   auto step = [&](f32x16* sc, f32x16* sn, PFrag& pp, PFrag& pc) {
     asm volatile("" : "+v"(o[0]), "+v"(o[1]));
     asm volatile("" : "+v"(Q[0]), "+v"(Q[1]), "+v"(Q[2]), "+v"(Q[3]));  // keeps the S MFMAs inside the loop
+    if (FORM == kChainLds2) asm volatile("" : "+v"(o2[0]), "+v"(o2[1]), "+v"(Q2[0]), "+v"(Q2[1]), "+v"(Q2[2]), "+v"(Q2[3]));
     if (FORM == kMfmaOnly) {
       s_mfma(sc, K, Q);
       for (int j = 0; j < 4; j++) pc.v[j] = __builtin_bit_cast(f16x8, __builtin_shufflevector(sc[j >> 1], sc[j >> 1], 0, 1, 2, 3));
@@ -143,6 +152,31 @@ __global__ void __launch_bounds__(256, WAVES) step_kernel(const f16x8* __restric
           const u32x2 hi = *reinterpret_cast<const u32x2*>(base + 8192 + (j * 4 + db * 2 + 1) * 512 + lane * 8);
           const u32x4 av = {lo[0], lo[1], hi[0], hi[1]};
           o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, av), pc.v[j], o[db], 0, 0, 0);
+        }
+      }
+    } else if (FORM == kChainLds2) {
+      // as kChainLds for two blocks of 32 query rows that share the fragment reads (second block: sn, pp, o2, m2, l2)
+      const unsigned char* base = lds + ((it_ & 1) ? 16384 : 0);
+      f16x8 Kl[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) Kl[i] = *reinterpret_cast<const f16x8*>(base + i * 1024 + lane * 16);
+      s_mfma(sc, Kl, Q);
+      s_mfma(sn, Kl, Q2);
+      softmax_max(sc, m, l, o, cs, nullptr);
+      softmax_exp(sc, m, l, cs, pc);
+      softmax_max(sn, m2, l2, o2, cs, nullptr);
+      softmax_exp(sn, m2, l2, cs, pp);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+#pragma unroll
+        for (int db = 0; db < 2; db++) {
+          typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+          typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+          const u32x2 lo = *reinterpret_cast<const u32x2*>(base + 8192 + (j * 4 + db * 2) * 512 + lane * 8);
+          const u32x2 hi = *reinterpret_cast<const u32x2*>(base + 8192 + (j * 4 + db * 2 + 1) * 512 + lane * 8);
+          const u32x4 av = {lo[0], lo[1], hi[0], hi[1]};
+          o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, av), pc.v[j], o[db], 0, 0, 0);
+          o2[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, av), pp.v[j], o2[db], 0, 0, 0);
         }
       }
     } else if (FORM == kChain) {
@@ -182,9 +216,9 @@ __global__ void __launch_bounds__(256, WAVES) step_kernel(const f16x8* __restric
     step(sb, sa, pb, pa);
   }
   if (FORM == kAheadPV) pv_mfma(o, V, pa);
-  float acc = l + m;
+  float acc = l + m + l2 + m2;
   for (int n = 0; n < 2; n++)
-    for (int i = 0; i < 16; i++) acc += o[n][i] + sa[n][i];
+    for (int i = 0; i < 16; i++) acc += o[n][i] + sa[n][i] + o2[n][i];
   out[blockIdx.x * 256 + tid] = acc;
   if (blockIdx.x == 0 && tid == 0) { g_clk[0] = __builtin_readcyclecounter() - c0; g_clk[1] = wall_clock64() - w0; }
 }
@@ -208,9 +242,10 @@ static void run(const char* name) {
   ms /= 5;
   long long hc[2];
   hipMemcpyFromSymbol(hc, HIP_SYMBOL(g_clk), 16);
-  const double ghz = hc[0] / (hc[1] / 100.0) / 1e3, ns = ms * 1e6 / (iters * (double)WAVES);
-  printf("  %-46s %d waves/SIMD: %6.1f ns = %5.0f cycles per wave step, clock %.2f GHz", name, WAVES, ns, ns * ghz, ghz);
-  if (FORM != kValuOnly) printf(", %6.1f TFLOP/s", (double)blocks * 4 * iters * 16 * 32768.0 / ms / 1e9);
+  const int units = FORM == kChainLds2 ? 2 : 1;  // blocks of 32 query rows per wave and step
+  const double ghz = hc[0] / (hc[1] / 100.0) / 1e3, ns = ms * 1e6 / (iters * (double)WAVES * units);
+  printf("  %-46s %d waves/SIMD: %6.1f ns = %5.0f cycles per wave and 32-row step, clock %.2f GHz", name, WAVES, ns, ns * ghz, ghz);
+  if (FORM != kValuOnly) printf(", %6.1f TFLOP/s", (double)blocks * 4 * iters * units * 16 * 32768.0 / ms / 1e9);
   printf("\n");
 }
 
@@ -232,6 +267,7 @@ int main() {
   run<kChain, 0, 3>("chain: S -> softmax -> PV");
   run<kChainLds, 0, 2>("chain, K and V fragments read from LDS");
   run<kChainLds, 0, 4>("chain, K and V fragments read from LDS");
+  run<kChainLds2, 0, 2>("chain from LDS, 64 query rows per wave");
   run<kAhead, 0, 2>("next S ahead of the exponentials");
   run<kAhead, 16, 2>("next S ahead, 1 MFMA : 16 VALU");
   run<kAheadPV, 0, 2>("next S and previous PV ahead");
