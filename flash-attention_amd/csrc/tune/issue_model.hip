@@ -148,6 +148,11 @@ __global__ void __launch_bounds__(512) op_kernel(float* out, int iters) {
       if (OP == 3) us[i] = us[i] * 0x9E3779B9u + 12345u;
       if (OP == 4) us[i] = __umulhi(us[i], 0xD2511F53u);
       if (OP == 5) xs[i] = __builtin_amdgcn_rcpf(xs[i]);
+      if (OP == 6) {  // 32 x 32 -> 64-bit product, both halves used (one Philox multiply): v_mad_u64_u32
+        const unsigned long long pr = (unsigned long long)us[i] * 0xD2511F53u;
+        us[i] = (unsigned)(pr >> 32) ^ (unsigned)pr ^ us[(i + 1) & 7];
+      }
+      if (OP == 7) us[i] = us[i] ^ us[(i + 1) & 7] ^ us[(i + 3) & 7];  // v_bitop3_b32
     }
   }
   float s = 0;
@@ -260,6 +265,8 @@ int main() {
   run_op<2>("v_max_f32");
   run_op<3>("v_mul_lo_u32 + add");
   run_op<4>("v_mul_hi_u32");
+  run_op<6>("v_mad_u64_u32 + v_bitop3");
+  run_op<7>("v_bitop3_b32");
 
   printf("4. LDS read bandwidth, 8 waves per CU\n");
   int offs[64];
