@@ -41,8 +41,11 @@ def sparse_layout(torch, N, density=0.25, seed=0, rows_per_draw=1):
 
 
 class Workload:
-    def __init__(self, torch, B, H, D, N, dtype, causal=False, p=0.0, lens=None, seed=0, blockmask=None):
+    def __init__(self, torch, B, H, D, N, dtype, causal=False, p=0.0, lens=None, seed=0, blockmask=None, alibi=False):
         self.B, self.H, self.D, self.N, self.dtype, self.causal, self.p = B, H, D, N, dtype, causal, p
+        # ALiBi slopes 2^(-8 (h + 1) / H), one per head (the engine's attention-bias extension)
+        self.alibi = torch.tensor([2.0 ** (-8.0 * (h + 1) / H) for h in range(H)], dtype=torch.float32, device="cuda") \
+            if alibi else None
         self.blockmask = blockmask  # (N/16, N/256) bool: the block-sparse entry points are timed instead
         g = torch.Generator(device="cuda").manual_seed(seed)
         lens = lens or [N] * B
@@ -72,7 +75,7 @@ class Workload:
                                               self.scale, self.causal, False, None)
             return
         self.out, self.lse = be.fwd(q, k, v, self.cu, self.cu, self.max_s, self.max_s, self.p, self.scale, False,
-                                    self.causal, False, None)
+                                    self.causal, False, None, self.alibi)
 
     def backward(self, be, events=None):
         q, k, v = self.qkv[:, 0], self.qkv[:, 1], self.qkv[:, 2]
@@ -86,7 +89,7 @@ class Workload:
                 events[1].record()  # whole backward: the sparse entry point has no per-kernel hook
             return
         be.bwd(self.dout, q, k, v, self.out, self.lse, dq, dk, dv, self.cu, self.cu, self.max_s, self.max_s, self.p,
-               self.scale, False, self.causal, None, main_kernel_events=events)
+               self.scale, False, self.causal, None, main_kernel_events=events, alibi_slopes=self.alibi)
 
 
 def time_steps(torch, be, w, steps, warmup, settle_s=0.2):
@@ -147,10 +150,16 @@ def torch_attention_ms(torch, w, iters=8, want_memory=False):
     qkv.requires_grad_()
     ragged = min(w.lens) < N
     causal_mask = torch.triu(torch.ones(N, N, dtype=torch.bool, device="cuda"), 1) if w.causal else None
+    bias = None
+    if w.alibi is not None:  # (H, N, N) additive bias, as a model without a fused kernel would hold it
+        pos = torch.arange(N, device="cuda")
+        bias = (-w.alibi[:, None, None] * (pos[:, None] - pos[None, :]).abs()[None]).to(w.dtype)
 
     def step():
         q, k, v = qkv.unbind(dim=2)
         scores = torch.einsum("bthd,bshd->bhts", q * w.scale, k)
+        if bias is not None:
+            scores = scores + bias[None]
         if ragged:
             scores = scores.masked_fill(~keep[:, None, None, :], float("-inf"))
         if causal_mask is not None:
@@ -325,6 +334,7 @@ def main():
             ("GPT2 causal bf16 N=1024", dict(B=8, H=12, D=64, N=1024, dtype=torch.bfloat16, causal=True)),
             ("GPT2 causal bf16 N=2048", dict(B=8, H=12, D=64, N=2048, dtype=torch.bfloat16, causal=True)),
             ("GPT2 causal bf16 N=4096", dict(B=8, H=12, D=64, N=4096, dtype=torch.bfloat16, causal=True)),
+            ("  + ALiBi slopes, N=2048", dict(B=8, H=12, D=64, N=2048, dtype=torch.bfloat16, causal=True, alibi=True)),
             ("d128 fp16 N=2048", dict(B=16, H=12, D=128, N=2048, dtype=torch.float16)),
             ("d128 fp16 N=2048 causal", dict(B=16, H=12, D=128, N=2048, dtype=torch.float16, causal=True)),
             ("blocksparse 25% 16x256", dict(B=4, H=16, D=64, N=4096, dtype=torch.float16, blockmask=sparse_layout(torch, 4096))),

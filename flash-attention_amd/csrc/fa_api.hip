@@ -157,6 +157,8 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
                  stride_ok(a->o_row_stride) && stride_ok(a->o_head_stride),
              "row and head strides must be multiples of 8 elements in [0, 2^24)");
 
+  if (sparse && a->alibi_slopes) return fail(FA_ERR_UNSUPPORTED, "alibi_slopes are not supported together with a blockmask");
+
   const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, sparse);
   hipStream_t stream = reinterpret_cast<hipStream_t>(a->stream);
   const bool dropout = a->p_dropout > 0.f;
@@ -193,6 +195,7 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
   p.rp_keep = 1.f / p_keep;
   p.keep_thr = (uint32_t)std::floor(p_keep * 65535.0);  // fmha_api.cpp:110
   p.pk = make_key(a->philox_seed, a->philox_offset);
+  p.alibi = a->alibi_slopes;
   // short query side, long key side: split the keys over several workgroups if the caller brought the scratch for it
   const SplitPlan sp = split_plan(a->batch, a->nheads, a->head_dim, a->total_q, a->max_seqlen_q, a->max_seqlen_k, r.sq_r,
                                   a->is_causal != 0, sparse);
@@ -217,7 +220,7 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
     d.sq_r = r.sq_r; d.sk_r = r.sk_r;
     d.scale = a->softmax_scale;
     d.causal = a->is_causal != 0; d.dropout = dropout; d.sparse = sparse;
-    d.keep_thr = p.keep_thr; d.pk = p.pk; d.sp = p.sp;
+    d.keep_thr = p.keep_thr; d.pk = p.pk; d.sp = p.sp; d.alibi = p.alibi;
     FA_LAUNCH(fa::launch_dump_probs(d, a->dtype, stream));
   }
   return FA_OK;
@@ -230,6 +233,7 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
   if (rc) return rc;
   const bool sparse = a->blockmask != nullptr;
   FA_REQUIRE(sparse == want_block, want_block ? "fa_bwd_block needs a blockmask" : "fa_bwd takes no blockmask; call fa_bwd_block");
+  if (sparse && a->alibi_slopes) return fail(FA_ERR_UNSUPPORTED, "alibi_slopes are not supported together with a blockmask");
   FA_REQUIRE(a->dout && a->q && a->k && a->v && a->out && a->softmax_lse && a->dq && a->dk && a->dv && a->softmax_d &&
                  a->cu_seqlens_q && a->cu_seqlens_k, "NULL tensor pointer");
   FA_REQUIRE(aligned16(a->dout) && aligned16(a->q) && aligned16(a->k) && aligned16(a->v) && aligned16(a->out) &&
@@ -291,6 +295,7 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
   p.rp_keep = 1.f / p_keep;
   p.keep_thr = (uint32_t)std::floor(p_keep * 65535.0);
   p.pk = make_key(a->philox_seed, a->philox_offset);
+  p.alibi = a->alibi_slopes;
 
   // short query side, long key side: the dQ kernel would walk all keys with one workgroup per (batch, head)
   const SplitPlan sp = split_plan(a->batch, a->nheads, a->head_dim, a->total_q, a->max_seqlen_q, a->max_seqlen_k, r.sq_r,

@@ -69,7 +69,9 @@ __global__ void __launch_bounds__(256) dump_probs_kernel(const DumpParams p) {
     float s = 0.f;
     for (int d = 0; d < p.D; d++) s += (float)qp[d] * (float)kp[d];
     const float lse = p.lse[((int64_t)b * p.H + h) * p.sq_r + qrow];
-    val = __expf(s * p.scale - lse);
+    float x = s * p.scale;
+    if (p.alibi) x -= p.alibi[h] * fabsf((float)(key - qrow));
+    val = __expf(x - lse);
     if (p.dropout) {
       const uint32_t bits = dropout_keep_bits16(p.pk, (uint32_t)bh, (uint32_t)qrow >> 2, (uint32_t)key >> 2, p.keep_thr);
       dropped = !((bits >> (4 * (qrow & 3) + (key & 3))) & 1u);

@@ -53,7 +53,7 @@ struct BwdCfg {
   static constexpr int kMinBlocks = D <= 64 ? 2 : 1;
 };
 
-template <typename T, int D, bool kCausal, bool kDropout, bool kSparse>
+template <typename T, int D, bool kCausal, bool kDropout, bool kSparse, bool kAlibi = false>
 __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
   using Cfg = BwdCfg<T, D>;
   using E = Elem<T>;
@@ -164,6 +164,7 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
     }
 
   const float cs = p.scale_log2;
+  const float sl2 = kAlibi ? p.alibi[h] * kLog2e : 0.f;  // ALiBi slope in base-2 exponent units (see fa_fwd_kernel)
   // element offsets inside a tile of this lane's row fragments and of its transposed reads (rows +0 and +8)
   int foff[D / 16], tlo[DV / 32], thi[DV / 32];
 #pragma unroll
@@ -266,6 +267,7 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
         for (int r = 0; r < 16; r++)
           if (!rb_on[r >> 3]) s[r] = -INFINITY;
       }
+      const float dbase = (float)(key - m0 - qb * 32 - 4 * hf);  // key - query of register 0 (kAlibi)
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_l + qb * 32 + 8 * j + 4 * hf);
@@ -274,7 +276,9 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           const int r = 4 * j + i;
-          const float pe = fast_exp2(__builtin_fmaf(s[r], cs, -lse4[i]));
+          float e = -lse4[i];
+          if (kAlibi) e = __builtin_fmaf(__builtin_fabsf(dbase - (float)(8 * j + i)), -sl2, -lse4[i]);
+          const float pe = fast_exp2(__builtin_fmaf(s[r], cs, e));
           float dpe = dp[r];  // dP - Dk
           float pm = pe;
           if (kDropout && !keep.keep_col(r, p.keep_thr)) { dpe = nd4[i]; pm = 0.f; }  // dropped: M o dP = 0
@@ -364,7 +368,7 @@ struct DqCfg {
   static constexpr int CH = D / 8;
 };
 
-template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse>
+template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, bool kAlibi = false>
 __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq_kernel(const BwdParams p) {
   using Cfg = DqCfg<T, D, BN>;
   using E = Elem<T>;
@@ -476,6 +480,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
     for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
 
   const float cs = p.scale_log2;
+  const float sl2 = kAlibi ? p.alibi[h] * kLog2e : 0.f;  // ALiBi slope in base-2 exponent units (see fa_fwd_kernel)
   // element offsets inside a tile: row fragments of K (dual swizzle) and V, transposed reads of K (rows +0, +8)
   int kfoff[D / 16], vfoff[D / 16], tlo[DV / 32], thi[DV / 32];
 #pragma unroll
@@ -544,9 +549,16 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
         }
         KeepFields keep;
         if (kDropout) keep = keep_fields_row_layout(p.pk, (uint32_t)bh, qrow, n0 + kb * 32, hf);
+        const float dbase = (float)(n0 + kb * 32 + hf * 4 - qrow);  // key - query of register 0 (kAlibi)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          const float pe = fast_exp2(__builtin_fmaf(s[r], cs, -lse2));  // 0 for dead scores and switched-off rows
+          float e = -lse2;
+          if (kAlibi) {  // -slope2 * |key - query| - lse; under a causal mask live scores have key <= query
+            const float cr = (float)((r >> 2) * 8 + (r & 3));
+            e = kCausal ? __builtin_fmaf(cr, sl2, __builtin_fmaf(dbase, sl2, -lse2))
+                        : __builtin_fmaf(__builtin_fabsf(dbase + cr), -sl2, -lse2);
+          }
+          const float pe = fast_exp2(__builtin_fmaf(s[r], cs, e));  // 0 for dead scores and switched-off rows
           float dpe = kInitNegD ? dp[r] : dp[r] - dkv;  // dP - Dk
           if (kDropout && !keep.keep_row(r, p.keep_thr)) dpe = -dkv;
           s[r] = pe * dpe;  // dS'

@@ -36,7 +36,9 @@ struct FwdCfg {
   static constexpr int CH = D / 8;
 };
 
-template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse>
+// kAlibi: the score of (query i, key j) gets -slope[head] * |i - j| added after scaling.  The scores are then moved to the
+// softmax's own units (base-2 exponent) before the row maximum is taken, and the running maximum is kept in those units.
+template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, bool kAlibi = false>
 __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2) fa_fwd_kernel(const FwdParams p) {
   using Cfg = FwdCfg<T, D, BN>;
   using E = Elem<T>;
@@ -130,6 +132,8 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
   float l_i = 0.f;        // this lane's share of the running row sum (other share in lane^32)
 
   const float cs = p.scale_log2;
+  const float cse = kAlibi ? 1.f : cs;                           // units of the scores the softmax works on
+  const float sl2 = kAlibi ? p.alibi[h] * kLog2e : 0.f;          // slope in base-2 exponent units
   int voff[DV / 32];  // element offsets of this lane's transposed V reads and K row fragments inside a tile
 #pragma unroll
   for (int db = 0; db < DV / 32; db++) voff[db] = tr_off<D, kSwzTr>(0, db * 4, lane);
@@ -191,6 +195,19 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
             if (dead) s[kb][r] = -INFINITY;
           }
       }
+      if (kAlibi) {  // s <- s * scale * log2(e) - slope2 * |key - query|; dead scores stay -inf
+#pragma unroll
+        for (int kb = 0; kb < BN / 32; kb++) {
+          const float dbase = (float)(n0 + kb * 32 + hf * 4 - qrow);  // key - query of register 0
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const float cr = (float)((r >> 2) * 8 + (r & 3));
+            // under a causal mask every live score has key <= query: -|key - query| = key - query, linear in cr
+            const float bias = kCausal ? __builtin_fmaf(cr, sl2, sl2 * dbase) : -sl2 * __builtin_fabsf(dbase + cr);
+            s[kb][r] = __builtin_fmaf(s[kb][r], cs, bias);
+          }
+        }
+      }
       // ---- online softmax (fmha_fprop_kernel_1xN.h:408-454,560-611 restated for a register-resident row)
       float mt = s[0][0];
 #pragma unroll
@@ -202,22 +219,22 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
       // 2^kRescaleLog2 since it was set; until then P may exceed 1 by at most that factor, which the fp32 accumulators and
       // the fp16/bf16 rounding of P absorb, and the accumulators need no rescaling (numerator and denominator carry the
       // same factor, so the result is unchanged).
-      if (__builtin_expect(__any((mt - m_i) * cs > kRescaleLog2), 0)) {  // wave-uniform; true on the first tile
+      if (__builtin_expect(__any((mt - m_i) * cse > kRescaleLog2), 0)) {  // wave-uniform; true on the first tile
         const float m_new = fmaxf(m_i, mt);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = fast_exp2(m_i * cs - m_use * cs);
+        const float alpha = fast_exp2(m_i * cse - m_use * cse);
         m_i = m_new;
         l_i *= alpha;
 #pragma unroll
         for (int i = 0; i < DV / 32; i++) o_acc[i] = o_acc[i] * alpha;
       }
-      const float mc = ((m_i == -INFINITY) ? 0.f : m_i) * cs;
+      const float mc = ((m_i == -INFINITY) ? 0.f : m_i) * cse;
       float rs = 0.f;
 #pragma unroll
       for (int kb = 0; kb < BN / 32; kb++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          const float pe = fast_exp2(__builtin_fmaf(s[kb][r], cs, -mc));
+          const float pe = fast_exp2(kAlibi ? s[kb][r] - mc : __builtin_fmaf(s[kb][r], cs, -mc));
           s[kb][r] = pe;
           if (kDropout) rs += pe;
         }
@@ -262,7 +279,7 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
   const bool empty = !(l_tot > 0.f);  // also catches NaN (fmha_fprop_kernel_1xN.h:575,606)
   float inv = empty ? 1.f : fast_rcp(l_tot);
   if (kDropout) inv *= p.rp_keep;
-  const float lse_val = empty ? -INFINITY : (m_i * cs + fast_log2(l_tot)) * kLn2;
+  const float lse_val = empty ? -INFINITY : (m_i * cse + fast_log2(l_tot)) * kLn2;
   if (p.n_splits > 1) {  // partial result of this key split, fp32, merged by fwd_combine_kernel
     if (qrow < Lq) {
       if (hf == 0) p.lse_part[(((int64_t)split * p.B + b) * p.H + h) * p.sq_r + qrow] = lse_val;

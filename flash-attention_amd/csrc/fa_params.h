@@ -50,6 +50,7 @@ struct FwdParams {
   int n_splits;
   float* o_part;
   float* lse_part;
+  const float* alibi;  // null, or one slope per head: the score of (query i, key j) gets -slope * |i - j| added
 };
 
 struct DumpParams {  // return_softmax path
@@ -69,6 +70,7 @@ struct DumpParams {  // return_softmax path
   uint32_t keep_thr;
   PhiloxKey pk;
   SparseMaps sp;
+  const float* alibi;
 };
 
 struct BwdParams {
@@ -104,6 +106,7 @@ struct BwdParams {
   // writes its scaled fp32 partial dQ to dq_part [n_splits, total_q, H, d]; dq_combine_kernel sums them into dq.
   int n_splits;
   float* dq_part;
+  const float* alibi;  // as in FwdParams
 };
 
 // Sequence extent of batch entry b, clamped so that a cu_seqlens array that disagrees with the declared
@@ -155,6 +158,7 @@ inline int tile_grid(bool tile_major, int tiles_per_bh, int BH) {
 }
 
 // Launchers (defined in fa_fwd.hip / fa_bwd.hip / fa_aux.hip).  Return hipError_t of the launch.
+// p.alibi != null selects the ALiBi variants (not available together with sparse)
 hipError_t launch_fwd(const FwdParams& p, int dtype, int head_dim, bool causal, bool dropout, bool sparse,
                       hipStream_t stream);
 hipError_t launch_fwd_combine(const FwdParams& p, int dtype, int head_dim, hipStream_t stream);

@@ -44,6 +44,7 @@ class FwdArgs(ctypes.Structure):
         ("philox_seed", ctypes.c_uint64), ("philox_offset", ctypes.c_uint64),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("stream", ctypes.c_void_p),
+        ("alibi_slopes", ctypes.c_void_p),
     ]
 
 
@@ -73,6 +74,7 @@ class BwdArgs(ctypes.Structure):
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("stream", ctypes.c_void_p),
         ("ev_main_start", ctypes.c_void_p), ("ev_main_stop", ctypes.c_void_p),
+        ("alibi_slopes", ctypes.c_void_p),
     ]
 
 
@@ -230,8 +232,18 @@ def _raise(rc, lib):
     raise RuntimeError("flash_attn_gfx950 error %d: %s" % (rc, msg))
 
 
+def _check_alibi(alibi_slopes, nheads, device, sparse):
+    """alibi_slopes: None or nheads fp32 slopes on the tensors' device (an extension: the reference has no attention bias)."""
+    if alibi_slopes is None:
+        return None
+    _check(not sparse, "alibi_slopes are not supported together with a blockmask")
+    _check(alibi_slopes.device == device and alibi_slopes.dtype == torch.float32 and alibi_slopes.is_contiguous() and
+           tuple(alibi_slopes.shape) == (nheads,), "alibi_slopes must be a contiguous fp32 tensor of nheads slopes on the GPU")
+    return alibi_slopes.data_ptr()
+
+
 def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
-              zero_tensors, is_causal, return_softmax, gen):
+              zero_tensors, is_causal, return_softmax, gen, alibi_slopes=None):
     lib = load_library()
     code = _dtype_code(q)
     _check(q.dim() == 3, "q must be (total_q, nheads, head_size)")
@@ -282,6 +294,7 @@ def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_
         a.workspace = ws.data_ptr() if ws is not None else None
         a.workspace_bytes = ws_bytes
         a.stream = _stream_handle(dev)
+        a.alibi_slopes = _check_alibi(alibi_slopes, nheads, dev, sparse)
         rc = (lib.fa_fwd_block if sparse else lib.fa_fwd)(ctypes.byref(a))
         if rc != 0:
             _raise(rc, lib)
@@ -289,7 +302,8 @@ def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_
 
 
 def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q,
-              max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen, main_kernel_events=None):
+              max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen, main_kernel_events=None,
+              alibi_slopes=None):
     lib = load_library()
     code = _dtype_code(q)
     _check(q.dim() == 3, "q must be (total_q, nheads, head_size)")
@@ -354,6 +368,7 @@ def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seql
                     ev.record()
             a.ev_main_start = main_kernel_events[0].cuda_event
             a.ev_main_stop = main_kernel_events[1].cuda_event
+        a.alibi_slopes = _check_alibi(alibi_slopes, nheads, dev, sparse)
         rc = (lib.fa_bwd_block if sparse else lib.fa_bwd)(ctypes.byref(a))
         if rc != 0:
             _raise(rc, lib)
@@ -361,18 +376,20 @@ def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seql
 
 
 def fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors,
-        is_causal, return_softmax, gen=None):
-    """mha_fwd (fmha_api.cpp:173-299): returns [o, softmax_lse] or [o, softmax_lse, s]."""
+        is_causal, return_softmax, gen=None, alibi_slopes=None):
+    """mha_fwd (fmha_api.cpp:173-299): returns [o, softmax_lse] or [o, softmax_lse, s].
+    alibi_slopes (extension, not in the reference): nheads fp32 slopes; scores get -slope * |i - j| added."""
     return _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, None, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
-                     zero_tensors, is_causal, return_softmax, gen)
+                     zero_tensors, is_causal, return_softmax, gen, alibi_slopes)
 
 
 def bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-        p_dropout, softmax_scale, zero_tensors, is_causal, gen=None, main_kernel_events=None):
+        p_dropout, softmax_scale, zero_tensors, is_causal, gen=None, main_kernel_events=None, alibi_slopes=None):
     """mha_bwd (fmha_api.cpp:302-449): fills dq, dk, dv in place, returns [dq, dk, dv, softmax_d].
-    main_kernel_events: optional (start, stop) timing events recorded around the dq/dk/dv kernel alone."""
+    main_kernel_events: optional (start, stop) timing events recorded around the dq/dk/dv kernel alone.
+    alibi_slopes: the slopes the forward was given (extension, not in the reference)."""
     return _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, None, max_seqlen_q,
-                     max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen, main_kernel_events)
+                     max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen, main_kernel_events, alibi_slopes)
 
 
 def fwd_block(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,

@@ -16,16 +16,17 @@ def _get_block_size(device, head_dim, is_dropout):
 
 
 def _flash_attn_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-                        softmax_scale, causal, return_softmax):
+                        softmax_scale, causal, return_softmax, alibi_slopes=None):
     res = _backend.fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale,
-                       False, causal, return_softmax, None)
+                       False, causal, return_softmax, None, alibi_slopes)
     return res[0], res[1], (res[2] if return_softmax else None)
 
 
 def _flash_attn_backward(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
-                         max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal):
+                         max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal, alibi_slopes=None):
     _, _, _, softmax_d = _backend.bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
-                                      max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, False, causal, None)
+                                      max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, False, causal, None,
+                                      alibi_slopes=alibi_slopes)
     return dq, dk, dv, softmax_d
 
 
@@ -41,15 +42,16 @@ def _split(packing, tensors):
 
 
 def _forward(ctx, packing, tensors, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-             softmax_scale, causal, return_softmax):
+             softmax_scale, causal, return_softmax, alibi_slopes=None):
     q, k, v = _split(packing, tensors)
     # the dropout mask is a function of the generator state at this point; the backward rewinds to it
     rng_state = torch.cuda.get_rng_state(q.device) if dropout_p > 0 else None
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
     out, softmax_lse, S_dmask = _flash_attn_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-                                                    dropout_p, softmax_scale, causal, return_softmax)
+                                                    dropout_p, softmax_scale, causal, return_softmax, alibi_slopes)
     ctx.save_for_backward(*tensors, out, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state)
+    ctx.alibi_slopes = alibi_slopes  # fixed slopes, not differentiated
     ctx.packing = packing
     ctx.n_in = len(tensors)
     ctx.dropout_p = dropout_p
@@ -71,23 +73,25 @@ def _backward(ctx, dout):
         cur_rng_state = torch.cuda.get_rng_state(dev)
         torch.cuda.set_rng_state(rng_state, dev)
     _flash_attn_backward(dout.contiguous(), q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
-                         ctx.max_seqlen_q, ctx.max_seqlen_k, ctx.dropout_p, ctx.softmax_scale, ctx.causal)
+                         ctx.max_seqlen_q, ctx.max_seqlen_k, ctx.dropout_p, ctx.softmax_scale, ctx.causal,
+                         ctx.alibi_slopes)
     if rng_state is not None:
         torch.cuda.set_rng_state(cur_rng_state, dev)
     return grads
 
 
 class FlashAttnQKVPackedFunc(torch.autograd.Function):
-    """apply(qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal, return_softmax)"""
+    """apply(qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal, return_softmax[, alibi_slopes])"""
 
     @staticmethod
-    def forward(ctx, qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal, return_softmax):
+    def forward(ctx, qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal, return_softmax, *alibi_slopes):
+        ctx.n_extra = 6 + len(alibi_slopes)  # the reference's six non-tensor arguments (:72), plus the optional slopes
         return _forward(ctx, "qkv", (qkv,), cu_seqlens, cu_seqlens, max_seqlen, max_seqlen, dropout_p, softmax_scale,
-                        causal, return_softmax)
+                        causal, return_softmax, *alibi_slopes)
 
     @staticmethod
     def backward(ctx, dout, *args):
-        return _backward(ctx, dout) + (None,) * 6
+        return _backward(ctx, dout) + (None,) * ctx.n_extra
 
 
 class FlashAttnKVPackedFunc(torch.autograd.Function):
@@ -96,13 +100,14 @@ class FlashAttnKVPackedFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, kv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal,
-                return_softmax):
+                return_softmax, *alibi_slopes):
+        ctx.n_extra = 8 + len(alibi_slopes)  # :111
         return _forward(ctx, "kv", (q, kv), cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-                        softmax_scale, causal, return_softmax)
+                        softmax_scale, causal, return_softmax, *alibi_slopes)
 
     @staticmethod
     def backward(ctx, dout, *args):
-        return _backward(ctx, dout) + (None,) * 8
+        return _backward(ctx, dout) + (None,) * ctx.n_extra
 
 
 class FlashAttnFunc(torch.autograd.Function):
@@ -111,13 +116,14 @@ class FlashAttnFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal,
-                return_softmax):
+                return_softmax, *alibi_slopes):
+        ctx.n_extra = 8 + len(alibi_slopes)  # :148
         return _forward(ctx, "sep", (q, k, v), cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-                        softmax_scale, causal, return_softmax)
+                        softmax_scale, causal, return_softmax, *alibi_slopes)
 
     @staticmethod
     def backward(ctx, dout, *args):
-        return _backward(ctx, dout) + (None,) * 8
+        return _backward(ctx, dout) + (None,) * ctx.n_extra
 
 
 _COMMON_DOC = """
@@ -131,6 +137,9 @@ _COMMON_DOC = """
         softmax_scale: float, multiplies Q K^T before the softmax; defaults to headdim ** -0.5.
         causal: bool, query i of a sequence attends only to keys j <= i of that sequence.
         return_attn_probs: bool, testing aid.
+        alibi_slopes: None, or (nheads,) fp32 on the GPU.  Not in the reference (its README lists attention bias as
+            planned): the score of query i and key j, positions counted inside their sequences, becomes
+            softmax_scale * q_i.k_j - alibi_slopes[head] * |i - j|.  The slopes are constants (no gradient).
     Returns
         out: (total_q, nheads, headdim).
         With return_attn_probs=True additionally
@@ -141,25 +150,25 @@ _COMMON_DOC = """
 
 
 def flash_attn_unpadded_qkvpacked_func(qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale=None,
-                                       causal=False, return_attn_probs=False):
+                                       causal=False, return_attn_probs=False, alibi_slopes=None):
     """Self-attention on a packed (total, 3, nheads, headdim) tensor of variable-length sequences."""
     return FlashAttnQKVPackedFunc.apply(qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal,
-                                        return_attn_probs)
+                                        return_attn_probs, alibi_slopes)
 
 
 def flash_attn_unpadded_kvpacked_func(q, kv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
                                       dropout_p, softmax_scale=None, causal=False,
-                                      return_attn_probs=False):
+                                      return_attn_probs=False, alibi_slopes=None):
     """Attention of q (total_q, nheads, headdim) over packed keys/values kv (total_k, 2, nheads, headdim)."""
     return FlashAttnKVPackedFunc.apply(q, kv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-                                       softmax_scale, causal, return_attn_probs)
+                                       softmax_scale, causal, return_attn_probs, alibi_slopes)
 
 
 def flash_attn_unpadded_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-                             dropout_p, softmax_scale=None, causal=False, return_attn_probs=False):
+                             dropout_p, softmax_scale=None, causal=False, return_attn_probs=False, alibi_slopes=None):
     """Attention of q (total_q, nheads, headdim) over k, v (total_k, nheads, headdim)."""
     return FlashAttnFunc.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-                               softmax_scale, causal, return_attn_probs)
+                               softmax_scale, causal, return_attn_probs, alibi_slopes)
 
 
 def flash_attn_func(qkv, cu_seqlens, dropout_p, max_s, softmax_scale=None, causal=False,

@@ -70,6 +70,10 @@ typedef struct fa_fwd_args {
   void* workspace; /* device scratch of >= fa_fwd_workspace_bytes() bytes (may be NULL if that is 0) */
   size_t workspace_bytes;
   void* stream; /* hipStream_t */
+  /* Attention bias (no counterpart in the reference's entry points; its README lists "attention bias (e.g. ALiBi)" as
+   * planned, README.md:49-50).  NULL, or a device array of nheads fp32 slopes: softmax_scale * q.k - slope[h] * |i - j|
+   * is what the softmax sees, i and j being the positions of query and key in their sequences.  Not with a blockmask. */
+  const float* alibi_slopes;
 } fa_fwd_args;
 
 /* Arguments of the backward pass.  Mirrors mha_bwd (fmha_api.cpp:302-321) and, when `blockmask`
@@ -115,6 +119,7 @@ typedef struct fa_bwd_args {
    * kernel, the longer of the two kernels of a backward call (dQ + softmax_d kernel, dK/dV kernel). */
   void* ev_main_start;
   void* ev_main_stop;
+  const float* alibi_slopes; /* as in fa_fwd_args: the slopes the forward was given */
 } fa_bwd_args;
 
 /* replaces flash_attn_cuda.fwd -> mha_fwd, csrc/flash_attn/fmha_api.cpp:173-299 */

@@ -14,6 +14,7 @@ It restates, in plain fp32/fp64 PyTorch and NumPy on the host, the algorithm of 
   convert_blockmask_ref    specification of flash_attn/flash_blocksparse_attn_interface.py:8-40
   unpad_ref / pad_ref      specification of flash_attn/bert_padding.py:60-95
   rotary_ref               rotation of flash_attn/rotary.py:22-42 (x * cos + rotate_half(x) * sin) in fp64
+  alibi_bias               -slope * |i - j| score bias of the engine's alibi_slopes extension (no reference counterpart)
 
 How each function is pinned (the reference has no tests, golden vectors or fixtures of its own):
   attention_ref / varlen_attention forward: against torch.nn.functional.scaled_dot_product_attention (library
@@ -25,6 +26,8 @@ How each function is pinned (the reference has no tests, golden vectors or fixtu
       the reference uses (tests/golden/philox_kat.json).
   dropout_keep_mask: it is the definition; tests compare the kernels' S_dmask signs to it bit for bit.
   convert_blockmask_ref: brute force over all small masks against an independent per-element definition.
+  alibi_bias (inside varlen_attention): torch's scaled_dot_product_attention with the same bias as a float attn_mask;
+      slope 0 is no bias; a bias that is constant along a row changes nothing.
   unpad_ref / pad_ref: round trip pad(unpad(x)) == x * mask, cu_seqlens against the cumulative sum of the lengths.
   rotary_ref: the cited definition evaluated literally; it is a rotation (norm kept, conjugate inverts it, angles add,
       position 0 is the identity).
@@ -80,8 +83,17 @@ def _score_mask(Lq, Lk, causal, layout, device="cpu"):
     return valid
 
 
+def alibi_bias(slopes, Lq, Lk, device="cpu", dtype=torch.float32):
+    """(H, Lq, Lk) additive score bias -slope[h] * |i - j| (ALiBi, Press et al. 2021, mirrored for keys after the
+    query).  The reference has no attention bias (its README lists it as planned, README.md:49-50); this is the
+    definition the engine's alibi_slopes extension follows."""
+    sl = torch.as_tensor(slopes, dtype=dtype, device=device)
+    dist = (torch.arange(Lq, device=device)[:, None] - torch.arange(Lk, device=device)[None, :]).abs().to(dtype)
+    return -sl[:, None, None] * dist[None]
+
+
 def varlen_attention(q, k, v, cu_q, cu_k, softmax_scale=None, causal=False, p_dropout=0.0, keep_mask=None,
-                     layout=None, dout=None, dtype=torch.float32):
+                     layout=None, dout=None, dtype=torch.float32, alibi_slopes=None):
     """Closed-form attention forward (+ backward if dout is given) on packed tensors.
 
     q (total_q, H, D), k, v (total_k, H, D) any float dtype (upcast to `dtype`); cu_q, cu_k int sequences of length
@@ -106,6 +118,8 @@ def varlen_attention(q, k, v, cu_q, cu_k, softmax_scale=None, causal=False, p_dr
         vb = vf[cu_k[b]:cu_k[b + 1]].transpose(0, 1)
         Lq, Lk = qb.shape[1], kb.shape[1]
         s = torch.einsum("hqd,hkd->hqk", qb, kb) * scale
+        if alibi_slopes is not None:
+            s = s + alibi_bias(alibi_slopes, Lq, Lk, qf.device, dtype)
         valid = _score_mask(Lq, Lk, causal, layout, qf.device)
         s = s.masked_fill(~valid[None], float("-inf"))
         lse = torch.logsumexp(s, dim=-1)  # -inf for empty rows

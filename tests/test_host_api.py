@@ -154,17 +154,20 @@ def test_public_signatures_match_the_reference():
         return [(n, p.default if p.default is not inspect.Parameter.empty else "<req>")
                 for n, p in inspect.signature(f).parameters.items()]
 
+    # the three functions that reach the kernels take the reference's parameters followed by one extension,
+    # alibi_slopes=None (attention bias: planned in the reference's README, absent from its API)
+    ext = [("alibi_slopes", None)]
     assert sig(fi.flash_attn_unpadded_qkvpacked_func) == [
         ("qkv", "<req>"), ("cu_seqlens", "<req>"), ("max_seqlen", "<req>"), ("dropout_p", "<req>"),
-        ("softmax_scale", None), ("causal", False), ("return_attn_probs", False)]
+        ("softmax_scale", None), ("causal", False), ("return_attn_probs", False)] + ext
     assert sig(fi.flash_attn_unpadded_kvpacked_func) == [
         ("q", "<req>"), ("kv", "<req>"), ("cu_seqlens_q", "<req>"), ("cu_seqlens_k", "<req>"),
         ("max_seqlen_q", "<req>"), ("max_seqlen_k", "<req>"), ("dropout_p", "<req>"), ("softmax_scale", None),
-        ("causal", False), ("return_attn_probs", False)]
+        ("causal", False), ("return_attn_probs", False)] + ext
     assert sig(fi.flash_attn_unpadded_func) == [
         ("q", "<req>"), ("k", "<req>"), ("v", "<req>"), ("cu_seqlens_q", "<req>"), ("cu_seqlens_k", "<req>"),
         ("max_seqlen_q", "<req>"), ("max_seqlen_k", "<req>"), ("dropout_p", "<req>"), ("softmax_scale", None),
-        ("causal", False), ("return_attn_probs", False)]
+        ("causal", False), ("return_attn_probs", False)] + ext
     assert sig(fi.flash_attn_func) == [
         ("qkv", "<req>"), ("cu_seqlens", "<req>"), ("dropout_p", "<req>"), ("max_s", "<req>"),
         ("softmax_scale", None), ("causal", False), ("return_attn_probs", False)]
@@ -178,7 +181,7 @@ def test_public_signatures_match_the_reference():
     from flash_attn import flash_attn_gfx950 as be
     assert list(inspect.signature(be.fwd).parameters) == [
         "q", "k", "v", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k", "p_dropout", "softmax_scale",
-        "zero_tensors", "is_causal", "return_softmax", "gen"]                      # fmha_api.cpp:173-186
+        "zero_tensors", "is_causal", "return_softmax", "gen", "alibi_slopes"]      # fmha_api.cpp:173-186 + extension
     assert list(inspect.signature(be.bwd_block).parameters) == [
         "dout", "q", "k", "v", "out", "softmax_lse", "dq", "dk", "dv", "cu_seqlens_q", "cu_seqlens_k", "blockmask",
         "max_seqlen_q", "max_seqlen_k", "p_dropout", "softmax_scale", "is_causal", "gen"]  # fmha_api.cpp:575-594

@@ -44,8 +44,8 @@ def _pick(res, *parts):
 def test_d64_kernels_keep_their_waves_per_simd():
     fwd = _resources("fa_fwd_d64.hip")
     bwd = _resources("fa_bwd_d64.hip")
-    # <f16, 64, ..., causal, dropout, sparse> mangled as ...IDF16_Li64E...Lb{0,1}E x3
-    plain, causal, dropout = "Lb0ELb0ELb0E", "Lb1ELb0ELb0E", "Lb0ELb1ELb0E"
+    # <f16, 64, ..., causal, dropout, sparse, alibi> mangled as ...IDF16_Li64E...Lb{0,1}E x4
+    plain, causal, dropout = "Lb0ELb0ELb0ELb0E", "Lb1ELb0ELb0ELb0E", "Lb0ELb1ELb0ELb0E"
     for flags, want in ((plain, 4), (causal, 4), (dropout, 3)):
         k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags)
         assert k["Occupancy"] >= want and k["VGPRs Spill"] == 0, ("forward", flags, k)

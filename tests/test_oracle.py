@@ -276,3 +276,27 @@ def test_rotary_ref_is_a_rotation_and_matches_the_elementwise_definition():
     twice = orc.rotary_ref(orc.rotary_ref(x, cos_h, sin_h, np.full(rows, 4)), cos_h, sin_h, np.full(rows, 9))
     assert np.allclose(twice, orc.rotary_ref(x, cos_h, sin_h, np.full(rows, 13)), atol=1e-13)
     assert np.allclose(orc.rotary_ref(x, cos_h, sin_h, np.zeros(rows, dtype=int)), x)
+
+
+def test_alibi_bias_against_sdpa_float_mask():
+    """varlen_attention with alibi_slopes against torch's scaled_dot_product_attention given the same bias as a float
+    attn_mask (library routine), with and without a causal mask; slope 0 is no bias; gradients flow the same way."""
+    g = torch.Generator().manual_seed(21)
+    H, D, Lq, Lk = 3, 16, 37, 37
+    q, k, v, do = (torch.randn(L, H, D, generator=g, dtype=torch.float64) for L in (Lq, Lk, Lk, Lq))
+    slopes = torch.tensor([0.5, 0.0625, 0.0])
+    cu = [0, Lq]
+    for causal in (False, True):
+        res = orc.varlen_attention(q, k, v, cu, cu, None, causal, dout=do, dtype=torch.float64, alibi_slopes=slopes)
+        bias = orc.alibi_bias(slopes, Lq, Lk, dtype=torch.float64)
+        if causal:
+            bias = bias.masked_fill(torch.triu(torch.ones(Lq, Lk, dtype=torch.bool), 1), float("-inf"))
+        qq, kk, vv = (x.transpose(0, 1).clone().requires_grad_() for x in (q, k, v))
+        ref = torch.nn.functional.scaled_dot_product_attention(qq[None], kk[None], vv[None], attn_mask=bias[None])[0]
+        ref.backward(do.transpose(0, 1))
+        assert torch.allclose(res["out"].transpose(0, 1), ref, atol=1e-12)
+        for name, t in (("dq", qq), ("dk", kk), ("dv", vv)):
+            assert torch.allclose(res[name].transpose(0, 1), t.grad, atol=1e-11), name
+        plain = orc.varlen_attention(q, k, v, cu, cu, None, causal, dtype=torch.float64)
+        assert torch.equal(res["out"][:, 2], plain["out"][:, 2])          # head with slope 0
+        assert not torch.allclose(res["out"][:, 0], plain["out"][:, 0], atol=1e-3)

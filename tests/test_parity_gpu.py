@@ -46,7 +46,7 @@ def _inputs(lens_q, lens_k, H, D, dtype, seed):
     return mk(tq), mk(tk), mk(tk), mk(tq)
 
 
-def half_attention(q, k, v, cu_q, cu_k, scale, causal, keep_mask=None, p=0.0, layout=None, dout=None):
+def half_attention(q, k, v, cu_q, cu_k, scale, causal, keep_mask=None, p=0.0, layout=None, dout=None, alibi_slopes=None):
     """the closed form evaluated in the tensors' own half dtype by PyTorch (the error yardstick)"""
     q, k, v = (x.detach().clone().requires_grad_(dout is not None) for x in (q, k, v))
     outs = []
@@ -55,6 +55,8 @@ def half_attention(q, k, v, cu_q, cu_k, scale, causal, keep_mask=None, p=0.0, la
         kb = k[cu_k[b]:cu_k[b + 1]].transpose(0, 1)
         vb = v[cu_k[b]:cu_k[b + 1]].transpose(0, 1)
         s = torch.matmul(qb, kb.transpose(1, 2)) * scale
+        if alibi_slopes is not None:
+            s = s + orc.alibi_bias(alibi_slopes, qb.shape[1], kb.shape[1], q.device).to(s.dtype)
         valid = orc._score_mask(qb.shape[1], kb.shape[1], causal, layout, q.device)
         s = s.masked_fill(~valid[None], float("-inf"))
         empty = ~valid.any(-1)
@@ -85,20 +87,22 @@ def check_against_oracle(ours, ref, half, dtype, names=("out", "dq", "dk", "dv")
         assert e_ours <= 2 * e_half + floor, "%s %s: ours %.3e vs half-precision PyTorch %.3e" % (what, n, e_ours, e_half)
 
 
-def run_ours(q, k, v, do, cu_q, cu_k, max_q, max_k, p, scale, causal, packing="sep", probs=False):
+def run_ours(q, k, v, do, cu_q, cu_k, max_q, max_k, p, scale, causal, packing="sep", probs=False, alibi_slopes=None):
     from flash_attn import flash_attn_interface as fi
     dev = "cuda"
     cu_q, cu_k = cu_q.to(dev), cu_k.to(dev)
     if packing == "qkv":
         qkv = torch.stack([q, k, v], 1).to(dev).requires_grad_()
-        res = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu_q, max_q, p, scale, causal, probs)
+        res = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu_q, max_q, p, scale, causal, probs, alibi_slopes=alibi_slopes)
     elif packing == "kv":
         qg = q.to(dev).requires_grad_()
         kv = torch.stack([k, v], 1).to(dev).requires_grad_()
-        res = fi.flash_attn_unpadded_kvpacked_func(qg, kv, cu_q, cu_k, max_q, max_k, p, scale, causal, probs)
+        res = fi.flash_attn_unpadded_kvpacked_func(qg, kv, cu_q, cu_k, max_q, max_k, p, scale, causal, probs,
+                                                   alibi_slopes=alibi_slopes)
     else:
         qg, kg, vg = (x.to(dev).requires_grad_() for x in (q, k, v))
-        res = fi.flash_attn_unpadded_func(qg, kg, vg, cu_q, cu_k, max_q, max_k, p, scale, causal, probs)
+        res = fi.flash_attn_unpadded_func(qg, kg, vg, cu_q, cu_k, max_q, max_k, p, scale, causal, probs,
+                                          alibi_slopes=alibi_slopes)
     out = res[0] if probs else res
     out.backward(do.to(dev))
     torch.cuda.synchronize()
@@ -471,6 +475,99 @@ def test_parity_random_shapes_sweep():
         print("case %d: D=%d %s B=%d H=%d causal=%s q=%s k=%s %s scale=%s" % (case, D, dtype, B, H, causal, lens_q, lens_k,
                                                                             packing, scale), flush=True)
         _parity_case(lens_q, lens_k, H, D, dtype, causal, packing=packing, seed=100 + case, scale=scale)
+
+
+# ------------------------------------------------------------------------------------------------
+# attention bias: ALiBi slopes (an extension; the reference's README lists attention bias as planned)
+# ------------------------------------------------------------------------------------------------
+def _alibi_slopes(H):
+    """the geometric sequence of the ALiBi paper for a power-of-two head count, cut to H heads"""
+    n = 1 << max(1, (H - 1).bit_length())
+    return torch.tensor([2.0 ** (-8.0 * (i + 1) / n) for i in range(H)], dtype=torch.float32)
+
+
+def test_alibi_random_shapes_sweep():
+    """Sixteen seeded cases with per-head ALiBi slopes: every head dim, both dtypes, causal and not, ragged self- and
+    cross-attention lengths, all packings, with and without dropout; out, lse, dq, dk, dv and the returned probabilities
+    against the closed form with the bias added to the scaled scores."""
+    rng = np.random.default_rng(909)
+    for case in range(16):
+        D = int(rng.choice([16, 32, 64, 128]))
+        dtype = torch.float16 if rng.integers(2) else torch.bfloat16
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 5))
+        causal = bool(rng.integers(2))
+        cross = bool(rng.integers(2)) and not causal
+        top = int(rng.choice([40, 150, 300, 520]))
+        lens_q = [int(x) for x in rng.integers(1, top + 1, B)]
+        lens_k = [int(x) for x in rng.integers(1, top + 1, B)] if cross else list(lens_q)
+        packing = "kv" if cross else str(rng.choice(["qkv", "kv", "sep"]))
+        p = float(rng.choice([0.0, 0.0, 0.15]))
+        slopes = _alibi_slopes(H) * float(rng.choice([1.0, 4.0]))
+        what = "case %d: D=%d %s B=%d H=%d causal=%s q=%s k=%s %s p=%.2f" % (case, D, dtype, B, H, causal, lens_q, lens_k,
+                                                                          packing, p)
+        print(what, flush=True)
+        q, k, v, do = _inputs(lens_q, lens_k, H, D, dtype, 700 + case)
+        cu_q, cu_k = _cu(lens_q, "cpu"), _cu(lens_k, "cpu")
+        sc = D ** -0.5
+        torch.manual_seed(case)
+        seed, offset = _gen_state()
+        ours = run_ours(q, k, v, do, cu_q, cu_k, max(lens_q), max(lens_k), p, None, causal, packing, probs=True,
+                        alibi_slopes=slopes.cuda())
+        masks = None
+        if p > 0:
+            masks = [torch.tensor(np.stack([orc.dropout_keep_mask(seed, offset, b * H + h, lens_q[b], lens_k[b], p)
+                                            for h in range(H)])) for b in range(B)]
+        ref = orc.varlen_attention(q, k, v, cu_q, cu_k, sc, causal, p_dropout=p, keep_mask=masks, dout=do,
+                                   alibi_slopes=slopes)
+        half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu_q.tolist(), cu_k.tolist(), sc, causal, masks, p, dout=do.cuda(),
+                              alibi_slopes=slopes)
+        check_against_oracle(ours, ref, half, dtype, what=what)
+        for b in range(B):
+            Lq, Lk = lens_q[b], lens_k[b]
+            got, want = ours["lse"][b, :, :Lq].cpu(), ref["lse"][b]
+            fin = torch.isfinite(want)
+            assert torch.equal(torch.isfinite(got), fin), what
+            if fin.any():
+                assert (got[fin] - want[fin]).abs().max().item() <= LSE_TOL[dtype], what
+            probs = ours["S_dmask"][b, :, :Lq, :Lk].float().cpu()
+            assert (probs.abs() - ref["probs"][b]).abs().max().item() < (2e-3 if dtype == torch.float16 else 1e-2), what
+
+
+def test_alibi_headline_shape_and_errors():
+    """ALiBi at the headline shape (all tiles full, no masking code in the way) against the fp32 closed form on the GPU
+    for one (batch, head) pair, slope 0 == no bias bit for bit, and the refusals: slopes of the wrong shape / dtype /
+    device, slopes together with a block layout."""
+    from flash_attn import flash_attn_interface as fi
+    from flash_attn.flash_blocksparse_attn_interface import convert_blockmask
+    from flash_attn import flash_attn_gfx950 as be
+    B, H, D, N = 2, 4, 64, 2048
+    g = torch.Generator(device="cuda").manual_seed(2)
+    qkv = torch.randn(B * N, 3, H, D, device="cuda", dtype=torch.float16, generator=g).requires_grad_()
+    do = torch.randn(B * N, H, D, device="cuda", dtype=torch.float16, generator=g)
+    cu = _cu([N] * B)
+    slopes = _alibi_slopes(H).cuda()
+    out = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0, causal=True, alibi_slopes=slopes)
+    out.backward(do)
+    torch.cuda.synchronize()
+    b, h = 1, 2
+    sl = slice(b * N, (b + 1) * N)
+    q, k, v = (qkv[sl, i, h].detach().float()[:, None] for i in range(3))
+    ref = orc.varlen_attention(q, k, v, [0, N], [0, N], None, True, dout=do[sl, h].float()[:, None],
+                               alibi_slopes=slopes[h:h + 1].cpu())
+    assert (out[sl, h].detach().float() - ref["out"][:, 0]).abs().max() < 2e-3
+    for i, name in enumerate(("dq", "dk", "dv")):
+        assert (qkv.grad[sl, i, h].float() - ref[name][:, 0]).abs().max() < 4e-3, name
+    plain = fi.flash_attn_unpadded_qkvpacked_func(qkv.detach(), cu, N, 0.0, causal=True)
+    zero = fi.flash_attn_unpadded_qkvpacked_func(qkv.detach(), cu, N, 0.0, causal=True, alibi_slopes=torch.zeros_like(slopes))
+    assert (zero.float() - plain.float()).abs().max() < 1e-3  # different kernel variants, same mathematics
+    for bad in (slopes[:3], slopes.double(), slopes.cpu(), slopes[None]):
+        with pytest.raises(RuntimeError):
+            fi.flash_attn_unpadded_qkvpacked_func(qkv.detach(), cu, N, 0.0, alibi_slopes=bad)
+    sq_r, sk_r = be.round_seqlens(D, N, N, True)
+    bm = convert_blockmask(torch.ones(sq_r // 16, sk_r // 256, device="cuda"), causal=False)
+    q3 = qkv.detach()
+    with pytest.raises(RuntimeError):
+        be._fwd_impl(q3[:, 0], q3[:, 1], q3[:, 2], cu, cu, bm, N, N, 0.0, D ** -0.5, False, False, False, None, slopes)
 
 
 # ------------------------------------------------------------------------------------------------
