@@ -533,6 +533,26 @@ def test_alibi_random_shapes_sweep():
             assert (probs.abs() - ref["probs"][b]).abs().max().item() < (2e-3 if dtype == torch.float16 else 1e-2), what
 
 
+def test_alibi_decode_shape_with_key_split():
+    """A few query rows against thousands of keys with ALiBi slopes: the key-split forward and the key-split dQ kernel
+    (partial results per key range, merged by a second launch) see the bias through the same scores."""
+    lens_q, lens_k, H, D = [3, 1], [4100, 2900], 4, 64
+    slopes = _alibi_slopes(H) * 0.25
+    q, k, v, do = _inputs(lens_q, lens_k, H, D, torch.float16, 77)
+    cu_q, cu_k = _cu(lens_q, "cpu"), _cu(lens_k, "cpu")
+    ours = run_ours(q, k, v, do, cu_q, cu_k, max(lens_q), max(lens_k), 0.0, None, False, "kv", probs=True,
+                    alibi_slopes=slopes.cuda())
+    ref = orc.varlen_attention(q, k, v, cu_q, cu_k, None, False, dout=do, alibi_slopes=slopes)
+    half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu_q.tolist(), cu_k.tolist(), D ** -0.5, False, dout=do.cuda(),
+                          alibi_slopes=slopes)
+    check_against_oracle(ours, ref, half, torch.float16, what="alibi decode shape")
+    for b, L in enumerate(lens_q):
+        assert (ours["lse"][b, :, :L].cpu() - ref["lse"][b]).abs().max() <= LSE_TOL[torch.float16]
+    # the bias matters here: without it the result is visibly different
+    plain = orc.varlen_attention(q, k, v, cu_q, cu_k, None, False)
+    assert (plain["out"] - ref["out"]).abs().max() > 0.05
+
+
 def test_alibi_headline_shape_and_errors():
     """ALiBi at the headline shape (all tiles full, no masking code in the way) against the fp32 closed form on the GPU
     for one (batch, head) pair, slope 0 == no bias bit for bit, and the refusals: slopes of the wrong shape / dtype /
