@@ -776,6 +776,13 @@ def test_flash_attention_module_three_input_modes():
     class KPM:
         bool_matrix = mask.cuda()
 
+    # ALiBi slopes through the module (padded input with a key padding mask)
+    slopes = _alibi_slopes(H)
+    out_al, _ = m(qkv.cuda(), key_padding_mask=KPM(), causal=True, alibi_slopes=slopes.cuda())
+    for b in range(B):
+        L = int(lens[b])
+        r = orc.varlen_attention(qkv[b, :L, 0], qkv[b, :L, 1], qkv[b, :L, 2], [0, L], [0, L], None, True, alibi_slopes=slopes)
+        assert (out_al[b, :L].float().cpu() - r["out"]).abs().max() < 2e-3
     ref = orc.attention_ref(qkv, mask, 0.0, upcast=True, causal=True).float()
     out_pad, _ = m(qkv.cuda(), key_padding_mask=KPM(), causal=True)
     assert tuple(out_pad.shape) == (B, S, H, D)
