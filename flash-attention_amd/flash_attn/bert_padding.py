@@ -30,71 +30,66 @@ def _scatter(values, indices, first_axis_dim):
     return out
 
 
-class IndexFirstAxis(torch.autograd.Function):
-    """rows = input[indices] for a 2-D input, with a scatter as backward."""
+def _rows(t):
+    """the kernels move rows whose elements are contiguous"""
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+class _MoveRows(torch.autograd.Function):
+    """One differentiable row move in either direction: gather=True picks rows `indices` of a 2-D tensor, gather=False
+    places the rows of a 2-D tensor at `indices` of a zero tensor with n_rows rows.  Each is the other's backward."""
 
     @staticmethod
-    def forward(ctx, input, indices):
-        assert input.ndim == 2
+    def forward(ctx, src, indices, n_rows, gather):
+        assert src.ndim == 2 and indices.ndim == 1
         ctx.save_for_backward(indices)
-        ctx.first_axis_dim = input.shape[0]
-        return _gather(input if input.stride(-1) == 1 else input.contiguous(), indices)
+        ctx.gather = gather
+        ctx.n_src = src.shape[0]
+        return _gather(_rows(src), indices) if gather else _scatter(_rows(src), indices, n_rows)
 
     @staticmethod
-    def backward(ctx, grad_output):
+    def backward(ctx, grad):
         (indices,) = ctx.saved_tensors
-        return _scatter(grad_output if grad_output.stride(-1) == 1 else grad_output.contiguous(), indices,
-                        ctx.first_axis_dim), None
+        g = _scatter(_rows(grad), indices, ctx.n_src) if ctx.gather else _gather(_rows(grad), indices)
+        return g, None, None, None
 
 
-index_first_axis = IndexFirstAxis.apply
+def index_first_axis(input, indices):
+    """input[indices] for a 2-D input (what the reference's IndexFirstAxis.apply computes, :9-33)."""
+    return _MoveRows.apply(input, indices, indices.shape[0], True)
 
 
-class IndexPutFirstAxis(torch.autograd.Function):
-    """output = zeros(first_axis_dim, dim); output[indices] = values, with a gather as backward."""
-
-    @staticmethod
-    def forward(ctx, values, indices, first_axis_dim):
-        assert indices.ndim == 1
-        assert values.ndim == 2
-        ctx.save_for_backward(indices)
-        return _scatter(values if values.stride(-1) == 1 else values.contiguous(), indices, first_axis_dim)
-
-    @staticmethod
-    def backward(ctx, grad_output):
-        (indices,) = ctx.saved_tensors
-        return _gather(grad_output if grad_output.stride(-1) == 1 else grad_output.contiguous(), indices), None, None
+def index_put_first_axis(values, indices, first_axis_dim):
+    """zeros(first_axis_dim, dim) with values written at rows `indices` (the reference's IndexPutFirstAxis.apply, :36-57)."""
+    return _MoveRows.apply(values, indices, first_axis_dim, False)
 
 
-index_put_first_axis = IndexPutFirstAxis.apply
+class IndexFirstAxis:
+    """kept for callers that spell it IndexFirstAxis.apply(input, indices)"""
+    apply = staticmethod(index_first_axis)
+
+
+class IndexPutFirstAxis:
+    """kept for callers that spell it IndexPutFirstAxis.apply(values, indices, first_axis_dim)"""
+    apply = staticmethod(index_put_first_axis)
 
 
 def unpad_input(hidden_states, attention_mask):
-    """
-    Arguments:
-        hidden_states: (batch, seqlen, dim)
-        attention_mask: (batch, seqlen), bool / int, nonzero = valid token.
-    Return:
-        hidden_states: (total_nnz, dim), the valid tokens in batch-major order.
-        indices: (total_nnz,), positions of those tokens in the flattened (batch * seqlen) axis.
-        cu_seqlens: (batch + 1,) int32 cumulative sequence lengths.
-        max_seqlen_in_batch: int
-    """
-    seqlens = attention_mask.sum(dim=-1, dtype=torch.int32)
-    indices = torch.nonzero(attention_mask.flatten(), as_tuple=False).flatten()
-    max_seqlen_in_batch = int(seqlens.max().item())
-    cu_seqlens = F.pad(torch.cumsum(seqlens, dim=0, dtype=torch.int32), (1, 0))
-    flat = hidden_states.reshape(hidden_states.shape[0] * hidden_states.shape[1], -1)
-    return index_first_axis(flat, indices), indices, cu_seqlens, max_seqlen_in_batch
+    """Drop the padding: hidden_states (batch, seqlen, dim) and a (batch, seqlen) mask whose nonzero entries mark real
+    tokens give
+        the real tokens as (total, dim) rows, batch-major,
+        their positions in the flattened batch * seqlen axis (int64, what pad_input takes back),
+        cu_seqlens (batch + 1,) int32, the running sum of the sequence lengths starting at 0,
+        the longest sequence length as a Python int."""
+    lengths = attention_mask.sum(dim=-1, dtype=torch.int32)
+    positions = torch.nonzero(attention_mask.flatten(), as_tuple=False).flatten()
+    cu_seqlens = F.pad(torch.cumsum(lengths, dim=0, dtype=torch.int32), (1, 0))
+    tokens = hidden_states.reshape(hidden_states.shape[0] * hidden_states.shape[1], -1)
+    return index_first_axis(tokens, positions), positions, cu_seqlens, int(lengths.max().item())
 
 
 def pad_input(hidden_states, indices, batch, seqlen):
-    """
-    Arguments:
-        hidden_states: (total_nnz, dim)
-        indices: (total_nnz,)
-    Return:
-        hidden_states: (batch, seqlen, dim), zero where no token was scattered.
-    """
-    output = index_put_first_axis(hidden_states, indices, batch * seqlen)
-    return output.reshape(batch, seqlen, hidden_states.shape[-1])
+    """Inverse of unpad_input: rows (total, dim) go back to their positions `indices` of a (batch, seqlen, dim) tensor
+    that is zero everywhere else."""
+    padded = index_put_first_axis(hidden_states, indices, batch * seqlen)
+    return padded.reshape(batch, seqlen, hidden_states.shape[-1])
