@@ -61,13 +61,3 @@ def test_d64_kernels_keep_their_waves_per_simd():
         assert _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", flags)["Occupancy"] >= 3, flags
         k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", flags)
         assert k["Occupancy"] >= 3 and k["VGPRs Spill"] <= 4, (flags, k)
-
-
-@pytest.mark.timeout(600)
-@pytest.mark.parametrize("src", ["issue_model.hip", "overlap_model.hip"])
-def test_microbenchmarks_build(src, tmp_path):
-    """The micro-benchmarks the design is argued from (csrc/tune) still build with the kernels' flags."""
-    flags = [f for f in fa_build.FLAGS if f != "-fPIC"]
-    cmd = [fa_build.HIPCC] + flags + [os.path.join(fa_build.CSRC, "tune", src), "-o", str(tmp_path / "bench")]
-    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    assert r.returncode == 0, r.stdout[-2000:]
