@@ -6,9 +6,16 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/flash_attn_gfx950.h"
 #include "fa_params.h"
+
+// ---- fa_fwd_block_noalloc: the block activity maps live in this file-scope device array instead of caller scratch.
+// Every GPU the library runs on holds its own copy at its own address until the process ends; `scratch` itself is only
+// a host-side handle, so the device address is looked up once per device (with that device current) and used from then on.
+constexpr size_t kNoAllocScratchBytes = FA_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
 
 namespace {
 
@@ -313,9 +320,49 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
   return FA_OK;
 }
 
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+int noalloc_scratch(void** out) {
+  int dev = -1;
+  FA_LAUNCH(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return fail(FA_ERR_UNSUPPORTED, "device ordinal %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    FA_LAUNCH(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return fail(FA_ERR_LAUNCH, "hipGetSymbolAddress returned a null address");
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return FA_OK;
+}
+
 }  // namespace
 
 extern "C" {
+
+int fa_fwd_block_noalloc(const fa_fwd_args* args) {
+  if (!args) return fail(FA_ERR_INVALID_ARGUMENT, "args is NULL");
+  if (args->struct_bytes != sizeof(fa_fwd_args))
+    return fail(FA_ERR_INVALID_ARGUMENT, "struct_bytes is %u, this library expects %zu (ABI mismatch)", args->struct_bytes,
+                sizeof(fa_fwd_args));
+  if (!args->blockmask) return fail(FA_ERR_INVALID_ARGUMENT, "fa_fwd_block_noalloc needs a blockmask");
+  if (args->max_seqlen_q <= 0 || args->max_seqlen_k <= 0) return fail(FA_ERR_INVALID_ARGUMENT, "max_seqlen must be positive");
+  const size_t need = sparse_layout(round_seqlens(args->head_dim, args->max_seqlen_q, args->max_seqlen_k, true)).bytes;
+  if (need > kNoAllocScratchBytes)
+    return fail(FA_ERR_WORKSPACE,
+                "fa_fwd_block_noalloc: this block layout needs %zu bytes of activity maps, the built-in scratch holds %zu "
+                "(use fa_fwd_block with caller scratch)", need, kNoAllocScratchBytes);
+  void* ptr = nullptr;
+  const int rc = noalloc_scratch(&ptr);
+  if (rc) return rc;
+  fa_fwd_args a = *args;
+  a.workspace = ptr;  // the device address, never the symbol
+  a.workspace_bytes = kNoAllocScratchBytes;
+  return fwd_impl(&a, true);
+}
 
 int fa_fwd(const fa_fwd_args* args) { return fwd_impl(args, false); }
 int fa_fwd_block(const fa_fwd_args* args) { return fwd_impl(args, true); }

@@ -93,7 +93,7 @@ class RotaryArgs(ctypes.Structure):
 
 
 EXPORTED_SYMBOLS = (
-    "fa_fwd", "fa_bwd", "fa_fwd_block", "fa_bwd_block", "fa_fwd_workspace_bytes", "fa_bwd_workspace_bytes",
+    "fa_fwd", "fa_bwd", "fa_fwd_block", "fa_bwd_block", "fa_fwd_block_noalloc", "fa_fwd_workspace_bytes", "fa_bwd_workspace_bytes",
     "fa_round_seqlens", "fa_philox_offset_increment", "fa_last_error", "fa_abi_version",
     "fa_gather_rows", "fa_scatter_rows", "fa_scatter_rows_workspace_bytes", "fa_rotary",
 )
@@ -115,7 +115,7 @@ def load_library():
                 "%s is not built (expected at %s); run `python flash-attention_amd/build.py`. "
                 "There is no non-HIP fallback." % (LIB_NAME, LIB_PATH))
         lib = ctypes.CDLL(LIB_PATH)
-        for name in ("fa_fwd", "fa_fwd_block"):
+        for name in ("fa_fwd", "fa_fwd_block", "fa_fwd_block_noalloc"):
             fn = getattr(lib, name)
             fn.argtypes = [ctypes.POINTER(FwdArgs)]
             fn.restype = ctypes.c_int

@@ -134,6 +134,17 @@ int fa_fwd_block(const fa_fwd_args* args);
 /* replaces flash_attn_cuda.bwd_block -> mha_bwd_block, csrc/flash_attn/fmha_api.cpp:575-718 */
 int fa_bwd_block(const fa_bwd_args* args);
 
+/* No counterpart in the reference.  fa_fwd_block for callers that cannot allocate device memory or carry scratch
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): the block activity maps that
+ * fa_fwd_block keeps in `workspace` live in a device array inside the library instead (FA_NOALLOC_SCRATCH_BYTES, held by
+ * every GPU the library runs on until the process ends).  args->workspace / workspace_bytes are ignored; inputs and
+ * outputs are the caller's as usual.  Layouts whose maps need more (fa_fwd_workspace_bytes() > FA_NOALLOC_SCRATCH_BYTES;
+ * the limit is reached between 16384 and 32768 tokens) are refused with FA_ERR_WORKSPACE.  The call allocates nothing
+ * and the maps are rebuilt by every call, but all calls on one GPU share the one array: calls that overlap on a GPU
+ * (different streams or host threads) race; serialise them.  Results are those of fa_fwd_block. */
+#define FA_NOALLOC_SCRATCH_BYTES (64u * 1024u)
+int fa_fwd_block_noalloc(const fa_fwd_args* args);
+
 /* Scratch the caller provides.  The dense forward and backward need none to be correct
  * (there is no o_tmp / dq_tmp, fmha_api.cpp:247,403-404).  The block-sparse paths need room for their block activity
  * maps (an error without it).  For a dense, non-causal forward with few query rows and many keys (max_seqlen_q <= 128,
