@@ -34,9 +34,10 @@ namespace fa {
 // ---------------------------------------------------------------------------------------------------------------
 // dK, dV
 // ---------------------------------------------------------------------------------------------------------------
-template <typename T, int D>
+template <typename T, int D, bool kDropout = false>
 struct BwdCfg {
-  static constexpr int BM = kBwdBM;  // query rows per step
+  static constexpr bool kVLds = D == 128 && !kDropout;  // see below
+  static constexpr int BM = kVLds ? 32 : 64;  // query rows per step
   static constexpr int BN = kBwdBN;  // keys per workgroup
   static constexpr int DV = D < 32 ? 32 : D;
   // Q tile followed by dO tile, both read as row fragments and transposed, double buffered (see fa_stage.h),
@@ -46,22 +47,30 @@ struct BwdCfg {
   static constexpr int kSlack = D < 32 ? 64 : 0;  // the 32-wide transposed reads run past a 16-wide row
   static constexpr int kOffStat = 2 * kBufBytes + kSlack;
   static constexpr int kStatBytes = 2 * BM * 4;   // lse[BM], -Dk[BM]
-  static constexpr int kTileBytes = kOffStat + 2 * kStatBytes;
+  // At d = 128 the K and V fragments plus the two accumulators of a wave would be 192 registers: more than two waves per
+  // SIMD allow next to the scores.  There (without dropout, whose Philox state needs the registers anyway and which
+  // stays at one wave per SIMD) the workgroup's V tile sits in LDS for the whole kernel instead, rows padded by
+  // 8 elements (16 lanes reading one 16-byte chunk of 16 consecutive rows then hit 16 distinct bank groups, and a
+  // fragment's address is one register plus a constant), and the query tile is one 32-row slab, so that two workgroups
+  // fit a compute unit's LDS.
+  static constexpr int VS = D + 8;  // V tile row stride in elements
+  static constexpr int kOffV = kOffStat + 2 * kStatBytes;
+  static constexpr int kTileBytes = kOffV + (kVLds ? BN * VS * 2 : 0);
   static constexpr int kEpiBytes = BN * (D + 8) * 2;
   static constexpr int kLdsBytes = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
   static constexpr int CH = D / 8;
-  static constexpr int kMinBlocks = D <= 64 ? 2 : 1;
+  static constexpr int kMinBlocks = (D == 128 && kDropout) ? 1 : 2;
 };
 
 template <typename T, int D, bool kCausal, bool kDropout, bool kSparse, bool kAlibi = false>
-__global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
-  using Cfg = BwdCfg<T, D>;
+__global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D, kDropout>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
+  using Cfg = BwdCfg<T, D, kDropout>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
   using vec4 = typename E::vec4;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, DV = Cfg::DV, CH = Cfg::CH, kBufBytes = Cfg::kBufBytes;
-  constexpr bool kPipe = D == 128;  // software-pipelined LDS fetches (see the main loop)
-  static_assert(BM == 64, "the main loop handles two 32-row slabs per tile");
+  static_assert(BM == 64 || BM == 32, "a tile is one or two 32-row slabs");
+  constexpr int RBT = BM / 16;  // 16-row blocks per tile (sparse activity bits per tile)
 
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
 
@@ -81,21 +90,39 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
   const int c = lane & 31, hf = lane >> 5;
   const int key = n0 + wave * 32 + c;  // this lane's key (sequence-local)
 
-  // ---- K and V fragments of this wave's 32 keys (B operands), registers for the whole kernel.
+  // ---- K and V fragments of this wave's 32 keys (B operands), registers for the whole kernel (V: LDS with kVLds).
   // Keys past the end are zero: their P is finite, their dK / dV rows are never stored.
-  vec8 kreg[D / 16], vreg[D / 16];
+  constexpr bool kVLds = Cfg::kVLds;
+  vec8 kreg[D / 16], vreg[kVLds ? 1 : D / 16];
   {
     const int kr = key < Lk ? key : Lk - 1;
     const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)(k_begin + kr) * p.k_rs + (int64_t)h * p.k_hs + hf * 8;
     const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)(k_begin + kr) * p.v_rs + (int64_t)h * p.v_hs + hf * 8;
 #pragma unroll
     for (int ks = 0; ks < D / 16; ks++) {
-      u32x4 a = ld_global16(kp + ks * 16), bb = ld_global16(vp + ks * 16);
-      if (key >= Lk) { a = u32x4{0, 0, 0, 0}; bb = u32x4{0, 0, 0, 0}; }
+      u32x4 a = ld_global16(kp + ks * 16);
+      if (key >= Lk) a = u32x4{0, 0, 0, 0};
       kreg[ks] = bitcast<vec8>(a);
-      vreg[ks] = bitcast<vec8>(bb);
+      if (!kVLds) {
+        u32x4 bb = ld_global16(vp + ks * 16);
+        if (key >= Lk) bb = u32x4{0, 0, 0, 0};
+        vreg[ks] = bitcast<vec8>(bb);
+      }
     }
   }
+  T* const Vl = reinterpret_cast<T*>(lds_raw + Cfg::kOffV);
+  if (kVLds) {  // the first barrier of the main loop orders these writes before the first read
+    const T* vt = reinterpret_cast<const T*>(p.v) + (int64_t)k_begin * p.v_rs + (int64_t)h * p.v_hs;
+#pragma unroll
+    for (int i = 0; i < BN * CH / 256; i++) {
+      const int id = tid + i * 256;
+      const int row = id / CH, ch = id % CH;
+      u32x4 x = {0, 0, 0, 0};
+      if (n0 + row < Lk) x = ld_global16(vt + (int64_t)(n0 + row) * p.v_rs + ch * 8);
+      *reinterpret_cast<u32x4*>(Vl + row * Cfg::VS + ch * 8) = x;
+    }
+  }
+  const T* const Vfrag = Vl + (wave * 32 + c) * Cfg::VS + hf * 8;  // this lane's V fragments: + 16 * ks elements
   int mt_begin = 0;
   if (kCausal) mt_begin = n0 / BM;  // query rows above the tile's first key see none of its keys
   const int mt_end = (Lq + BM - 1) / BM;
@@ -135,21 +162,22 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
   // pair; a query tile is visited iff one of its four row blocks attends the key block.
   uint64_t col_bits = 0;
   int bits_word = -1;
+  constexpr int TPW = 64 / RBT;  // query tiles per 64-bit activity word
   auto tile_rows_on = [&](int mt) -> uint32_t {  // bit j: 16-row block j of query tile mt attends this key block
-    if ((mt >> 4) != bits_word) {
-      bits_word = __builtin_amdgcn_readfirstlane(mt >> 4);
+    if ((mt / TPW) != bits_word) {
+      bits_word = __builtin_amdgcn_readfirstlane(mt / TPW);
       col_bits = uniform64(p.sp.cbits[(int64_t)(n0 >> 8) * p.sp.nrw + bits_word]);
     }
-    return (uint32_t)(col_bits >> (4 * (mt & 15))) & 0xfu;
+    return (uint32_t)(col_bits >> (RBT * (mt % TPW))) & ((1u << RBT) - 1);
   };
   // First query tile >= mt with a set bit (mt_end if none), found with a count-trailing-zeros on the loaded word
   auto next_active = [&](int mt) -> int {
     if (!kSparse) return mt;
     while (mt < mt_end) {
       tile_rows_on(mt);  // loads the word of mt if needed
-      const uint64_t rest = col_bits >> (4 * (mt & 15));  // bits 0..3: this tile's row blocks
-      if (rest & 0xf) break;
-      mt = rest ? mt + ((int)__builtin_ctzll(rest) >> 2) : (mt | 15) + 1;
+      const uint64_t rest = col_bits >> (RBT * (mt % TPW));  // low RBT bits: this tile's row blocks
+      if (rest & ((1u << RBT) - 1)) break;
+      mt = rest ? mt + (int)__builtin_ctzll(rest) / RBT : (mt | (TPW - 1)) + 1;
     }
     return mt < mt_end ? mt : mt_end;
   };
@@ -184,7 +212,7 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
     float* const lse_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffStat + buf * Cfg::kStatBytes);
     float* const dk_l = lse_l + BM;
     if (tid < 2 * BM) lse_l[tid] = stat_value();
-    uint32_t rows_on = 0xfu;  // bit j: 16-row block j of this tile attends this key block
+    uint32_t rows_on = (1u << RBT) - 1;  // bit j: 16-row block j of this tile attends this key block
     if (kSparse) rows_on = tile_rows_on(mt);
     __syncthreads();  // tile `mt` is complete, and nobody still reads the other buffer
     const int mt_next = next_active(mt + 1);
@@ -195,10 +223,7 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
 
     const bool diag = kCausal && (m0 < n0 + wave * 32 + 32);  // some (q, key) of this wave's slab has key > q
 
-    // LDS fragment fetches.  With kPipe (d = 128: one wave per SIMD, nobody else hides LDS latency) they are issued a
-    // stage ahead of their MFMAs - the row fragments of a 32-row slab before the previous slab's last MFMAs, the
-    // transposed fragments of a 16-row step under the exponentials / the previous step's MFMAs - and scheduling
-    // barriers keep the compiler from sinking them back.  Otherwise they sit next to their use and other waves hide them.
+    // LDS fragment fetches sit next to their use; the other waves of the SIMD hide their latency.
     auto load_rows = [&](int qb, vec8* aq, vec8* ad) {
 #pragma unroll
       for (int ks = 0; ks < D / 16; ks++) aq[ks] = *reinterpret_cast<const vec8*>(Ql + qb * 32 * D + foff[ks]);
@@ -216,21 +241,16 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
         aqs[db] = u32x4{lo[0], lo[1], hi[0], hi[1]};
       }
     };
-    vec8 aq[2][D / 16], ad[2][D / 16];
-    if (kPipe) load_rows(0, aq[0], ad[0]);
 #pragma unroll
     for (int qb = 0; qb < BM / 32; qb++) {
       // dropout: the two slabs' Philox streams are not to be interleaved by the scheduler (it would, for the sake of
       // instruction-level parallelism, and need 70 more registers: one wave per SIMD fewer)
-      if (kDropout && !kPipe) __builtin_amdgcn_sched_barrier(0);
+      if (kDropout) __builtin_amdgcn_sched_barrier(0);
       bool rb_on[2] = {true, true};
       if (kSparse) {
         rb_on[0] = (rows_on >> (2 * qb)) & 1;
         rb_on[1] = (rows_on >> (2 * qb + 1)) & 1;
-        if (!(rb_on[0] || rb_on[1])) {  // no row of this slab attends the key block: nothing to add to dK, dV
-          if (kPipe && qb + 1 < BM / 32) load_rows(qb + 1, aq[qb + 1], ad[qb + 1]);
-          continue;
-        }
+        if (!(rb_on[0] || rb_on[1])) continue;  // no row of this slab attends the key block: nothing to add to dK, dV
       }
       // ---- S = Q K^T and dP = dO V^T for 32 query rows x this wave's 32 keys
       // dP starts from -Dk of its query row (fmha_dgrad_kernel_1xN_loop.h:361-371), so the MFMA delivers dP - Dk
@@ -241,17 +261,13 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
 #pragma unroll
         for (int i = 0; i < 4; i++) { s[4 * j + i] = 0.f; dp[4 * j + i] = nd4[i]; }
       }
-      if (kPipe) __builtin_amdgcn_sched_barrier(0);
-      else load_rows(qb, aq[qb], ad[qb]);
+      vec8 aq[D / 16], ad[D / 16];
+      load_rows(qb, aq, ad);
 #pragma unroll
-      for (int ks = 0; ks < D / 16; ks++) s = E::mfma32(aq[qb][ks], kreg[ks], s);
+      for (int ks = 0; ks < D / 16; ks++) s = E::mfma32(aq[ks], kreg[ks], s);
 #pragma unroll
-      for (int ks = 0; ks < D / 16; ks++) dp = E::mfma32(ad[qb][ks], vreg[ks], dp);
-      u32x4 avs[2][DV / 32], aqs[2][DV / 32];
-      if (kPipe) {
-        load_tr(qb, 0, avs[0], aqs[0]);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+      for (int ks = 0; ks < D / 16; ks++)
+        dp = E::mfma32(ad[ks], kVLds ? *reinterpret_cast<const vec8*>(Vfrag + ks * 16) : vreg[ks], dp);
       // ---- P and dS'
       KeepFields keep;
       if (kDropout) keep = keep_fields_col_layout(p.pk, (uint32_t)bh, m0 + qb * 32, key, hf);
@@ -294,17 +310,12 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
         for (int i = 0; i < 8; i++) { pf[i] = s[8 * t + i]; df[i] = dp[8 * t + i]; }
         const vec8 pb = cvt8<T>(pf);
         const vec8 db8 = cvt8<T>(df);
-        if (kPipe) {
-          if (t == 0) load_tr(qb, 1, avs[1], aqs[1]);
-          else if (qb + 1 < BM / 32) load_rows(qb + 1, aq[qb + 1], ad[qb + 1]);
-          __builtin_amdgcn_sched_barrier(0);
-        } else {
-          load_tr(qb, t, avs[t], aqs[t]);
-        }
+        u32x4 avs[DV / 32], aqs[DV / 32];
+        load_tr(qb, t, avs, aqs);
 #pragma unroll
         for (int db = 0; db < DV / 32; db++) {
-          acc_dv[db] = E::mfma32(bitcast<vec8>(avs[t][db]), pb, acc_dv[db]);
-          acc_dk[db] = E::mfma32(bitcast<vec8>(aqs[t][db]), db8, acc_dk[db]);
+          acc_dv[db] = E::mfma32(bitcast<vec8>(avs[db]), pb, acc_dv[db]);
+          acc_dk[db] = E::mfma32(bitcast<vec8>(aqs[db]), db8, acc_dk[db]);
         }
       }
     }

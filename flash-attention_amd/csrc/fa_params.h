@@ -196,6 +196,5 @@ hipError_t launch_zero_rows(void* base, int64_t row_stride, int64_t head_stride,
 // Tile shapes, needed by the front end for grid sizes and workspace layout.
 constexpr int kFwdBM = 128;   // query rows per forward workgroup
 constexpr int kBwdBN = 128;   // keys per dK/dV workgroup
-constexpr int kBwdBM = 64;    // query rows per dK/dV inner step
 
 }  // namespace fa

@@ -61,3 +61,16 @@ def test_d64_kernels_keep_their_waves_per_simd():
         assert _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", flags)["Occupancy"] >= 3, flags
         k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", flags)
         assert k["Occupancy"] >= 3 and k["VGPRs Spill"] <= 4, (flags, k)
+
+
+@pytest.mark.timeout(600)
+def test_d128_backward_keeps_two_waves_per_simd():
+    """d = 128: the dK/dV kernel holds its V tile in LDS so that K, the two accumulators and the scores fit 256 registers
+    (two waves per SIMD, nothing spilled: a spill's scratch load would wait behind the tile prefetch on every step)."""
+    bwd = _resources("fa_bwd_d128.hip")
+    for dt in ("IDF16_", "IDF16b"):
+        for flags in ("Lb0ELb0ELb0ELb0E", "Lb1ELb0ELb0ELb0E", "Lb0ELb0ELb1ELb0E", "Lb1ELb0ELb1ELb0E"):
+            k = _pick(bwd, "fa_bwd_dkdv_kernel%sLi128E" % dt, flags)
+            assert k["Occupancy"] >= 2 and k["VGPRs Spill"] == 0 and k["LDS Size"] <= 80 * 1024, (dt, flags, k)
+            k = _pick(bwd, "fa_bwd_dq_kernel%sLi128E" % dt, flags)
+            assert k["Occupancy"] >= 2 and k["VGPRs Spill"] <= (1 if "Lb1ELb0E" in flags[8:] else 0), ("dq", dt, flags, k)
