@@ -6,6 +6,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <atomic>
 #include <mutex>
 
 #include "../../include/flash_attn_gfx950.h"
@@ -16,6 +17,13 @@
 // a host-side handle, so the device address is looked up once per device (with that device current) and used from then on.
 constexpr size_t kNoAllocScratchBytes = FA_NOALLOC_SCRATCH_BYTES;
 static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+namespace {
+std::atomic<int> g_launch_policy{0};
+}
+namespace fa {
+int launch_policy() { return g_launch_policy.load(std::memory_order_relaxed); }
+}  // namespace fa
 
 namespace {
 
@@ -459,6 +467,12 @@ int fa_rotary(const fa_rotary_args* a) {
   p.n_parts = a->n_parts; p.n_rotated = a->n_rotated; p.n_heads = a->n_heads; p.head_dim = a->head_dim;
   p.seqlen = a->seqlen; p.table_rows = a->table_rows; p.conjugate = a->conjugate;
   FA_LAUNCH(fa::launch_rotary(p, a->dtype, reinterpret_cast<hipStream_t>(a->stream)));
+  return FA_OK;
+}
+
+int fa_set_launch_policy(int policy) {
+  FA_REQUIRE(policy >= 0 && policy <= 2, "launch policy must be 0 (automatic), 1 (full-size tiles) or 2 (half-size tiles)");
+  g_launch_policy.store(policy, std::memory_order_relaxed);
   return FA_OK;
 }
 

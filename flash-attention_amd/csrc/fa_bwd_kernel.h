@@ -364,9 +364,15 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
 // ---------------------------------------------------------------------------------------------------------------
 // dQ
 // ---------------------------------------------------------------------------------------------------------------
-template <typename T, int D, int BN>
+// KS: key split as in the forward kernel (FwdCfg): 1 = four waves with 32 of the workgroup's 128 query rows each;
+// 2 = 64 query rows, the waves w and w + 2 share 32 rows, split every key tile's two 32-key blocks between them and add
+// up their partial dQ in the epilogue.
+template <typename T, int D, int BN, int KS = 1>
 struct DqCfg {
-  static constexpr int BM = kFwdBM;  // query rows per workgroup (same tiling as the forward: shares its sparse map)
+  static constexpr int BM = kFwdBM / KS;  // query rows per workgroup (KS = 1: the forward's tiling, shares its sparse map)
+  static constexpr int RW = 4 / KS;       // 32-row slabs per workgroup
+  static constexpr int KBW = BN / 32 / KS;  // 32-key blocks of a tile per wave
+  static_assert(KS == 1 || (KS == 2 && BN == 64), "key split: two waves per 32 rows, one 32-key block each");
   static constexpr int DV = D < 32 ? 32 : D;
   static constexpr int OS = D + 8;
   // K tile (read as row fragments and transposed) followed by V tile (row fragments), double buffered (fa_stage.h)
@@ -375,16 +381,19 @@ struct DqCfg {
   static constexpr int kSlack = D < 32 ? 64 : 0;  // the 32-wide transposed reads run past a 16-wide K row
   static constexpr int kTileBytes = 2 * kBufBytes + kSlack;
   static constexpr int kEpiBytes = BM * OS * 2;
-  static constexpr int kLdsBytes = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
+  static constexpr int kMergeBytes = KS > 1 ? RW * (DV / 32 * 16) * 64 * 4 : 0;  // partial dQ of RW waves
+  static constexpr int kLdsBytes0 = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
+  static constexpr int kLdsBytes = kLdsBytes0 > kMergeBytes ? kLdsBytes0 : kMergeBytes;
   static constexpr int CH = D / 8;
 };
 
-template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, bool kAlibi = false>
+template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, bool kAlibi = false, int KS = 1>
 __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq_kernel(const BwdParams p) {
-  using Cfg = DqCfg<T, D, BN>;
+  using Cfg = DqCfg<T, D, BN, KS>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
-  constexpr int BM = Cfg::BM, DV = Cfg::DV, CH = Cfg::CH, kBufBytes = Cfg::kBufBytes;
+  constexpr int BM = Cfg::BM, DV = Cfg::DV, CH = Cfg::CH, kBufBytes = Cfg::kBufBytes, KBW = Cfg::KBW;
+  static_assert(KS == 1 || !kSparse, "the block-sparse maps are built for 128-row query tiles");
 
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
 
@@ -405,7 +414,9 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 31, hf = lane >> 5;
-  const int mw = m0 + wave * 32;
+  const int rs = KS > 1 ? wave % Cfg::RW : wave;  // this wave's 32-row slab of the tile
+  const int kh = KS > 1 ? wave / Cfg::RW : 0;     // ... and its share of every key tile's 32-key blocks
+  const int mw = m0 + rs * 32;
   const int qrow = mw + c;
 
   // ---- Q and dO fragments (B operands), lse and Dk of this lane's query row.  Dk = keep * rowsum(dO o O) is computed
@@ -434,7 +445,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
       const float x = p.lse[((int64_t)b * p.H + h) * p.lse_stride + qrow];
       lse2 = (x == -INFINITY) ? INFINITY : x * kLog2e;
       dkv = dsum;
-      if (hf == 0 && split == 0) p.dsoftmax[((int64_t)b * p.H + h) * p.sq_r + qrow] = dsum;
+      if (hf == 0 && split == 0 && kh == 0) p.dsoftmax[((int64_t)b * p.H + h) * p.sq_r + qrow] = dsum;
     }
   }
   // For d <= 64 the dP^T accumulator starts from -Dk of this lane's query row (16 registers that save 16 subtractions
@@ -523,7 +534,9 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
     buf ^= 1;
 
     bool wave_work = mw < Lq;  // a wave whose 32 rows all lie past the sequence's end only helps with the staging
-    if (kCausal && n0 > mw + 31) wave_work = false;
+    const int kb0 = kh * KBW;  // this wave's 32-key blocks of the tile: kb0, kb0 + 1, ... (all of them without a key split)
+    if (kCausal && n0 + kb0 * 32 > mw + 31) wave_work = false;  // every key of the wave's share is above its diagonal
+    if (KS > 1 && n0 + kb0 * 32 >= Lk) wave_work = false;       // ... or past the last key
     bool row_on = true;
     if (kSparse) {
       row_on = row_on_cur;
@@ -534,7 +547,8 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
       // tiles that straddle the key length, the diagonal or an inactive row block get their dead scores set to -inf
       const bool need_mask = (n0 + BN > Lk) || (kCausal && (n0 + BN - 1 > mw)) || (kSparse && !row_on);
 #pragma unroll
-      for (int kb = 0; kb < BN / 32; kb++) {
+      for (int kbi = 0; kbi < KBW; kbi++) {
+        const int kb = kb0 + kbi;
         f32x16 s, dp = negd;
 #pragma unroll
         for (int r = 0; r < 16; r++) s[r] = 0.f;
@@ -593,6 +607,27 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
     it = it_next;
   }
 
+  // ---- key split: the waves kh > 0 hand their partial dQ to the wave kh == 0 of their rows, in the accumulator's own
+  // register order (word (rs * 16 DV/32 + j) * 64 + lane: consecutive lanes, no bank conflicts)
+  if (KS > 1) {
+    __syncthreads();  // every wave has left the tiles
+    float* const X = reinterpret_cast<float*>(lds_raw) + rs * (DV / 32 * 16) * 64 + lane;
+    if (kh != 0) {
+#pragma unroll
+      for (int db = 0; db < DV / 32; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) X[(db * 16 + r) * 64] = acc[db][r];
+    }
+    __syncthreads();
+    if (kh == 0) {
+#pragma unroll
+      for (int db = 0; db < DV / 32; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[db][r] += X[(db * 16 + r) * 64];
+    }
+    __syncthreads();  // the staging area of the stores below overlaps the exchange area
+    if (kh != 0) return;
+  }
   // ---- epilogue: dQ = dQ^T acc * scale / keep, transposed through LDS, coalesced stores
   const float f = p.scale * p.rp_keep;
   if (p.n_splits > 1) {  // partial sum of this key split, fp32, added up by dq_combine_kernel
@@ -613,9 +648,9 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
     }
     return;
   }
-  __syncthreads();
+  if (KS == 1) __syncthreads();
   constexpr int OS = Cfg::OS;
-  T* Os = reinterpret_cast<T*>(lds_raw) + wave * 32 * OS;
+  T* Os = reinterpret_cast<T*>(lds_raw) + rs * 32 * OS;
 #pragma unroll
   for (int db = 0; db < DV / 32; db++)
 #pragma unroll

@@ -20,10 +20,17 @@
 
 namespace fa {
 
-template <typename T, int D, int BN>
+// KS (key split) = 1: the workgroup's four waves own 32 of its 128 query rows each and every wave sees all keys of a tile.
+// KS = 2 (short sequences, where 128-row tiles are too few workgroups to fill the chip and one workgroup's walk over the
+// keys is the launch's critical path): 64 query rows per workgroup; waves w and w + 2 share 32 rows and split the keys
+// of every tile between them, each with its own running maximum, sum and output accumulator, merged in the epilogue.
+template <typename T, int D, int BN, int KS = 1>
 struct FwdCfg {
-  static constexpr int BM = kFwdBM;
-  static constexpr int NW = 4;                 // waves per workgroup, 32 query rows each
+  static constexpr int BM = kFwdBM / KS;
+  static constexpr int NW = 4;                 // waves per workgroup
+  static constexpr int RW = NW / KS;           // 32-row slabs per workgroup
+  static constexpr int KBW = BN / 32 / KS;     // 32-key blocks of a tile per wave
+  static_assert(KS == 1 || (KS == 2 && BN == 64), "key split: two waves per 32 rows, one 32-key block each");
   static constexpr int DV = D < 32 ? 32 : D;   // rows of the V^T MFMA operand (for D = 16 the upper 16 are don't-care)
   static constexpr int OS = D + 8;             // epilogue staging row stride
   // K tile (read as row fragments) followed by V tile (read transposed), double buffered; see fa_stage.h
@@ -32,18 +39,21 @@ struct FwdCfg {
   static constexpr int kSlack = D < 32 ? 64 : 0;                // the 32-wide transposed reads run past a 16-wide V row
   static constexpr int kTileBytes = 2 * kBufBytes + kSlack;
   static constexpr int kEpiBytes = BM * OS * 2;
-  static constexpr int kLdsBytes = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
+  static constexpr int kMergeBytes = KS > 1 ? RW * (DV / 32 * 16 + 2) * 64 * 4 : 0;  // partial (O, max, sum) of RW waves
+  static constexpr int kLdsBytes0 = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
+  static constexpr int kLdsBytes = kLdsBytes0 > kMergeBytes ? kLdsBytes0 : kMergeBytes;
   static constexpr int CH = D / 8;
 };
 
 // kAlibi: the score of (query i, key j) gets -slope[head] * |i - j| added after scaling.  The scores are then moved to the
 // softmax's own units (base-2 exponent) before the row maximum is taken, and the running maximum is kept in those units.
-template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, bool kAlibi = false>
+template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, bool kAlibi = false, int KS = 1>
 __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2) fa_fwd_kernel(const FwdParams p) {
-  using Cfg = FwdCfg<T, D, BN>;
+  using Cfg = FwdCfg<T, D, BN, KS>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
-  constexpr int BM = Cfg::BM, DV = Cfg::DV, CH = Cfg::CH, kBufBytes = Cfg::kBufBytes;
+  constexpr int BM = Cfg::BM, DV = Cfg::DV, CH = Cfg::CH, kBufBytes = Cfg::kBufBytes, KBW = Cfg::KBW;
+  static_assert(KS == 1 || !kSparse, "the block-sparse maps are built for 128-row query tiles");
 
   __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
 
@@ -66,7 +76,9 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int c = lane & 31, hf = lane >> 5;
-  const int mw = m0 + wave * 32;  // first query row of this wave
+  const int rs = KS > 1 ? wave % Cfg::RW : wave;  // this wave's 32-row slab of the tile
+  const int kh = KS > 1 ? wave / Cfg::RW : 0;     // ... and its share of every key tile's 32-key blocks
+  const int mw = m0 + rs * 32;    // first query row of this wave
   const int qrow = mw + c;        // this lane's query row (sequence-local)
 
   // ---- Q fragment (B operand of S^T = K Q^T), held in registers for the whole kernel
@@ -75,11 +87,9 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
     const int qr = qrow < Lq ? qrow : Lq - 1;
     const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)(q_begin + qr) * p.q_rs + (int64_t)h * p.q_hs + hf * 8;
 #pragma unroll
-    for (int ks = 0; ks < D / 16; ks++) {
-      u32x4 raw = ld_global16(qp + ks * 16);
-      if (qrow >= Lq) raw = u32x4{0, 0, 0, 0};
-      qreg[ks] = bitcast<vec8>(raw);
-    }
+    for (int ks = 0; ks < D / 16; ks++) qreg[ks] = bitcast<vec8>(ld_global16(qp + ks * 16));
+    // rows past the end work on a copy of the last row and are never stored (no select on the loaded data here: it
+    // would make the wave wait for the load before it has issued its first tile)
   }
 
   int n_end = Lk;
@@ -160,7 +170,8 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
     buf ^= 1;
 
     bool wave_work = mw < Lq;  // a wave whose 32 rows all lie past the sequence's end only helps with the staging
-    if (kCausal && n0 > mw + 31) wave_work = false;  // every key of this tile is above the wave's diagonal
+    if (kCausal && n0 + kh * 32 * KBW > mw + 31) wave_work = false;  // every key of the wave's share is above its diagonal
+    if (KS > 1 && n0 + kh * 32 * KBW >= Lk) wave_work = false;       // ... or past the last key
     bool row_on = true;
     if (kSparse) {
       row_on = row_on_cur;
@@ -170,14 +181,16 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
 
     if (wave_work) {
       // ---- S^T = K Q^T
-      f32x16 s[BN / 32];
+      // this wave's 32-key blocks of the tile: kb0, kb0 + 1, ... (all of them without a key split)
+      const int kb0 = kh * KBW;
+      f32x16 s[KBW];
 #pragma unroll
-      for (int kb = 0; kb < BN / 32; kb++) {
+      for (int kb = 0; kb < KBW; kb++) {
 #pragma unroll
         for (int r = 0; r < 16; r++) s[kb][r] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < D / 16; ks++) {
-          vec8 a = *reinterpret_cast<const vec8*>(Ks + kb * 32 * D + koff[ks]);
+          vec8 a = *reinterpret_cast<const vec8*>(Ks + (kb0 + kb) * 32 * D + koff[ks]);
           s[kb] = E::mfma32(a, qreg[ks], s[kb]);
         }
       }
@@ -185,10 +198,10 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
       const bool need_mask = (n0 + BN > Lk) || (kCausal && (n0 + BN - 1 > mw)) || (kSparse && !row_on);
       if (need_mask) {
 #pragma unroll
-        for (int kb = 0; kb < BN / 32; kb++)
+        for (int kb = 0; kb < KBW; kb++)
 #pragma unroll
           for (int r = 0; r < 16; r++) {
-            const int key = n0 + kb * 32 + (r >> 2) * 8 + hf * 4 + (r & 3);
+            const int key = n0 + (kb0 + kb) * 32 + (r >> 2) * 8 + hf * 4 + (r & 3);
             bool dead = key >= Lk;
             if (kCausal) dead = dead || key > qrow;
             if (kSparse) dead = dead || !row_on;
@@ -197,8 +210,8 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
       }
       if (kAlibi) {  // s <- s * scale * log2(e) - slope2 * |key - query|; dead scores stay -inf
 #pragma unroll
-        for (int kb = 0; kb < BN / 32; kb++) {
-          const float dbase = (float)(n0 + kb * 32 + hf * 4 - qrow);  // key - query of register 0
+        for (int kb = 0; kb < KBW; kb++) {
+          const float dbase = (float)(n0 + (kb0 + kb) * 32 + hf * 4 - qrow);  // key - query of register 0
 #pragma unroll
           for (int r = 0; r < 16; r++) {
             const float cr = (float)((r >> 2) * 8 + (r & 3));
@@ -211,7 +224,7 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
       // ---- online softmax (fmha_fprop_kernel_1xN.h:408-454,560-611 restated for a register-resident row)
       float mt = s[0][0];
 #pragma unroll
-      for (int kb = 0; kb < BN / 32; kb++)
+      for (int kb = 0; kb < KBW; kb++)
 #pragma unroll
         for (int r = 0; r < 16; r++) mt = fmaxf(mt, s[kb][r]);
       mt = half_max(mt);
@@ -229,21 +242,21 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
         for (int i = 0; i < DV / 32; i++) o_acc[i] = o_acc[i] * alpha;
       }
       const float mc = ((m_i == -INFINITY) ? 0.f : m_i) * cse;
-      float rs = 0.f;
+      float rsum = 0.f;
 #pragma unroll
-      for (int kb = 0; kb < BN / 32; kb++)
+      for (int kb = 0; kb < KBW; kb++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
           const float pe = fast_exp2(kAlibi ? s[kb][r] - mc : __builtin_fmaf(s[kb][r], cs, -mc));
           s[kb][r] = pe;
-          if (kDropout) rs += pe;
+          if (kDropout) rsum += pe;
         }
-      if (kDropout) l_i += rs;  // the sum uses P before dropout (fmha_fprop_kernel_1xN.h:454 vs :471)
+      if (kDropout) l_i += rsum;  // the sum uses P before dropout (fmha_fprop_kernel_1xN.h:454 vs :471)
 
       if (kDropout) {
 #pragma unroll
-        for (int kb = 0; kb < BN / 32; kb++) {
-          const KeepFields keep = keep_fields_row_layout(p.pk, (uint32_t)bh, qrow, n0 + kb * 32, hf);
+        for (int kb = 0; kb < KBW; kb++) {
+          const KeepFields keep = keep_fields_row_layout(p.pk, (uint32_t)bh, qrow, n0 + (kb0 + kb) * 32, hf);
 #pragma unroll
           for (int r = 0; r < 16; r++)
             if (!keep.keep_row(r, p.keep_thr)) s[kb][r] = 0.f;
@@ -252,7 +265,7 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
 
       // ---- O^T += V^T P^T
 #pragma unroll
-      for (int kb = 0; kb < BN / 32; kb++) {
+      for (int kb = 0; kb < KBW; kb++) {
 #pragma unroll
         for (int t = 0; t < 2; t++) {
           f32x8 pf;
@@ -262,7 +275,7 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
           if (!kDropout) l_i = sum8_acc(pb, l_i);
 #pragma unroll
           for (int db = 0; db < DV / 32; db++) {
-            const T* vp = Vs + (kb * 32 + 16 * t) * D + voff[db];
+            const T* vp = Vs + ((kb0 + kb) * 32 + 16 * t) * D + voff[db];
             u32x2 lo = lds_read_tr16(vp);
             u32x2 hi = lds_read_tr16(vp + 8 * D);
             u32x4 av = {lo[0], lo[1], hi[0], hi[1]};
@@ -274,6 +287,36 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
     it = it_next;
   }
 
+  // ---- key split: the waves kh > 0 hand their partial (O, maximum, sum) to the wave kh == 0 of their rows, in the
+  // accumulator's own register order (word (rs * (16 DV/32 + 2) + j) * 64 + lane: consecutive lanes, no bank conflicts)
+  if (KS > 1) {
+    __syncthreads();  // every wave has left the tiles
+    constexpr int NJ = DV / 32 * 16 + 2;
+    float* const X = reinterpret_cast<float*>(lds_raw) + rs * NJ * 64 + lane;
+    if (kh != 0) {
+#pragma unroll
+      for (int db = 0; db < DV / 32; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) X[(db * 16 + r) * 64] = o_acc[db][r];
+      X[(NJ - 2) * 64] = m_i;
+      X[(NJ - 1) * 64] = l_i;
+    }
+    __syncthreads();
+    if (kh == 0) {
+      const float m_b = X[(NJ - 2) * 64], l_b = X[(NJ - 1) * 64];
+      const float m_new = fmaxf(m_i, m_b);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float wa = fast_exp2(m_i * cse - m_use * cse), wb = fast_exp2(m_b * cse - m_use * cse);  // exp2(-inf) = 0
+      m_i = m_new;
+      l_i = l_i * wa + l_b * wb;
+#pragma unroll
+      for (int db = 0; db < DV / 32; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o_acc[db][r] = o_acc[db][r] * wa + X[(db * 16 + r) * 64] * wb;
+    }
+    __syncthreads();  // the staging area of the stores below overlaps the exchange area
+    if (kh != 0) return;
+  }
   // ---- epilogue: normalise, write lse, transpose O^T through LDS for coalesced 16-byte stores
   const float l_tot = half_sum(l_i);
   const bool empty = !(l_tot > 0.f);  // also catches NaN (fmha_fprop_kernel_1xN.h:575,606)
@@ -300,9 +343,9 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
     return;
   }
   if (hf == 0 && qrow < Lq) p.lse[((int64_t)b * p.H + h) * p.sq_r + qrow] = lse_val;
-  __syncthreads();
+  if (KS == 1) __syncthreads();
   constexpr int OS = Cfg::OS;
-  T* Os = reinterpret_cast<T*>(lds_raw) + wave * 32 * OS;
+  T* Os = reinterpret_cast<T*>(lds_raw) + rs * 32 * OS;
 #pragma unroll
   for (int db = 0; db < DV / 32; db++)
 #pragma unroll

@@ -122,8 +122,8 @@ FA_DEVICE bool seq_extent(const int32_t* cu, int b, int total, int max_len, int*
 
 // Workgroup id -> (batch*head, tile rank).  The hardware deals consecutive workgroup ids to the 8 XCDs in turn
 // (id % 8), and each XCD has its own L2.
-//   kTileMajor = false (tiles of equal cost): every XCD gets a contiguous range of (bh, tile) pairs, so the tiles of
-//     one (batch, head) run on one XCD at about the same time and share its L2 copy of the streamed operand.
+//   kTileMajor = false (tiles of equal cost): the tiles of one (batch, head) are consecutive in one XCD's share of the
+//     ids, so they run on one XCD at about the same time and share its L2 copy of the streamed operand.
 //   kTileMajor = true (causal: tile cost grows with the rank reversed): ids enumerate tile ranks outermost, so the
 //     most expensive tiles of all (batch, head) pairs start first; batch*head is padded to a multiple of 8 so that a
 //     given (batch, head) still always lands on the same XCD.
@@ -146,15 +146,31 @@ FA_DEVICE bool map_tile(int block, int tiles_per_bh, int BH, int* bh, int* rank)
     *bh = block - *rank * bhp;
     return *bh < BH && *rank < tiles_per_bh;
   }
-  const int total = tiles_per_bh * BH;
-  const int per_xcd = (total + 7) >> 3;
-  const int vid = (block & 7) * per_xcd + (block >> 3);
-  *bh = vid / tiles_per_bh;
-  *rank = vid - *bh * tiles_per_bh;
-  return vid < total;
+  // XCD x takes the (batch, head) pairs x, x + 8, x + 16, ... and all their tiles: the heads of one batch entry - which
+  // share its sequence length - are spread over the XCDs, so a ragged batch loads the XCDs evenly
+  // The tile ranks are rotated from one pair to the next: the hardware deals consecutive ids of an XCD to its compute
+  // units in turn, so with a power-of-two tile count a compute unit would always get the same rank - and in a ragged
+  // batch the last ranks are the ones that often lie beyond a sequence's end.
+  const int j = block >> 3;
+  const int q = j / tiles_per_bh;
+  *bh = (block & 7) + 8 * q;
+  *rank = (j - q * tiles_per_bh + q) % tiles_per_bh;
+  return *bh < BH;
 }
 inline int tile_grid(bool tile_major, int tiles_per_bh, int BH) {
-  return tile_major ? ((BH + 7) & ~7) * tiles_per_bh : ((tiles_per_bh * BH + 7) / 8) * 8;
+  return ((BH + 7) & ~7) * tiles_per_bh;
+}
+
+// Launch shape: with 128-row (128-key) tiles a short-sequence batch gives fewer workgroups than three per compute unit;
+// the kernels then run their half-size tile variants (twice the workgroups, half the serial work of each).
+// launch_policy(): 0 = by this rule, 1 = always the full-size tiles, 2 = the half-size tiles wherever they exist
+// (fa_set_launch_policy; the parity tests run both shapes on the same inputs).
+int launch_policy();
+inline bool small_launch(int BH, int max_s, bool causal) {
+  const int policy = launch_policy();
+  if (policy != 0) return policy == 2;
+  const int64_t wgs = (int64_t)BH * ((max_s + 127) / 128);
+  return wgs < (causal ? 6 : 3) * 256;
 }
 
 // Launchers (defined in fa_fwd.hip / fa_bwd.hip / fa_aux.hip).  Return hipError_t of the launch.

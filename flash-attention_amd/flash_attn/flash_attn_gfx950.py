@@ -95,7 +95,7 @@ class RotaryArgs(ctypes.Structure):
 EXPORTED_SYMBOLS = (
     "fa_fwd", "fa_bwd", "fa_fwd_block", "fa_bwd_block", "fa_fwd_block_noalloc", "fa_fwd_workspace_bytes", "fa_bwd_workspace_bytes",
     "fa_round_seqlens", "fa_philox_offset_increment", "fa_last_error", "fa_abi_version",
-    "fa_gather_rows", "fa_scatter_rows", "fa_scatter_rows_workspace_bytes", "fa_rotary",
+    "fa_gather_rows", "fa_scatter_rows", "fa_scatter_rows_workspace_bytes", "fa_rotary", "fa_set_launch_policy",
 )
 
 _lib = None
@@ -144,10 +144,21 @@ def load_library():
         lib.fa_scatter_rows_workspace_bytes.restype = ctypes.c_size_t
         lib.fa_rotary.argtypes = [ctypes.POINTER(RotaryArgs)]
         lib.fa_rotary.restype = ctypes.c_int
+        lib.fa_set_launch_policy.argtypes = [ctypes.c_int]
+        lib.fa_set_launch_policy.restype = ctypes.c_int
         if lib.fa_abi_version() != FA_ABI_VERSION:
             raise RuntimeError("%s has ABI version %d, binding expects %d" % (LIB_NAME, lib.fa_abi_version(), FA_ABI_VERSION))
         _lib = lib
     return _lib
+
+
+def set_launch_policy(policy):
+    """0: tile shapes chosen per launch (default); 1: always the full-size tiles; 2: the half-size tiles wherever they
+    exist (fa_set_launch_policy)."""
+    lib = load_library()
+    rc = lib.fa_set_launch_policy(int(policy))
+    if rc != 0:
+        _raise(rc, lib)
 
 
 @functools.lru_cache(maxsize=256)

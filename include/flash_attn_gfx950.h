@@ -209,6 +209,13 @@ typedef struct fa_rotary_args {
 } fa_rotary_args;
 int fa_rotary(const fa_rotary_args* args);
 
+/* Tile shape selection (process-wide; no counterpart in the reference, whose launchers pick their tile by head size
+ * and sequence length alone, fmha_api.cpp:232-241).  0 (default): short-sequence launches that would leave compute units
+ * idle with the full-size tiles (128 query rows / 128 keys per workgroup) use the half-size variants where they exist
+ * (head_dim <= 64, no blockmask, no alibi_slopes); 1: always full-size; 2: always half-size where they exist.  Results
+ * agree within rounding between the shapes (the order of fp32 summation differs), not bit for bit. */
+int fa_set_launch_policy(int policy);
+
 /* Message for the last non-zero status returned on the calling thread. */
 const char* fa_last_error(void);
 int fa_abi_version(void);

@@ -35,6 +35,25 @@ def _need_gpu(lib):
     assert torch.cuda.is_available(), "these tests need the MI355X"
 
 
+@pytest.fixture(params=[1, 2], ids=["full-size tiles", "half-size tiles"])
+def tile_shape(request):
+    """Runs a test with both tile shapes of the dense kernels (the library picks per launch by default; the half-size
+    variants exist for head dims up to 64): fa_set_launch_policy."""
+    from flash_attn import flash_attn_gfx950 as be
+    be.set_launch_policy(request.param)
+    yield request.param
+    be.set_launch_policy(0)
+
+
+@pytest.fixture
+def full_size_tiles():
+    """Bitwise comparisons between launches of different sizes hold for one tile shape, not across the automatic choice."""
+    from flash_attn import flash_attn_gfx950 as be
+    be.set_launch_policy(1)
+    yield
+    be.set_launch_policy(0)
+
+
 def _cu(lens, device="cuda"):
     return torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32, device=device)
 
@@ -143,7 +162,7 @@ def _parity_case(lens_q, lens_k, H, D, dtype, causal, packing="sep", seed=0, sca
 @pytest.mark.parametrize("D", [16, 32, 64, 128])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("causal", [False, True])
-def test_parity_head_dims(D, dtype, causal):
+def test_parity_head_dims(D, dtype, causal, tile_shape):
     _parity_case([113, 256, 37], [113, 256, 37], 3, D, dtype, causal, packing="qkv", seed=D)
 
 
@@ -157,7 +176,7 @@ def test_parity_head_dims(D, dtype, causal):
     ([5, 0, 9], [5, 0, 9]),          # an empty sequence in the batch
 ])
 @pytest.mark.parametrize("causal", [False, True])
-def test_parity_ragged_shapes(lens_q, lens_k, causal):
+def test_parity_ragged_shapes(lens_q, lens_k, causal, tile_shape):
     _parity_case(lens_q, lens_k, 2, 64, torch.float16, causal, packing="kv", seed=len(lens_q))
 
 
@@ -166,7 +185,7 @@ def test_parity_separate_qkv_and_scale():
     _parity_case([100, 140], [100, 140], 4, 32, torch.float16, True, packing="sep", seed=6, scale=0.05)
 
 
-def test_max_seqlen_may_exceed_the_longest_sequence():
+def test_max_seqlen_may_exceed_the_longest_sequence(tile_shape):
     _parity_case([70, 33], [70, 33], 2, 64, torch.float16, False, packing="qkv", seed=7, max_pad=200)
 
 
@@ -211,7 +230,7 @@ def test_softmax_d_and_raw_c_abi():
     assert torch.equal(o2, o) and torch.isinf(lse2[0, :, 50:]).all() and torch.equal(lse2[1, :, :77], lse[1, :, :77])
 
 
-def test_strided_views_and_noncontiguous_grads():
+def test_strided_views_and_noncontiguous_grads(tile_shape):
     """q, k, v as views of a packed tensor with extra padding between rows (row stride != 3*H*D)."""
     from flash_attn import flash_attn_gfx950 as be
     lens = [40, 90]
@@ -268,7 +287,7 @@ def _gen_state():
 
 
 @pytest.mark.parametrize("D,dtype,causal", [(64, torch.float16, False), (32, torch.bfloat16, True), (128, torch.float16, False)])
-def test_dropout_mask_is_the_defined_one_and_is_applied(D, dtype, causal):
+def test_dropout_mask_is_the_defined_one_and_is_applied(D, dtype, causal, tile_shape):
     p = 0.17
     lens_q, lens_k, H = [70, 130], [70, 130], 3
     q, k, v, do = _inputs(lens_q, lens_k, H, D, dtype, 21)
@@ -295,7 +314,7 @@ def test_dropout_mask_is_the_defined_one_and_is_applied(D, dtype, causal):
     check_against_oracle(ours, ref, half, dtype, what="dropout D%d" % D)
 
 
-def test_dropout_random_shapes_sweep():
+def test_dropout_random_shapes_sweep(tile_shape):
     """Eight seeded random dropout cases (rates, head dims, ragged self- and cross-attention lengths, packings): the
     returned mask equals its definition bit for bit and out / gradients equal the closed form with that mask."""
     rng = np.random.default_rng(77)
@@ -457,7 +476,7 @@ def test_sequence_of_64k_tokens(causal):
     assert (grad[cols, 1].float().transpose(0, 1) - dk_ref).abs().max() < tol(dk_ref)
 
 
-def test_parity_random_shapes_sweep():
+def test_parity_random_shapes_sweep(tile_shape):
     """Twenty-four seeded random cases over what the parametrised tests hold fixed: batch size, ragged query and key
     lengths (self- and cross-attention, empty key sides excluded), heads, head dim, dtype, causal, packing, scale."""
     rng = np.random.default_rng(2024)
@@ -695,7 +714,7 @@ def test_blocksparse_random_layouts_sweep():
         check_against_oracle(ours, ref, half, dtype, what=what)
 
 
-def test_blocksparse_full_layout_equals_dense():
+def test_blocksparse_full_layout_equals_dense(full_size_tiles):
     from flash_attn.flash_blocksparse_attn_interface import flash_blocksparse_attn_func
     from flash_attn.flash_attn_interface import flash_attn_unpadded_qkvpacked_func
     N, H, D = 600, 2, 64
@@ -837,7 +856,7 @@ def _full_size_check(lens, H, D, dtype, causal, p=0.0, seed=0):
     return q, k, v, do, cu, ours
 
 
-def test_config_bert_varlen_dropout():
+def test_config_bert_varlen_dropout(tile_shape):
     """BASELINE config 2: fp16, B=8, H=12, d=64, lengths uniform in [256, 512], p=0.1."""
     g = torch.Generator().manual_seed(0)
     lens = torch.randint(256, 513, (8,), generator=g).tolist()
@@ -886,7 +905,7 @@ def test_config_blocksparse_long_sequence():
     check_against_oracle(ours, ref, half, torch.float16, what="blocksparse N4096")
 
 
-def test_size_independent_properties_at_full_size():
+def test_size_independent_properties_at_full_size(full_size_tiles):
     """varlen == per-sequence dense; batch permutation; linearity in V; uniform attention for q = 0."""
     from flash_attn.flash_attn_interface import flash_attn_unpadded_func
     H, D = 12, 64
