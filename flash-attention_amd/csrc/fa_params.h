@@ -170,7 +170,8 @@ inline bool small_launch(int BH, int max_s, bool causal) {
   const int policy = launch_policy();
   if (policy != 0) return policy == 2;
   const int64_t wgs = (int64_t)BH * ((max_s + 127) / 128);
-  return wgs < (causal ? 6 : 3) * 256;
+  (void)causal;
+  return wgs < 3 * 256;
 }
 
 // Launchers (defined in fa_fwd.hip / fa_bwd.hip / fa_aux.hip).  Return hipError_t of the launch.

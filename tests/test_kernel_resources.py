@@ -44,21 +44,27 @@ def _pick(res, *parts):
 def test_d64_kernels_keep_their_waves_per_simd():
     fwd = _resources("fa_fwd_d64.hip")
     bwd = _resources("fa_bwd_d64.hip")
-    # <f16, 64, ..., causal, dropout, sparse, alibi> mangled as ...IDF16_Li64E...Lb{0,1}E x4
+    # <f16, 64, ..., causal, dropout, sparse, alibi, key split> mangled as ...IDF16_Li64E...Lb{0,1}E x4 Li{1,2}E
+    # (the dK/dV kernel has no key-split parameter)
     plain, causal, dropout = "Lb0ELb0ELb0ELb0E", "Lb1ELb0ELb0ELb0E", "Lb0ELb1ELb0ELb0E"
+    full = "Li1EEEv"
     for flags, want in ((plain, 4), (causal, 4), (dropout, 3)):
-        k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags)
+        k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags + full)
         assert k["Occupancy"] >= want and k["VGPRs Spill"] == 0, ("forward", flags, k)
+        k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags + "Li2EEEv")  # half-size tiles
+        assert k["Occupancy"] >= 4 and k["VGPRs Spill"] == 0, ("forward, key split", flags, k)
     for flags, want in ((plain, 3), (causal, 3), (dropout, 3)):
-        k = _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", flags)
+        k = _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", flags + full)
         assert k["Occupancy"] >= want and k["VGPRs Spill"] == 0, ("dq", flags, k)
+        k = _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", flags + "Li2EEEv")
+        assert k["Occupancy"] >= 3 and k["VGPRs Spill"] == 0, ("dq, key split", flags, k)
     for flags, want, spill in ((plain, 3, 2), (causal, 3, 2), (dropout, 2, 0)):
         k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", flags)
         assert k["Occupancy"] >= want and k["VGPRs Spill"] <= spill, ("dkdv", flags, k)
     # the ALiBi variants (fourth flag set) keep the waves per SIMD of their plain counterparts
     for flags in ("Lb0ELb0ELb0ELb1E", "Lb1ELb0ELb0ELb1E"):
-        assert _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags)["Occupancy"] >= 4, flags
-        assert _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", flags)["Occupancy"] >= 3, flags
+        assert _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags + full)["Occupancy"] >= 4, flags
+        assert _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", flags + full)["Occupancy"] >= 3, flags
         k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", flags)
         assert k["Occupancy"] >= 3 and k["VGPRs Spill"] <= 4, (flags, k)
 
@@ -72,5 +78,5 @@ def test_d128_backward_keeps_two_waves_per_simd():
         for flags in ("Lb0ELb0ELb0ELb0E", "Lb1ELb0ELb0ELb0E", "Lb0ELb0ELb1ELb0E", "Lb1ELb0ELb1ELb0E"):
             k = _pick(bwd, "fa_bwd_dkdv_kernel%sLi128E" % dt, flags)
             assert k["Occupancy"] >= 2 and k["VGPRs Spill"] == 0 and k["LDS Size"] <= 80 * 1024, (dt, flags, k)
-            k = _pick(bwd, "fa_bwd_dq_kernel%sLi128E" % dt, flags)
+            k = _pick(bwd, "fa_bwd_dq_kernel%sLi128E" % dt, flags + "Li1EEEv")
             assert k["Occupancy"] >= 2 and k["VGPRs Spill"] <= (1 if "Lb1ELb0E" in flags[8:] else 0), ("dq", dt, flags, k)
