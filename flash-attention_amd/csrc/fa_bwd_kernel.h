@@ -545,7 +545,9 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
     }
     if (wave_work) {
       // tiles that straddle the key length, the diagonal or an inactive row block get their dead scores set to -inf
-      const bool need_mask = (n0 + BN > Lk) || (kCausal && (n0 + BN - 1 > mw)) || (kSparse && !row_on);
+      // (an inactive row block inside an active tile is switched off through its lanes' lse, not score by score)
+      const bool need_mask = (n0 + BN > Lk) || (kCausal && (n0 + BN - 1 > mw));
+      const float lse_t = (kSparse && !row_on) ? INFINITY : lse2;  // P = exp2(finite - inf) = 0
 #pragma unroll
       for (int kbi = 0; kbi < KBW; kbi++) {
         const int kb = kb0 + kbi;
@@ -568,7 +570,6 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
             const int key = n0 + kb * 32 + (r >> 2) * 8 + hf * 4 + (r & 3);
             bool dead = key >= Lk;
             if (kCausal) dead = dead || key > qrow;
-            if (kSparse) dead = dead || !row_on;
             if (dead) s[r] = -INFINITY;
           }
         }
@@ -577,11 +578,11 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
         const float dbase = (float)(n0 + kb * 32 + hf * 4 - qrow);  // key - query of register 0 (kAlibi)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          float e = -lse2;
+          float e = -lse_t;
           if (kAlibi) {  // -slope2 * |key - query| - lse; under a causal mask live scores have key <= query
             const float cr = (float)((r >> 2) * 8 + (r & 3));
-            e = kCausal ? __builtin_fmaf(cr, sl2, __builtin_fmaf(dbase, sl2, -lse2))
-                        : __builtin_fmaf(__builtin_fabsf(dbase + cr), -sl2, -lse2);
+            e = kCausal ? __builtin_fmaf(cr, sl2, __builtin_fmaf(dbase, sl2, -lse_t))
+                        : __builtin_fmaf(__builtin_fabsf(dbase + cr), -sl2, -lse_t);
           }
           const float pe = fast_exp2(__builtin_fmaf(s[r], cs, e));  // 0 for dead scores and switched-off rows
           float dpe = kInitNegD ? dp[r] : dp[r] - dkv;  // dP - Dk

@@ -195,7 +195,9 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
         }
       }
       // ---- mask (only tiles that straddle the key length, the diagonal, or an inactive row block)
-      const bool need_mask = (n0 + BN > Lk) || (kCausal && (n0 + BN - 1 > mw)) || (kSparse && !row_on);
+      // (an inactive row block inside an active tile is not masked score by score: its lanes' maximum is dropped and their
+      // exponentials are taken against +inf below, which costs three instructions instead of two per score)
+      const bool need_mask = (n0 + BN > Lk) || (kCausal && (n0 + BN - 1 > mw));
       if (need_mask) {
 #pragma unroll
         for (int kb = 0; kb < KBW; kb++)
@@ -204,7 +206,6 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
             const int key = n0 + (kb0 + kb) * 32 + (r >> 2) * 8 + hf * 4 + (r & 3);
             bool dead = key >= Lk;
             if (kCausal) dead = dead || key > qrow;
-            if (kSparse) dead = dead || !row_on;
             if (dead) s[kb][r] = -INFINITY;
           }
       }
@@ -228,6 +229,7 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
 #pragma unroll
         for (int r = 0; r < 16; r++) mt = fmaxf(mt, s[kb][r]);
       mt = half_max(mt);
+      if (kSparse && !row_on) mt = -INFINITY;  // this lane's row block does not attend the tile
       // The reference point m_i of the exponentials only moves when some row's maximum has grown by more than
       // 2^kRescaleLog2 since it was set; until then P may exceed 1 by at most that factor, which the fp32 accumulators and
       // the fp16/bf16 rounding of P absorb, and the accumulators need no rescaling (numerator and denominator carry the
@@ -241,7 +243,8 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
 #pragma unroll
         for (int i = 0; i < DV / 32; i++) o_acc[i] = o_acc[i] * alpha;
       }
-      const float mc = ((m_i == -INFINITY) ? 0.f : m_i) * cse;
+      float mc = ((m_i == -INFINITY) ? 0.f : m_i) * cse;
+      if (kSparse && !row_on) mc = INFINITY;  // P = exp2(finite - inf) = 0
       float rsum = 0.f;
 #pragma unroll
       for (int kb = 0; kb < KBW; kb++)
