@@ -158,28 +158,48 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
     return -statpre;
   };
 
-  // Sparse: the activity bits of 64 consecutive 16-row blocks (16 query tiles) for this key block sit in a register
-  // pair; a query tile is visited iff one of its four row blocks attends the key block.
-  uint64_t col_bits = 0;
-  int bits_word = -1;
-  constexpr int TPW = 64 / RBT;  // query tiles per 64-bit activity word
-  auto tile_rows_on = [&](int mt) -> uint32_t {  // bit j: 16-row block j of query tile mt attends this key block
-    if ((mt / TPW) != bits_word) {
-      bits_word = __builtin_amdgcn_readfirstlane(mt / TPW);
-      col_bits = uniform64(p.sp.cbits[(int64_t)(n0 >> 8) * p.sp.nrw + bits_word]);
-    }
-    return (uint32_t)(col_bits >> (RBT * (mt % TPW))) & ((1u << RBT) - 1);
+  // Sparse: the tiles are not slices of the query side but packed lists of the 16-row blocks that attend this key block
+  // (what the reference's converted block list holds per key block, fmha_blockmask.h:41-53): RBT listed blocks make a
+  // tile, their rows are gathered when the tile is staged, so no row of an MFMA is masked and no tile is staged for
+  // less than RBT active blocks (but the last).  The list is read off the key block's activity bits, 64 row blocks per word.
+  struct BlockTile {
+    int rb[RBT];  // sequence-local 16-row block indices, ascending; -1 = none (only at the end of the last tile)
   };
-  // First query tile >= mt with a set bit (mt_end if none), found with a count-trailing-zeros on the loaded word
-  auto next_active = [&](int mt) -> int {
-    if (!kSparse) return mt;
-    while (mt < mt_end) {
-      tile_rows_on(mt);  // loads the word of mt if needed
-      const uint64_t rest = col_bits >> (RBT * (mt % TPW));  // low RBT bits: this tile's row blocks
-      if (rest & ((1u << RBT) - 1)) break;
-      mt = rest ? mt + (int)__builtin_ctzll(rest) / RBT : (mt | (TPW - 1)) + 1;
+  uint64_t word = 0;
+  const int nrb_q = (Lq + 15) >> 4;                               // row blocks that hold rows of this sequence
+  const int rb_first = kCausal ? (n0 >> 4) : 0;                   // earlier rows see none of this tile's keys
+  const int nwords = kSparse ? (((nrb_q < p.sp.nrb ? nrb_q : p.sp.nrb) + 63) >> 6) : 0;
+  int wi = (rb_first >> 6) - 1;
+  auto next_tile = [&](BlockTile& t) -> bool {  // the next RBT listed blocks; false if there is none
+#pragma unroll
+    for (int j = 0; j < RBT; j++) {
+      while (word == 0 && wi + 1 < nwords) {
+        wi = __builtin_amdgcn_readfirstlane(wi + 1);
+        word = uniform64(p.sp.cbits[(int64_t)(n0 >> 8) * p.sp.nrw + wi]);
+        if (wi * 64 < rb_first) word &= ~uint64_t(0) << (rb_first - wi * 64);        // (only the first word)
+        if (nrb_q - wi * 64 < 64) word &= (uint64_t(1) << (nrb_q - wi * 64)) - 1;     // (only the last word)
+      }
+      t.rb[j] = -1;
+      if (word != 0) {
+        t.rb[j] = wi * 64 + (int)__builtin_ctzll(word);
+        word &= word - 1;
+      }
     }
-    return mt < mt_end ? mt : mt_end;
+    return t.rb[0] >= 0;
+  };
+  auto stage_blocks = [&](const BlockTile& t, int buf) {
+    if (tid < 2 * BM) {
+      const int tr = tid < BM ? tid : tid - BM;
+      int blk = -1;
+#pragma unroll
+      for (int j = 0; j < RBT; j++)
+        if ((tr >> 4) == j) blk = t.rb[j];
+      const int row = blk * 16 + (tr & 15);
+      const bool live = blk >= 0 && row < Lq;
+      statpre = tid < BM ? INFINITY : 0.f;  // rows of no block or past the end are switched off (P = 0)
+      if (live) statpre = tid < BM ? lsebase[row] : dsbase[row];
+    }
+    stager.issue_blocks(lds_raw + buf * kBufBytes, t.rb, Lq);
   };
 
   f32x16 acc_dk[DV / 32], acc_dv[DV / 32];
@@ -204,24 +224,31 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
   }
   int buf = 0;
 
-  int mt = next_active(mt_begin);
-  if (mt < mt_end) stage(mt, 0);
-  while (mt < mt_end) {
+  int mt = mt_begin;          // dense: the query tile in use
+  BlockTile tc, tn;           // sparse: the packed tile in use / being staged
+  bool more = kSparse ? next_tile(tc) : mt < mt_end;
+  if (more) {
+    if (kSparse) stage_blocks(tc, 0);
+    else stage(mt, 0);
+  }
+  while (more) {
     const int m0 = mt * BM;
-    wait_vmem();  // this thread's share of tile `mt` has arrived (LDS) / is in statpre
+    wait_vmem();  // this thread's share of the tile has arrived (LDS) / is in statpre
     float* const lse_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffStat + buf * Cfg::kStatBytes);
     float* const dk_l = lse_l + BM;
     if (tid < 2 * BM) lse_l[tid] = stat_value();
-    uint32_t rows_on = (1u << RBT) - 1;  // bit j: 16-row block j of this tile attends this key block
-    if (kSparse) rows_on = tile_rows_on(mt);
-    __syncthreads();  // tile `mt` is complete, and nobody still reads the other buffer
-    const int mt_next = next_active(mt + 1);
-    if (mt_next < mt_end) stage(mt_next, buf ^ 1);
+    __syncthreads();  // the tile is complete, and nobody still reads the other buffer
+    if (kSparse) {
+      more = next_tile(tn);
+      if (more) stage_blocks(tn, buf ^ 1);
+    } else {
+      more = mt + 1 < mt_end;
+      if (more) stage(mt + 1, buf ^ 1);
+    }
     const T* const Ql = reinterpret_cast<const T*>(lds_raw + buf * kBufBytes);
     const T* const dOl = Ql + BM * D;
     buf ^= 1;
 
-    const bool diag = kCausal && (m0 < n0 + wave * 32 + 32);  // some (q, key) of this wave's slab has key > q
 
     // LDS fragment fetches sit next to their use; the other waves of the SIMD hide their latency.
     auto load_rows = [&](int qb, vec8* aq, vec8* ad) {
@@ -246,12 +273,11 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
       // dropout: the two slabs' Philox streams are not to be interleaved by the scheduler (it would, for the sake of
       // instruction-level parallelism, and need 70 more registers: one wave per SIMD fewer)
       if (kDropout) __builtin_amdgcn_sched_barrier(0);
-      bool rb_on[2] = {true, true};
-      if (kSparse) {
-        rb_on[0] = (rows_on >> (2 * qb)) & 1;
-        rb_on[1] = (rows_on >> (2 * qb + 1)) & 1;
-        if (!(rb_on[0] || rb_on[1])) continue;  // no row of this slab attends the key block: nothing to add to dK, dV
-      }
+      // first query rows of the slab's two 16-row halves (sparse: of the two listed blocks; ascending)
+      const int q_lo = kSparse ? tc.rb[2 * qb] * 16 : m0 + qb * 32;
+      const int q_hi = kSparse ? tc.rb[2 * qb + 1] * 16 : q_lo + 16;
+      if (kSparse && q_lo < 0) continue;  // the last tile's list ended before this slab
+      const bool diag = kCausal && ((kSparse ? q_lo : m0) < n0 + wave * 32 + 32);  // some (q, key) of the wave's has key > q
       // ---- S = Q K^T and dP = dO V^T for 32 query rows x this wave's 32 keys
       // dP starts from -Dk of its query row (fmha_dgrad_kernel_1xN_loop.h:361-371), so the MFMA delivers dP - Dk
       f32x16 s, dp;
@@ -270,20 +296,19 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
         dp = E::mfma32(ad[ks], kVLds ? *reinterpret_cast<const vec8*>(Vfrag + ks * 16) : vreg[ks], dp);
       // ---- P and dS'
       KeepFields keep;
-      if (kDropout) keep = keep_fields_col_layout(p.pk, (uint32_t)bh, m0 + qb * 32, key, hf);
+      if (kDropout) {  // this lane draws micro-block 2 (key % 4) + hf of the slab's eight (four query rows each)
+        const int mb = 2 * (key & 3) + hf;
+        keep = keep_fields_col_layout_q4(p.pk, (uint32_t)bh, (uint32_t)((mb < 4 ? q_lo : q_hi) >> 2) + (mb & 3), key);
+      }
       if (kCausal && diag) {  // only slabs that straddle the diagonal: scores above it become -inf (P = 0)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          const int qrow = m0 + qb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
+          const int qrow = kSparse ? (r < 8 ? q_lo : q_hi) + 8 * ((r >> 2) & 1) + 4 * hf + (r & 3)
+                                   : q_lo + 8 * (r >> 2) + 4 * hf + (r & 3);
           if (key > qrow) s[r] = -INFINITY;
         }
       }
-      if (kSparse && !(rb_on[0] && rb_on[1])) {  // an inactive 16-row block inside an active tile
-#pragma unroll
-        for (int r = 0; r < 16; r++)
-          if (!rb_on[r >> 3]) s[r] = -INFINITY;
-      }
-      const float dbase = (float)(key - m0 - qb * 32 - 4 * hf);  // key - query of register 0 (kAlibi)
+      const float dbase = (float)(key - m0 - qb * 32 - 4 * hf);  // key - query of register 0 (kAlibi; dense only)
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_l + qb * 32 + 8 * j + 4 * hf);
@@ -319,7 +344,8 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
         }
       }
     }
-    mt = mt_next;
+    if (kSparse) tc = tn;
+    else mt++;
   }
 
   // ---- epilogue: scale, transpose dK^T / dV^T through LDS, coalesced stores

@@ -244,10 +244,12 @@ FA_DEVICE KeepFields keep_fields_row_layout(const PhiloxKey& pk, uint32_t bh, in
   return e;
 }
 
-FA_DEVICE KeepFields keep_fields_col_layout(const PhiloxKey& pk, uint32_t bh, int q0, int key, int hf) {
+// Q4: the micro-block row (query row / 4) this lane draws - micro-block 2 (key % 4) + hf of the eight that cover the
+// tile's 32 query rows
+FA_DEVICE KeepFields keep_fields_col_layout_q4(const PhiloxKey& pk, uint32_t bh, uint32_t Q4, int key) {
   const int t = key & 3;
   uint32_t a[8];
-  philox_micro_block(pk, bh, ((uint32_t)q0 >> 2) + 2 * t + hf, (uint32_t)key >> 2, a);
+  philox_micro_block(pk, bh, Q4, (uint32_t)key >> 2, a);
   // Column c of a micro-block is half (c & 1) of its words of parity c >> 1.  Stage 1 swaps lane bit 1 against the
   // word parity; stage 2 swaps lane bit 0 against the half, by a byte permute whose selector depends on the lane:
   // even lanes keep their low half and take the neighbour's low half as high half, odd lanes the reverse.
@@ -263,6 +265,10 @@ FA_DEVICE KeepFields keep_fields_col_layout(const PhiloxKey& pk, uint32_t bh, in
       g.w[4 * pi + rho] = __builtin_amdgcn_perm(quad_perm<kQuadXor1>(cw), cw, sel);
     }
   return g;
+}
+// ... for 32 consecutive query rows q0 .. q0 + 31
+FA_DEVICE KeepFields keep_fields_col_layout(const PhiloxKey& pk, uint32_t bh, int q0, int key, int hf) {
+  return keep_fields_col_layout_q4(pk, bh, ((uint32_t)q0 >> 2) + 2 * (key & 3) + hf, key);
 }
 
 }  // namespace fa

@@ -125,6 +125,40 @@ struct TilePairStager {
       }
     }
   }
+
+  // The same for a tile whose rows are gathered from 16-row blocks of the tensors: tile rows 16 j .. 16 j + 15 are tensor
+  // rows 16 blk[j] .. 16 blk[j] + 15 (blk[j] wave-uniform; < 0: no block - some valid row is fetched and the caller
+  // switches those tile rows off).  Rows >= n_rows re-read the last valid row.
+  FA_DEVICE void issue_blocks(unsigned char* lds, const int (&blk)[ROWS / 16], int n_rows) const {
+    constexpr int SEG = RPI < 16 ? RPI : 16;  // rows of one block that one instruction covers
+    const int jb = row0 >> 4;                 // first block this wave fetches from
+#pragma unroll
+    for (int i = 0; i < NI; i++) {
+#pragma unroll
+      for (int sg = 0; sg < RPI / SEG; sg++) {  // two segments when an instruction spans two blocks (16-element rows)
+        const int tr = i * RPI + sg * 16;       // first tile row of the segment, relative to row0 (a multiple of 16)
+        int b = -1;
+#pragma unroll
+        for (int j = 0; j < ROWS / 16; j++)
+          if (jb + (tr >> 4) == j) b = blk[j];
+        int srow = (b < 0 ? 0 : b * 16) + (tr & 15);  // tensor row of the segment's first tile row
+        if (srow > n_rows - 1) srow = n_rows - 1;
+        const bool mine = RPI / SEG == 1 || (rl >> 4) == sg;
+        if (__builtin_expect(srow + SEG <= n_rows, 1)) {
+          // lane offsets count rows from the instruction's first tile row: rl rows (sg * 16 of them before this segment)
+          if (mine) dma16(base + ((int64_t)srow - sg * 16) * rsb, src_off[i % NOFF], lds + dst0 + i * 1024);
+        } else {
+          int rlv = rl, pchv = pch;
+          asm volatile("" : "+v"(rlv), "+v"(pchv));
+          const int within = rlv - sg * 16;
+          const int rc = srow + within < n_rows ? within : n_rows - 1 - srow;
+          if (mine)
+            dma16(base + (int64_t)srow * rsb, (uint32_t)(rc * rsb) + 16u * (uint32_t)(pchv ^ swz(row0 + i * RPI + rlv)),
+                  lds + dst0 + i * 1024);
+        }
+      }
+    }
+  }
 };
 
 // s_waitcnt vmcnt(0): every global load this wave has issued, direct-to-LDS ones included, has completed.
