@@ -53,6 +53,9 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 // strides are in elements: multiples of 8 (16-byte vectors), non-negative, and below 2^24 so that the kernels' 32-bit
 // per-lane byte offsets inside a tile (up to 63 rows) cannot overflow
 inline bool stride_ok(int64_t s) { return s % 8 == 0 && s >= 0 && s < ((int64_t)1 << 24); }
+// tensors that are written: rows and heads must not overlap (a zero or short stride would make several workgroups write
+// the same bytes)
+inline bool out_stride_ok(int64_t s, int head_dim) { return stride_ok(s) && s >= head_dim; }
 
 struct Rounded {
   int sq_r, sk_r;
@@ -171,10 +174,16 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
                  stride_ok(a->k_head_stride) && stride_ok(a->v_row_stride) && stride_ok(a->v_head_stride) &&
                  stride_ok(a->o_row_stride) && stride_ok(a->o_head_stride),
              "row and head strides must be multiples of 8 elements in [0, 2^24)");
+  FA_REQUIRE(out_stride_ok(a->o_row_stride, a->head_dim) && out_stride_ok(a->o_head_stride, a->head_dim),
+             "row and head strides of o must be at least head_dim (the output's rows and heads may not overlap)");
 
   if (sparse && a->alibi_slopes) return fail(FA_ERR_UNSUPPORTED, "alibi_slopes are not supported together with a blockmask");
 
   const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, sparse);
+  // the probability dump puts the rounded query length and batch * heads into grid dimensions: refuse what does not fit
+  // before anything is enqueued
+  if (a->s_dmask && (r.sq_r > 65535 || (int64_t)a->batch * a->nheads > 65535))
+    return fail(FA_ERR_UNSUPPORTED, "s_dmask is limited to max_seqlen_q <= 65535 and batch * nheads <= 65535");
   hipStream_t stream = reinterpret_cast<hipStream_t>(a->stream);
   const bool dropout = a->p_dropout > 0.f;
   const float p_keep = 1.f - a->p_dropout;
@@ -192,6 +201,9 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
   if (a->zero_tensors) {  // fmha_api.cpp:256-260
     FA_LAUNCH(fa::launch_zero_rows(a->o, a->o_row_stride, a->o_head_stride, a->total_q, a->nheads, a->head_dim, stream));
     FA_LAUNCH(fa::launch_fill_f32(a->softmax_lse, (size_t)a->batch * a->nheads * r.sq_r, -INFINITY, stream));
+    if (a->s_dmask)  // 16-bit elements, an even number of them (the rounded key length is a multiple of 128)
+      FA_LAUNCH(fa::launch_fill_f32(reinterpret_cast<float*>(a->s_dmask),
+                                    (size_t)a->batch * a->nheads * r.sq_r * r.sk_r / 2, 0.f, stream));
   }
 
   p.q = a->q; p.k = a->k; p.v = a->v; p.o = a->o; p.lse = a->softmax_lse;
@@ -258,6 +270,9 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
                              a->dq_row_stride, a->dq_head_stride, a->dk_row_stride, a->dk_head_stride, a->dv_row_stride,
                              a->dv_head_stride};
   for (int64_t s : strides) FA_REQUIRE(stride_ok(s), "row and head strides must be multiples of 8 elements in [0, 2^24)");
+  for (int i = 10; i < 16; i++)
+    FA_REQUIRE(out_stride_ok(strides[i], a->head_dim),
+               "row and head strides of dq, dk, dv must be at least head_dim (the gradients' rows and heads may not overlap)");
 
   const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, sparse);
   FA_REQUIRE(a->lse_seq_stride >= a->max_seqlen_q, "softmax_lse is shorter than max_seqlen_q");
@@ -453,6 +468,8 @@ int fa_rotary(const fa_rotary_args* a) {
   if (a->n_rows == 0) return FA_OK;
   FA_REQUIRE(a->src && a->dst && a->cos_table && a->sin_table, "fa_rotary: null pointer");
   FA_REQUIRE(a->table_rows >= 1 && (a->positions || a->seqlen >= 1), "fa_rotary: empty table or no positions");
+  FA_REQUIRE(a->positions || a->seqlen <= a->table_rows, "fa_rotary: the tables have %d rows, the sequence %d positions",
+             a->table_rows, a->seqlen);
   FA_REQUIRE(aligned16(a->src) && aligned16(a->dst) && (reinterpret_cast<uintptr_t>(a->cos_table) & 7) == 0 &&
                  (reinterpret_cast<uintptr_t>(a->sin_table) & 7) == 0,
              "fa_rotary: pointers must be 16-byte (tensors) / 8-byte (tables) aligned");

@@ -58,7 +58,7 @@ typedef struct fa_fwd_args {
   int64_t q_row_stride, q_head_stride;
   int64_t k_row_stride, k_head_stride;
   int64_t v_row_stride, v_head_stride;
-  int64_t o_row_stride, o_head_stride;
+  int64_t o_row_stride, o_head_stride; /* both >= head_dim: written rows and heads may not overlap */
   int32_t batch, nheads, head_dim;
   int32_t total_q, total_k;
   int32_t max_seqlen_q, max_seqlen_k; /* as given by the caller, before rounding */
@@ -91,7 +91,8 @@ typedef struct fa_bwd_args {
   void* dq;
   void* dk;
   void* dv;
-  float* softmax_d; /* [batch, nheads, max_seqlen_q_rounded] fp32: rowsum(dout * out) */
+  float* softmax_d; /* [batch, nheads, max_seqlen_q_rounded] fp32: (1 - p_dropout) * rowsum(dout * out), the reference's
+                       dp_sum * p_dropout (fmha_dgrad_kernel_1xN_loop.h:15-30,226) */
   const int32_t* cu_seqlens_q;
   const int32_t* cu_seqlens_k;
   const int32_t* blockmask;
@@ -190,7 +191,9 @@ size_t fa_scatter_rows_workspace_bytes(int64_t n_dst_rows);
  * src).  Parts 0 .. n_rotated-1 are rotated, the remaining parts are copied (packed qkv: n_parts 3, n_rotated 2).
  * Pair (x[2i], x[2i+1]) of a row at position t becomes (x[2i] c - x[2i+1] s, x[2i+1] c + x[2i] s) with
  * c = cos_table[t, i], s = sin_table[t, i]; tables are [table_rows, head_dim / 2] in the tensor's dtype;
- * t = positions[row] if positions != NULL, else row % seqlen.  conjugate != 0 negates s (the backward pass).
+ * t = positions[row] if positions != NULL (entries outside [0, table_rows) are clamped to the nearest table row: callers
+ * that cannot vouch for them check positions themselves), else row % seqlen (seqlen <= table_rows is required).
+ * conjugate != 0 negates s (the backward pass).
  * head_dim must be a multiple of 8; base pointers and strides must keep 16-byte alignment. */
 typedef struct fa_rotary_args {
   uint32_t struct_bytes;

@@ -4,9 +4,12 @@ same seeded inputs.
 Tolerance (stated by the build's target): for every output X in {out, dq, dk, dv}
     max|X_ours - X_ref32| <= 2 * max|X_half - X_ref32| + floor
 where X_ref32 is the fp32 closed form (oracle), X_half the same closed form evaluated by PyTorch in the input dtype
-(fp16/bf16) on the GPU, and floor = 1e-3 (fp16) / 8e-3 (bf16), or half an ulp of the largest |X_ref32| if that is more,
-absorbs outputs that are exactly representable in the half evaluation.  softmax_lse is fp32 on both sides:
-|lse_ours - lse_ref32| <= LSE_TOL = 1e-3 (fp16) / 4.5e-3 (bf16).
+(fp16/bf16) on the GPU, and floor = 2e-4 (fp16) / 2e-3 (bf16), or half an ulp of the largest |X_ref32| if that is more
+(two correct roundings of the same sum differ by that much), absorbs outputs that are exactly representable in the half
+evaluation.  Every comparison is recorded (error, yardstick, their ratio, how much of the floor was used) and the list is
+written to gpurun_out/parity_error_ratios.json at the end of the session.
+softmax_lse is fp32 on both sides and is held to two bounds: the same yardstick - the logsumexp PyTorch computes from
+half-precision scores - and an absolute cap |lse_ours - lse_ref32| <= LSE_TOL = 1e-3 (fp16) / 4.5e-3 (bf16).
 The inputs are exact; the forward kernel sums the probabilities after they have been rounded to the tensor dtype (the
 values the P V product consumes), so a row dominated by one key carries that one rounding: at most 2^-11 (fp16) or
 2^-8 (bf16) relative in the row sum, i.e. 4.9e-4 / 3.9e-3 absolute in its logarithm.  Dropout masks are compared bit for
@@ -24,7 +27,7 @@ from oracle import attention_oracle as orc
 
 pytestmark = pytest.mark.gpu
 
-FLOOR = {torch.float16: 1e-3, torch.bfloat16: 8e-3}
+FLOOR = {torch.float16: 2e-4, torch.bfloat16: 2e-3}
 LSE_TOL = {torch.float16: 1e-3, torch.bfloat16: 4.5e-3}
 HALF_ULP = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}
 GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
@@ -68,7 +71,7 @@ def _inputs(lens_q, lens_k, H, D, dtype, seed):
 def half_attention(q, k, v, cu_q, cu_k, scale, causal, keep_mask=None, p=0.0, layout=None, dout=None, alibi_slopes=None):
     """the closed form evaluated in the tensors' own half dtype by PyTorch (the error yardstick)"""
     q, k, v = (x.detach().clone().requires_grad_(dout is not None) for x in (q, k, v))
-    outs = []
+    outs, lses = [], []
     for b in range(len(cu_q) - 1):
         qb = q[cu_q[b]:cu_q[b + 1]].transpose(0, 1)
         kb = k[cu_k[b]:cu_k[b + 1]].transpose(0, 1)
@@ -81,12 +84,13 @@ def half_attention(q, k, v, cu_q, cu_k, scale, causal, keep_mask=None, p=0.0, la
         empty = ~valid.any(-1)
         s = s.masked_fill(empty[None, :, None], 0.0)
         pr = torch.softmax(s, dim=-1)
+        lses.append(torch.logsumexp(s, dim=-1).masked_fill(empty[None], float("-inf")).detach())
         pr = pr.masked_fill(~valid[None], 0.0)
         if keep_mask is not None:
             pr = pr * keep_mask[b].to(device=q.device, dtype=pr.dtype) / (1.0 - p)
         outs.append(torch.matmul(pr, vb).transpose(0, 1))
     out = torch.cat(outs, 0)
-    res = {"out": out.detach()}
+    res = {"out": out.detach(), "lse": lses}
     if dout is not None:
         out.backward(dout)
         res.update(dq=q.grad, dk=k.grad, dv=v.grad)
@@ -97,13 +101,42 @@ def _maxerr(a, b):
     return (a.float().cpu() - b.float().cpu()).abs().max().item()
 
 
+RATIOS = []  # one record per comparison against the oracle, written out by _write_ratios at the end of the session
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _write_ratios():
+    yield
+    out_dir = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
+    if RATIOS and os.path.isdir(out_dir):
+        import json
+        with open(os.path.join(out_dir, "parity_error_ratios.json"), "w") as f:
+            json.dump(RATIOS, f, indent=0)
+
+
 def check_against_oracle(ours, ref, half, dtype, names=("out", "dq", "dk", "dv"), what=""):
     for n in names:
         e_ours, e_half = _maxerr(ours[n], ref[n]), _maxerr(half[n], ref[n])
         # the floor is at least half an ulp of the largest output (gradients of a few tens are stored with a spacing of
         # 0.016 in fp16: two correct roundings of the same sum can differ by that much from the fp32 value)
         floor = max(FLOOR[dtype], HALF_ULP[dtype] * ref[n].float().abs().max().item())
+        RATIOS.append({"case": what, "output": n, "dtype": str(dtype)[6:], "err": e_ours, "err_half_precision_pytorch": e_half,
+                       "ratio": e_ours / e_half if e_half > 0 else None, "floor": floor,
+                       "floor_used": max(0.0, e_ours - 2 * e_half) / floor})
         assert e_ours <= 2 * e_half + floor, "%s %s: ours %.3e vs half-precision PyTorch %.3e" % (what, n, e_ours, e_half)
+
+
+def check_lse(got, want, half_lse, dtype, what=""):
+    """got, want, half_lse: (H, L) for one sequence; want fp32 oracle, half_lse PyTorch's logsumexp of half-precision scores"""
+    fin = torch.isfinite(want)
+    assert torch.equal(torch.isfinite(got), fin), what
+    if not fin.any():
+        return
+    e_ours = (got[fin] - want[fin]).abs().max().item()
+    e_half = (half_lse.float().cpu()[fin] - want[fin]).abs().max().item()
+    RATIOS.append({"case": what, "output": "lse", "dtype": str(dtype)[6:], "err": e_ours, "err_half_precision_pytorch": e_half,
+                   "ratio": e_ours / e_half if e_half > 0 else None, "floor": 1e-4, "floor_used": max(0.0, e_ours - 2 * e_half) / 1e-4})
+    assert e_ours <= 2 * e_half + 1e-4 and e_ours <= LSE_TOL[dtype], "%s lse: ours %.3e vs half-precision PyTorch %.3e" % (what, e_ours, e_half)
 
 
 def run_ours(q, k, v, do, cu_q, cu_k, max_q, max_k, p, scale, causal, packing="sep", probs=False, alibi_slopes=None):
@@ -148,11 +181,7 @@ def _parity_case(lens_q, lens_k, H, D, dtype, causal, packing="sep", seed=0, sca
     what = "q%s k%s H%d D%d %s causal=%s %s" % (lens_q, lens_k, H, D, dtype, causal, packing)
     check_against_oracle(ours, ref, half, dtype, what=what)
     for b, L in enumerate(lens_q):  # lse: only rows < seqlen_q are defined
-        got = ours["lse"][b, :, :L].cpu()
-        want = ref["lse"][b]
-        fin = torch.isfinite(want)
-        assert torch.equal(torch.isfinite(got), fin), what
-        assert (got[fin] - want[fin]).abs().max().item() <= LSE_TOL[dtype] if fin.any() else True, what
+        check_lse(ours["lse"][b, :, :L].cpu(), ref["lse"][b], half["lse"][b], dtype, what)
     return ours, ref
 
 
@@ -275,6 +304,41 @@ def test_error_behaviour_on_device():
     o, lse = be.fwd(q, q, q, cu2, cu2, 16, 16, 0.0, 0.125, False, False, False, None)
     torch.cuda.synchronize()
     assert torch.isfinite(o).all()
+
+
+def test_zero_tensors_prefills_what_the_kernels_do_not_write():
+    """zero_tensors = True (fmha_api.cpp:256-260, 406-411): rows of the packed tensors that belong to no sequence
+    (cu_seqlens[-1] < total) and the padding of lse / softmax_d / S_dmask come out as 0 / -inf instead of whatever the
+    buffers held; the rows of real sequences are what a call without the flag computes."""
+    from flash_attn import flash_attn_gfx950 as be
+    H, D, lens, extra = 2, 32, [40, 23], 9
+    total = sum(lens) + extra
+    g = torch.Generator().manual_seed(11)
+    q, k, v, do = (torch.randn(total, H, D, generator=g).half().cuda() for _ in range(4))
+    cu = _cu(lens)
+    used = sum(lens)
+    o, lse, S = be.fwd(q, k, v, cu, cu, max(lens), max(lens), 0.0, D ** -0.5, True, False, True, None)
+    o0, lse0 = be.fwd(q, k, v, cu, cu, max(lens), max(lens), 0.0, D ** -0.5, False, False, False, None)
+    torch.cuda.synchronize()
+    assert torch.equal(o[:used], o0[:used]) and o[used:].abs().max() == 0
+    assert torch.equal(lse[0, :, :40], lse0[0, :, :40]) and torch.isinf(lse[0, :, 40:]).all() and torch.isinf(lse[1, :, 23:]).all()
+    assert S[1, :, 23:].abs().max() == 0 and S[1, :, :, 23:].abs().max() == 0 and S[0, :, :40, :40].abs().max() > 0
+    grads = [torch.full((total, H, D), 7.0, dtype=torch.half, device="cuda") for _ in range(3)]
+    dq, dk, dv, sd = be.bwd(do, q, k, v, o, lse, grads[0], grads[1], grads[2], cu, cu, max(lens), max(lens), 0.0, D ** -0.5,
+                            True, False, None)
+    ref_g = [torch.full((total, H, D), 7.0, dtype=torch.half, device="cuda") for _ in range(3)]
+    _, _, _, sd0 = be.bwd(do, q, k, v, o0, lse0, ref_g[0], ref_g[1], ref_g[2], cu, cu, max(lens), max(lens), 0.0, D ** -0.5,
+                          False, False, None)
+    torch.cuda.synchronize()
+    for got, want in zip((dq, dk, dv), ref_g):
+        assert torch.equal(got[:used], want[:used]) and got[used:].abs().max() == 0 and (want[used:] == 7).all()
+    assert torch.equal(sd[0, :, :40], sd0[0, :, :40]) and sd[0, :, 40:].abs().max() == 0 and sd[1, :, 23:].abs().max() == 0
+    want_sd = (do[:40].float() * o[:40].float()).sum(-1).transpose(0, 1)  # p_dropout = 0: rowsum(dout * out)
+    assert (sd[0, :, :40] - want_sd).abs().max() < 2e-3
+    # written tensors may not overlap: a zero head stride of the output is refused before anything is launched
+    with pytest.raises(RuntimeError, match="may not overlap"):
+        bad = torch.empty(total, 1, D, dtype=torch.half, device="cuda").expand(total, H, D)
+        be.bwd(do, q, k, v, o, lse, bad, grads[1], grads[2], cu, cu, max(lens), max(lens), 0.0, D ** -0.5, False, False, None)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -543,11 +607,7 @@ def test_alibi_random_shapes_sweep():
         check_against_oracle(ours, ref, half, dtype, what=what)
         for b in range(B):
             Lq, Lk = lens_q[b], lens_k[b]
-            got, want = ours["lse"][b, :, :Lq].cpu(), ref["lse"][b]
-            fin = torch.isfinite(want)
-            assert torch.equal(torch.isfinite(got), fin), what
-            if fin.any():
-                assert (got[fin] - want[fin]).abs().max().item() <= LSE_TOL[dtype], what
+            check_lse(ours["lse"][b, :, :Lq].cpu(), ref["lse"][b], half["lse"][b], dtype, what)
             probs = ours["S_dmask"][b, :, :Lq, :Lk].float().cpu()
             assert (probs.abs() - ref["probs"][b]).abs().max().item() < (2e-3 if dtype == torch.float16 else 1e-2), what
 
