@@ -186,8 +186,10 @@ def test_philox_vectorised_equals_scalar():
 
 
 def test_keep_threshold_and_rate():
-    assert orc.keep_threshold(0.1) == int(math.floor(0.9 * 65535.0))  # fmha_api.cpp:110
-    assert orc.keep_threshold(0.0) == 65535 and orc.keep_probability(0.0) == 1.0
+    # fmha_api.cpp:110 computes floor(p_keep * 65535) for the uint16 comparison: values worked out by hand / exact
+    # binary fractions (0.5 * 65535 = 32767.5, 0.75 * 65535 = 49151.25, 0.9 * 65535 = 58981.5)
+    assert [orc.keep_threshold(x) for x in (0.0, 0.5, 0.25, 0.1)] == [65535, 32767, 49151, 58981]
+    assert orc.keep_probability(0.0) == 1.0 and orc.keep_probability(0.5) == 0.5 and orc.keep_probability(0.25) == 0.75
     p = 0.17
     m = orc.dropout_keep_mask(seed=42, offset=8, bh=3, Lq=256, Lk=512, p_dropout=p)
     n = m.size
