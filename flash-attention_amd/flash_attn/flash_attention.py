@@ -83,9 +83,10 @@ class FlashMHA(nn.Module):
     def forward(self, x, x_ignored_, x_ignored_1_, attn_mask=None, key_padding_mask=None, need_weights=False):
         b, s = x.shape[0], x.shape[1]
         qkv = self.Wqkv(x).reshape(b, s, 3, self.num_heads, self.head_dim)
-        if self.use_rotary_emb == "1d" and qkv.is_cuda and qkv.dtype in (torch.float16, torch.bfloat16):
-            qkv = self.rotary_emb.rotate_qkv_(qkv)  # q and k rotated in place by one kernel
-        elif self.use_rotary_emb:  # "2d" (no fused kernel for it): the reference's elementwise formulation, on the GPU
+        if self.use_rotary_emb and qkv.is_cuda and qkv.dtype in (torch.float16, torch.bfloat16) and (
+                self.use_rotary_emb == "1d" or self.head_dim % 16 == 0):
+            qkv = self.rotary_emb.rotate_qkv_(qkv)  # q and k rotated in place by the HIP kernel (one pass; "2d": two)
+        elif self.use_rotary_emb:  # other devices / dtypes: the reference's elementwise formulation
             query, key, value = qkv.unbind(dim=2)
             query, key = self.rotary_emb(query, key, seq_dimension=-3)
             qkv = torch.stack([query, key, value], dim=2)

@@ -91,6 +91,34 @@ class RotaryEmbedding(torch.nn.Module):
         return (apply_rotary_pos_emb(q, cos, sin, seq_dimension), apply_rotary_pos_emb(k, cos, sin, seq_dimension))
 
 
+class _ApplyRotaryQKV2D(torch.autograd.Function):
+    """In-place 2-D rotation of q and k of a packed qkv: channels [0, d/2) by the token's column, [d/2, d) by its row
+    (two passes of the same kernel over the two half-channel views, the position of every token given explicitly).  The
+    backward applies the opposite rotations to the incoming gradient."""
+
+    @staticmethod
+    def _rotate(t, cos_half, sin_half, col_pos, row_pos, conjugate):
+        from . import flash_attn_gfx950 as backend
+        half = t.shape[-1] // 2
+        lo, hi = t[..., :half], t[..., half:]
+        backend.rotary(lo, lo, cos_half, sin_half, n_rotated=2, conjugate=conjugate, positions=col_pos)
+        backend.rotary(hi, hi, cos_half, sin_half, n_rotated=2, conjugate=conjugate, positions=row_pos)
+
+    @staticmethod
+    def forward(ctx, qkv, cos_half, sin_half, col_pos, row_pos):
+        ctx.save_for_backward(cos_half, sin_half, col_pos, row_pos)
+        _ApplyRotaryQKV2D._rotate(qkv, cos_half, sin_half, col_pos, row_pos, False)
+        ctx.mark_dirty(qkv)
+        return qkv
+
+    @staticmethod
+    def backward(ctx, grad):
+        cos_half, sin_half, col_pos, row_pos = ctx.saved_tensors
+        grad = grad.clone(memory_format=torch.contiguous_format)
+        _ApplyRotaryQKV2D._rotate(grad, cos_half, sin_half, col_pos, row_pos, True)
+        return grad, None, None, None, None
+
+
 class RotaryEmbedding2D(torch.nn.Module):
     """Rotary embedding for a square grid of tokens (seqlen = side * side): the first half of the channels is
     rotated by the column index, the second half by the row index."""
@@ -99,6 +127,24 @@ class RotaryEmbedding2D(torch.nn.Module):
         super().__init__()
         assert dim % 4 == 0
         self.rotary_emb1d = RotaryEmbedding(dim // 2)
+        self._pos_cached = None
+
+    def rotate_qkv_(self, qkv):
+        """q and k of a packed (batch, side * side, 3, nheads, headdim) fp16 / bf16 GPU tensor rotated in place by the HIP
+        kernel (headdim a multiple of 16); returns qkv.  Same map as forward() on q and k, products in fp32, one rounding."""
+        b, seqlen = qkv.shape[0], qkv.shape[1]
+        side = int(math.sqrt(seqlen))
+        assert seqlen == side * side
+        grid = qkv[:, :side, 0, :, :qkv.shape[-1] // 2]  # (b, side, nheads, headdim / 2): `side` positions per axis
+        cos, sin = self.rotary_emb1d._update_cos_sin_tables(grid, seq_dimension=-3)
+        key = (b, side, qkv.device)
+        if self._pos_cached is None or self._pos_cached[0] != key:
+            tok = torch.arange(seqlen, device=qkv.device, dtype=torch.int32)
+            col = (tok % side).repeat(b).contiguous()
+            row = torch.div(tok, side, rounding_mode="floor").to(torch.int32).repeat(b).contiguous()
+            self._pos_cached = (key, col, row)
+        _, col, row = self._pos_cached
+        return _ApplyRotaryQKV2D.apply(qkv, cos[:, ::2].contiguous(), sin[:, ::2].contiguous(), col, row)
 
     def forward(self, q: torch.Tensor, k: torch.Tensor, seq_dimension=-2):
         assert seq_dimension in [-2, -3]

@@ -1213,6 +1213,46 @@ def test_rotary_kernel_matches_oracle(dtype, D):
     assert torch.equal(x.grad[:, :, 2].cpu(), go[:, :, 2])
 
 
+@pytest.mark.parametrize("dtype,D", [(torch.float16, 64), (torch.bfloat16, 32), (torch.float16, 16)])
+def test_rotary_2d_kernel_path_matches_oracle(dtype, D):
+    """RotaryEmbedding2D.rotate_qkv_ (flash_attn/rotary.py:103-135 done by two passes of fa_rotary over the half-channel
+    views, positions = column / row of the token in its square grid): against the fp64 rotation of each half, against
+    the module's own elementwise forward(), and its backward against the opposite rotation."""
+    from flash_attn.rotary import RotaryEmbedding2D
+    g = torch.Generator().manual_seed(D + 1)
+    B, side, H = 2, 7, 3
+    S, half = side * side, D // 2
+    qkv = torch.randn(B, S, 3, H, D, generator=g).to(dtype)
+    emb = RotaryEmbedding2D(D).cuda()
+    x = qkv.cuda().clone().requires_grad_(True)
+    y = emb.rotate_qkv_(x * 1.0)
+    cos, sin = emb.rotary_emb1d._cos_cached[:, ::2].double().cpu().numpy(), emb.rotary_emb1d._sin_cached[:, ::2].double().cpu().numpy()
+    tok = np.tile(np.arange(S), B)
+    col, row = tok % side, tok // side
+    ulp = 2.0 ** (-10 if dtype == torch.float16 else -7)
+
+    def close(got, want64):
+        got = got.detach().double().cpu().numpy()
+        assert np.all(np.abs(got - want64) <= ulp * np.abs(want64) * 0.51 + 1e-7), np.abs(got - want64).max()
+
+    for part in range(2):
+        src = qkv[:, :, part].reshape(B * S, H, D).double().numpy()
+        close(y[:, :, part, :, :half].reshape(B * S, H, half), orc.rotary_ref(src[..., :half], cos, sin, col))
+        close(y[:, :, part, :, half:].reshape(B * S, H, half), orc.rotary_ref(src[..., half:], cos, sin, row))
+    y_d = y.detach()
+    assert torch.equal(y_d[:, :, 2].cpu(), qkv[:, :, 2])
+    q_t, k_t = emb(qkv[:, :, 0].cuda(), qkv[:, :, 1].cuda(), seq_dimension=-3)  # elementwise formulation, three roundings
+    assert (q_t.float() - y_d[:, :, 0].float()).abs().max() <= 4.5 * ulp * qkv.abs().max()
+    assert (k_t.float() - y_d[:, :, 1].float()).abs().max() <= 4.5 * ulp * qkv.abs().max()
+    go = torch.randn(B, S, 3, H, D, generator=g).to(dtype)
+    y.backward(go.cuda())
+    for part in range(2):
+        src = go[:, :, part].reshape(B * S, H, D).double().numpy()
+        close(x.grad[:, :, part, :, :half].reshape(B * S, H, half), orc.rotary_ref(src[..., :half], cos, sin, col, conjugate=True))
+        close(x.grad[:, :, part, :, half:].reshape(B * S, H, half), orc.rotary_ref(src[..., half:], cos, sin, row, conjugate=True))
+    assert torch.equal(x.grad[:, :, 2].cpu(), go[:, :, 2])
+
+
 # ------------------------------------------------------------------------------------------------
 # key-split forward (short query side, long key side: decode / cross-attention shapes)
 # ------------------------------------------------------------------------------------------------
