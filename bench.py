@@ -1,14 +1,18 @@
 #!/usr/bin/env python3
 """Benchmark of the fused attention path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all] [--no-cpu] [--no-configs]
 
 One step = one forward + one backward pass of the headline workload (fp16, B=8, H=12, d=64, N=2048, packed qkv,
 non-causal, dropout 0, synthetic N(0,1) data resident in HBM), called through the C ABI.  Prints ONE JSON line:
 whole-job fwd+bwd TFLOP/s (4*B*H*N^2*d forward, 2.5x that backward), the roofline position of the dominant kernel
 (the backward dK/dV kernel, timed with HIP events recorded around it on its stream) and the CPU baseline (the
 oracle's standard attention, fp32 PyTorch on the host cores, timed on a bounded sample of the same workload).
---all additionally prints, to stderr, a table over the other BASELINE configurations.
+The line also carries `configs` (the other BASELINE configurations: TFLOP/s, share of the MFMA peak and the HBM GB/s of
+their algorithmic bytes; --no-configs skips them) and `sustained_mfma` (what a library fp16 GEMM reaches on this GPU in
+the same process: the matrix cores' rate under their power limit, to read the attention figures against).
+--all additionally prints the configurations as a table to stderr, with PyTorch standard attention timed beside each,
+and the unpad / pad / rotary kernels.
 """
 import argparse
 import json
@@ -256,6 +260,63 @@ def device_peak(torch):
             "tflops": round(cus * 4096 * mhz * 1e6 / 1e12, 1) if mhz else None}
 
 
+def sustained_mfma(torch, n=8192, iters=20):
+    """fp16 and bf16 torch.matmul (hipBLASLt / rocBLAS) on random n x n operands, timed after a settle phase: a library
+    routine's answer to what the matrix cores sustain on this GPU (they are power limited on operands that toggle)."""
+    out = {"what": "torch.matmul %d^3, random N(0,1) operands, after 0.3 s of the same GEMM" % n}
+    for name, dt in (("fp16_tflops", torch.float16), ("bf16_tflops", torch.bfloat16)):
+        a = torch.randn(n, n, device="cuda", dtype=dt)
+        b = torch.randn(n, n, device="cuda", dtype=dt)
+        t_end = time.perf_counter() + 0.3
+        while time.perf_counter() < t_end:
+            for _ in range(5):
+                a @ b
+            torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            a @ b
+        e1.record()
+        torch.cuda.synchronize()
+        out[name] = round(2.0 * n ** 3 / (e0.elapsed_time(e1) / iters * 1e-3) / 1e12, 1)
+        del a, b
+    return out
+
+
+TRAFFIC_PROFILE = os.path.join("profiles", "headline_fp16_b8_h12_d64_n2048_hbm_traffic.md")
+
+
+def measured_traffic():
+    """HBM bytes per launch of the dominant kernel, from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary (the line
+    `traffic_bytes_per_launch(<kernel>): <bytes>` there); None if the file does not carry it."""
+    try:
+        for line in open(os.path.join(ROOT, TRAFFIC_PROFILE)):
+            if line.startswith("traffic_bytes_per_launch(fa_bwd_dkdv_kernel"):
+                return float(line.split(":")[1])
+    except OSError:
+        pass
+    return None
+
+
+def config_list(torch):
+    return [
+        ("BERT varlen p=0.1 fp16", dict(B=8, H=12, D=64, N=512, dtype=torch.float16, p=0.1,
+                                        lens=torch.randint(256, 513, (8,), generator=torch.Generator().manual_seed(0)).tolist())),
+        # the configuration of the reference's own script (benchmarks/benchmark_flash_attention.py:39-70)
+        ("reference script B64 H16 p=0.1", dict(B=64, H=16, D=64, N=1024, dtype=torch.float16, p=0.1,
+                                                lens=torch.randint(1004, 1024, (64,), generator=torch.Generator().manual_seed(0)).tolist())),
+        ("GPT2 causal bf16 N=1024", dict(B=8, H=12, D=64, N=1024, dtype=torch.bfloat16, causal=True)),
+        ("GPT2 causal bf16 N=2048", dict(B=8, H=12, D=64, N=2048, dtype=torch.bfloat16, causal=True)),
+        ("GPT2 causal bf16 N=4096", dict(B=8, H=12, D=64, N=4096, dtype=torch.bfloat16, causal=True)),
+        ("  + ALiBi slopes, N=2048", dict(B=8, H=12, D=64, N=2048, dtype=torch.bfloat16, causal=True, alibi=True)),
+        ("d128 fp16 N=2048", dict(B=16, H=12, D=128, N=2048, dtype=torch.float16)),
+        ("d128 fp16 N=2048 causal", dict(B=16, H=12, D=128, N=2048, dtype=torch.float16, causal=True)),
+        ("blocksparse 25% 16x256", dict(B=4, H=16, D=64, N=4096, dtype=torch.float16, blockmask=sparse_layout(torch, 4096))),
+        ("blocksparse 25% 256x256", dict(B=4, H=16, D=64, N=4096, dtype=torch.float16,
+                                         blockmask=sparse_layout(torch, 4096, rows_per_draw=16))),
+    ]
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -263,6 +324,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--all", action="store_true", help="also time the other BASELINE configurations (stderr table)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-configs", action="store_true", help="skip the other BASELINE configurations (`configs` in the JSON line)")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
     ap.add_argument("--settle", type=float, default=0.2,
                     help="seconds of untimed steps before the warm-up (0 for counter-collection runs)")
@@ -310,10 +372,10 @@ def main():
                      "achieved": round(bwd_kernel_tflops, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(bwd_kernel_tflops / MFMA_PEAK_TFLOPS, 4),
                      "avg_launch_ms": round(t["bwd_main_kernel_ms"], 4),
-                     # HBM bytes per launch from rocprofv3 FETCH_SIZE x2.00 + WRITE_SIZE x1.00 (scale factors from a
-                     # 256 MiB copy): 101 461 KiB read + 50 688 KiB written
-                     "traffic": 155.8e6},
+                     # HBM bytes per launch from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE summary
+                     "traffic": measured_traffic(), "traffic_source": TRAFFIC_PROFILE},
     }
+    res["sustained_mfma"] = sustained_mfma(torch)
     pt_ms, pt_mem = torch_attention_ms(torch, w, want_memory=True)
     our_mem = fused_step_memory(torch, w)
     res["pytorch_attention_same_gpu"] = {
@@ -328,38 +390,33 @@ def main():
     else:
         res["cpu_baseline"] = None
 
-    if a.all:
-        cfgs = [
-            ("BERT varlen p=0.1 fp16", dict(B=8, H=12, D=64, N=512, dtype=torch.float16, p=0.1,
-                                            lens=torch.randint(256, 513, (8,), generator=torch.Generator().manual_seed(0)).tolist())),
-            # the configuration of the reference's own script (benchmarks/benchmark_flash_attention.py:39-70)
-            ("reference script B64 H16 p=0.1", dict(B=64, H=16, D=64, N=1024, dtype=torch.float16, p=0.1,
-                                                    lens=torch.randint(1004, 1024, (64,), generator=torch.Generator().manual_seed(0)).tolist())),
-            ("GPT2 causal bf16 N=1024", dict(B=8, H=12, D=64, N=1024, dtype=torch.bfloat16, causal=True)),
-            ("GPT2 causal bf16 N=2048", dict(B=8, H=12, D=64, N=2048, dtype=torch.bfloat16, causal=True)),
-            ("GPT2 causal bf16 N=4096", dict(B=8, H=12, D=64, N=4096, dtype=torch.bfloat16, causal=True)),
-            ("  + ALiBi slopes, N=2048", dict(B=8, H=12, D=64, N=2048, dtype=torch.bfloat16, causal=True, alibi=True)),
-            ("d128 fp16 N=2048", dict(B=16, H=12, D=128, N=2048, dtype=torch.float16)),
-            ("d128 fp16 N=2048 causal", dict(B=16, H=12, D=128, N=2048, dtype=torch.float16, causal=True)),
-            ("blocksparse 25% 16x256", dict(B=4, H=16, D=64, N=4096, dtype=torch.float16, blockmask=sparse_layout(torch, 4096))),
-            ("blocksparse 25% 256x256", dict(B=4, H=16, D=64, N=4096, dtype=torch.float16,
-                                             blockmask=sparse_layout(torch, 4096, rows_per_draw=16))),
-        ]
-        print("%-31s %9s %9s %9s %9s %8s %10s %11s %8s" % ("config", "fwd ms", "bwd ms", "fwd TF", "f+b TF", "% peak", "f+b GB/s",
-                                                          "PyTorch ms", "speedup"), file=sys.stderr)
-        for name, kw in cfgs:
+    if not a.no_configs or a.all:
+        if a.all:
+            print("%-31s %9s %9s %9s %9s %8s %10s %11s %8s" % ("config", "fwd ms", "bwd ms", "fwd TF", "f+b TF", "% peak", "f+b GB/s",
+                                                              "PyTorch ms", "speedup"), file=sys.stderr)
+        res["configs"] = []
+        for name, kw in config_list(torch):
             wl = Workload(torch, **kw)
             tt = time_steps(torch, be, wl, max(10, a.steps // 2), 5, a.settle)
             fb = 3.5 * wl.fwd_flops / ((tt["fwd_ms"] + tt["bwd_ms"]) * 1e-3) / 1e12
             gbs = (wl.bytes_fwd + wl.bytes_bwd) / ((tt["fwd_ms"] + tt["bwd_ms"]) * 1e-3) / 1e9
-            # PyTorch standard attention on the same GPU (no counterpart for a block layout)
-            pt = torch_attention_ms(torch, wl, 4) if wl.blockmask is None else None
-            print("%-31s %9.4f %9.4f %9.1f %9.1f %8.2f %10.1f %11s %8s" % (
-                name, tt["fwd_ms"], tt["bwd_ms"], wl.fwd_flops / (tt["fwd_ms"] * 1e-3) / 1e12, fb,
-                100 * fb / MFMA_PEAK_TFLOPS, gbs, "%.3f" % pt if pt else "-",
-                "%.1fx" % (pt / (tt["fwd_ms"] + tt["bwd_ms"])) if pt else "-"), file=sys.stderr)
+            row = {"config": name.strip(), "fwd_ms": round(tt["fwd_ms"], 4), "bwd_ms": round(tt["bwd_ms"], 4),
+                   "fwd_tflops": round(wl.fwd_flops / (tt["fwd_ms"] * 1e-3) / 1e12, 1), "fwd_bwd_tflops": round(fb, 1),
+                   "pct_of_mfma_peak": round(100 * fb / MFMA_PEAK_TFLOPS, 2), "hbm_gbs": round(gbs, 1),
+                   "pct_of_hbm_peak": round(100 * gbs / HBM_PEAK_GBS, 2)}
+            if a.all:
+                # PyTorch standard attention on the same GPU (no counterpart for a block layout)
+                pt = torch_attention_ms(torch, wl, 4) if wl.blockmask is None else None
+                if pt:
+                    row["pytorch_ms"] = round(pt, 3)
+                print("%-31s %9.4f %9.4f %9.1f %9.1f %8.2f %10.1f %11s %8s" % (
+                    name, tt["fwd_ms"], tt["bwd_ms"], wl.fwd_flops / (tt["fwd_ms"] * 1e-3) / 1e12, fb,
+                    100 * fb / MFMA_PEAK_TFLOPS, gbs, "%.3f" % pt if pt else "-",
+                    "%.1fx" % (pt / (tt["fwd_ms"] + tt["bwd_ms"])) if pt else "-"), file=sys.stderr)
+            res["configs"].append(row)
             del wl
             torch.cuda.empty_cache()
+    if a.all:
         # unpad / pad (row gather and scatter, HBM-bound): BERT-large-like padded batch, 75 % of the tokens valid
         from flash_attn.bert_padding import unpad_input
         Bp, Sp, dim = 64, 512, 1024

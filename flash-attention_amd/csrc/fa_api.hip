@@ -253,7 +253,7 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
   return FA_OK;
 }
 
-int bwd_impl(const fa_bwd_args* a, bool want_block) {
+int bwd_impl(const fa_bwd_args* a, bool want_block, void* ev_main_start = nullptr, void* ev_main_stop = nullptr) {
   if (!a) return fail(FA_ERR_INVALID_ARGUMENT, "args is NULL");
   int rc = check_common(a->struct_bytes, sizeof(fa_bwd_args), a->dtype, a->batch, a->nheads, a->head_dim, a->total_q,
                         a->total_k, a->max_seqlen_q, a->max_seqlen_k, a->p_dropout, a->softmax_scale);
@@ -337,9 +337,9 @@ int bwd_impl(const fa_bwd_args* a, bool want_block) {
   }
   FA_LAUNCH(fa::launch_bwd(p, 0, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));  // dQ, softmax_d
   if (split) FA_LAUNCH(fa::launch_dq_combine(p, a->dtype, a->head_dim, stream));
-  if (a->ev_main_start) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(a->ev_main_start), stream));
+  if (ev_main_start) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(ev_main_start), stream));
   FA_LAUNCH(fa::launch_bwd(p, 1, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));  // dK, dV
-  if (a->ev_main_stop) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(a->ev_main_stop), stream));
+  if (ev_main_stop) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(ev_main_stop), stream));
   return FA_OK;
 }
 
@@ -390,6 +390,9 @@ int fa_fwd_block_noalloc(const fa_fwd_args* args) {
 int fa_fwd(const fa_fwd_args* args) { return fwd_impl(args, false); }
 int fa_fwd_block(const fa_fwd_args* args) { return fwd_impl(args, true); }
 int fa_bwd(const fa_bwd_args* args) { return bwd_impl(args, false); }
+int fa_bwd_profiled(const fa_bwd_args* args, void* ev_main_start, void* ev_main_stop) {
+  return bwd_impl(args, false, ev_main_start, ev_main_stop);
+}
 int fa_bwd_block(const fa_bwd_args* args) { return bwd_impl(args, true); }
 
 size_t fa_fwd_workspace_bytes(const fa_fwd_args* a) {

@@ -20,7 +20,7 @@ LIB_NAME = "libflash_attn_gfx950.so"
 LIB_PATH = os.path.join(_HERE, LIB_NAME)
 
 FA_FP16, FA_BF16 = 0, 1
-FA_ABI_VERSION = 1
+FA_ABI_VERSION = 2
 
 _c_i32p = ctypes.c_void_p
 
@@ -73,7 +73,6 @@ class BwdArgs(ctypes.Structure):
         ("philox_seed", ctypes.c_uint64), ("philox_offset", ctypes.c_uint64),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("stream", ctypes.c_void_p),
-        ("ev_main_start", ctypes.c_void_p), ("ev_main_stop", ctypes.c_void_p),
         ("alibi_slopes", ctypes.c_void_p),
     ]
 
@@ -93,7 +92,7 @@ class RotaryArgs(ctypes.Structure):
 
 
 EXPORTED_SYMBOLS = (
-    "fa_fwd", "fa_bwd", "fa_fwd_block", "fa_bwd_block", "fa_fwd_block_noalloc", "fa_fwd_workspace_bytes", "fa_bwd_workspace_bytes",
+    "fa_fwd", "fa_bwd", "fa_bwd_profiled", "fa_fwd_block", "fa_bwd_block", "fa_fwd_block_noalloc", "fa_fwd_workspace_bytes", "fa_bwd_workspace_bytes",
     "fa_round_seqlens", "fa_philox_offset_increment", "fa_last_error", "fa_abi_version",
     "fa_gather_rows", "fa_scatter_rows", "fa_scatter_rows_workspace_bytes", "fa_rotary", "fa_set_launch_policy",
 )
@@ -123,6 +122,8 @@ def load_library():
             fn = getattr(lib, name)
             fn.argtypes = [ctypes.POINTER(BwdArgs)]
             fn.restype = ctypes.c_int
+        lib.fa_bwd_profiled.argtypes = [ctypes.POINTER(BwdArgs), ctypes.c_void_p, ctypes.c_void_p]
+        lib.fa_bwd_profiled.restype = ctypes.c_int
         lib.fa_fwd_workspace_bytes.argtypes = [ctypes.POINTER(FwdArgs)]
         lib.fa_fwd_workspace_bytes.restype = ctypes.c_size_t
         lib.fa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdArgs)]
@@ -373,14 +374,14 @@ def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seql
         a.workspace = ws.data_ptr() if ws is not None else None
         a.workspace_bytes = ws_bytes
         a.stream = _stream_handle(dev)
-        if main_kernel_events is not None:  # (start, stop) torch.cuda.Event created with enable_timing=True
+        a.alibi_slopes = _check_alibi(alibi_slopes, nheads, dev, sparse)
+        if main_kernel_events is not None and not sparse:  # (start, stop) torch.cuda.Event created with enable_timing=True
             for ev in main_kernel_events:
                 if not ev.cuda_event:  # torch creates the HIP event lazily, on first record
                     ev.record()
-            a.ev_main_start = main_kernel_events[0].cuda_event
-            a.ev_main_stop = main_kernel_events[1].cuda_event
-        a.alibi_slopes = _check_alibi(alibi_slopes, nheads, dev, sparse)
-        rc = (lib.fa_bwd_block if sparse else lib.fa_bwd)(ctypes.byref(a))
+            rc = lib.fa_bwd_profiled(ctypes.byref(a), main_kernel_events[0].cuda_event, main_kernel_events[1].cuda_event)
+        else:
+            rc = (lib.fa_bwd_block if sparse else lib.fa_bwd)(ctypes.byref(a))
         if rc != 0:
             _raise(rc, lib)
     return [dq, dk, dv, softmax_d]

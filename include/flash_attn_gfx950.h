@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FA_ABI_VERSION 1
+#define FA_ABI_VERSION 2
 
 enum fa_dtype { FA_FP16 = 0, FA_BF16 = 1 };
 
@@ -116,10 +116,6 @@ typedef struct fa_bwd_args {
   void* workspace;
   size_t workspace_bytes;
   void* stream;
-  /* Optional profiling hooks (hipEvent_t or NULL): recorded on `stream` immediately before and after the dK/dV
-   * kernel, the longer of the two kernels of a backward call (dQ + softmax_d kernel, dK/dV kernel). */
-  void* ev_main_start;
-  void* ev_main_stop;
   const float* alibi_slopes; /* as in fa_fwd_args: the slopes the forward was given */
 } fa_bwd_args;
 
@@ -127,6 +123,10 @@ typedef struct fa_bwd_args {
 int fa_fwd(const fa_fwd_args* args);
 /* replaces flash_attn_cuda.bwd -> mha_bwd, csrc/flash_attn/fmha_api.cpp:302-449 */
 int fa_bwd(const fa_bwd_args* args);
+/* fa_bwd with two timing events (hipEvent_t, either may be NULL) recorded on args->stream immediately before and after the
+ * dK/dV kernel, the longer of the backward's two kernels (dQ + softmax_d kernel first, then dK/dV).  No counterpart in
+ * the reference; for benchmarks that price that kernel against its roofline.  Results are those of fa_bwd. */
+int fa_bwd_profiled(const fa_bwd_args* args, void* ev_main_start, void* ev_main_stop);
 /* replaces flash_attn_cuda.fwd_block -> mha_fwd_block, csrc/flash_attn/fmha_api.cpp:451-573
  * (args->blockmask must be non-NULL).  is_causal may be set together with a blockmask, here and in fa_bwd_block: a score
  * counts iff its block is listed AND key <= query; blocks that lie wholly above the diagonal may be listed or not.  The

@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol(lib):
     assert declared == set(be.EXPORTED_SYMBOLS)
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.fa_abi_version() == 1
+    assert lib.fa_abi_version() == be.FA_ABI_VERSION == 2
 
 
 def test_struct_layout_matches_library(lib):
