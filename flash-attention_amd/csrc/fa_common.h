@@ -98,6 +98,7 @@ FA_DEVICE float sum8_acc(bf16x8 v, float acc) {
 
 // Threshold (log2 units) of the forward kernel's lazy accumulator rescale.
 constexpr float kRescaleLog2 = 8.f;
+constexpr float kRescaleLimit = 256.f;  // 2^kRescaleLog2
 
 // A wave-uniform 64-bit value moved to scalar registers (the compiler cannot always prove uniformity of a load)
 FA_DEVICE uint64_t uniform64(uint64_t x) {

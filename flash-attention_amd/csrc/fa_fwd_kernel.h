@@ -48,7 +48,7 @@ struct FwdCfg {
 // kAlibi: the score of (query i, key j) gets -slope[head] * |i - j| added after scaling.  The scores are then moved to the
 // softmax's own units (base-2 exponent) before the row maximum is taken, and the running maximum is kept in those units.
 template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, bool kAlibi = false, int KS = 1>
-__global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2) fa_fwd_kernel(const FwdParams p) {
+__global__ void __launch_bounds__(256, (!kDropout && !kAlibi && D <= 64) ? 4 : 2) fa_fwd_kernel(const FwdParams p) {
   using Cfg = FwdCfg<T, D, BN, KS>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
@@ -180,61 +180,108 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
     }
 
     if (wave_work) {
-      // ---- S^T = K Q^T
       // this wave's 32-key blocks of the tile: kb0, kb0 + 1, ... (all of them without a key split)
       const int kb0 = kh * KBW;
       f32x16 s[KBW];
+      // ---- S^T = K Q^T, dead scores set to -inf, bias added
+      auto scores = [&]() {
 #pragma unroll
-      for (int kb = 0; kb < KBW; kb++) {
+        for (int kb = 0; kb < KBW; kb++) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) s[kb][r] = 0.f;
+          for (int r = 0; r < 16; r++) s[kb][r] = 0.f;
 #pragma unroll
-        for (int ks = 0; ks < D / 16; ks++) {
-          vec8 a = *reinterpret_cast<const vec8*>(Ks + (kb0 + kb) * 32 * D + koff[ks]);
-          s[kb] = E::mfma32(a, qreg[ks], s[kb]);
+          for (int ks = 0; ks < D / 16; ks++) {
+            vec8 a = *reinterpret_cast<const vec8*>(Ks + (kb0 + kb) * 32 * D + koff[ks]);
+            s[kb] = E::mfma32(a, qreg[ks], s[kb]);
+          }
         }
-      }
-      // ---- mask (only tiles that straddle the key length, the diagonal, or an inactive row block)
-      // (an inactive row block inside an active tile is not masked score by score: its lanes' maximum is dropped and their
-      // exponentials are taken against +inf below, which costs three instructions instead of two per score)
-      const bool need_mask = (n0 + BN > Lk) || (kCausal && (n0 + BN - 1 > mw));
-      if (need_mask) {
+        // mask: only tiles that straddle the key length or the diagonal.  (An inactive row block inside an active tile is
+        // not masked score by score: its lanes' exponentials are taken against +inf below.)
+        const bool need_mask = (n0 + BN > Lk) || (kCausal && (n0 + BN - 1 > mw));
+        if (need_mask) {
+#pragma unroll
+          for (int kb = 0; kb < KBW; kb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+              const int key = n0 + (kb0 + kb) * 32 + (r >> 2) * 8 + hf * 4 + (r & 3);
+              bool dead = key >= Lk;
+              if (kCausal) dead = dead || key > qrow;
+              if (dead) s[kb][r] = -INFINITY;
+            }
+        }
+        if (kAlibi) {  // s <- s * scale * log2(e) - slope2 * |key - query|; dead scores stay -inf
+#pragma unroll
+          for (int kb = 0; kb < KBW; kb++) {
+            const float dbase = (float)(n0 + (kb0 + kb) * 32 + hf * 4 - qrow);  // key - query of register 0
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+              const float cr = (float)((r >> 2) * 8 + (r & 3));
+              // under a causal mask every live score has key <= query: -|key - query| = key - query, linear in cr
+              const float bias = kCausal ? __builtin_fmaf(cr, sl2, sl2 * dbase) : -sl2 * __builtin_fabsf(dbase + cr);
+              s[kb][r] = __builtin_fmaf(s[kb][r], cs, bias);
+            }
+          }
+        }
+      };
+      // ---- P = exp2(scores - reference point m_i), rounded to the tensor dtype (what the P V product consumes); lt = this
+      // lane's share of the tile's row sums: of the rounded values, or with dropout of P before the mask, in fp32 as the
+      // reference has it (fmha_fprop_kernel_1xN.h:454 vs :471)
+      vec8 pb[KBW][2];
+      float lt;
+      auto probabilities = [&]() {
+        float mc = ((m_i == -INFINITY) ? 0.f : m_i) * cse;
+        if (kSparse && !row_on) mc = INFINITY;  // this lane's row block does not attend the tile: P = exp2(x - inf) = 0
+        lt = 0.f;
 #pragma unroll
         for (int kb = 0; kb < KBW; kb++)
 #pragma unroll
           for (int r = 0; r < 16; r++) {
-            const int key = n0 + (kb0 + kb) * 32 + (r >> 2) * 8 + hf * 4 + (r & 3);
-            bool dead = key >= Lk;
-            if (kCausal) dead = dead || key > qrow;
-            if (dead) s[kb][r] = -INFINITY;
+            const float pe = fast_exp2(kAlibi ? s[kb][r] - mc : __builtin_fmaf(s[kb][r], cs, -mc));
+            s[kb][r] = pe;
+            if (kDropout) lt += pe;
           }
-      }
-      if (kAlibi) {  // s <- s * scale * log2(e) - slope2 * |key - query|; dead scores stay -inf
+        if (kDropout) {
 #pragma unroll
-        for (int kb = 0; kb < KBW; kb++) {
-          const float dbase = (float)(n0 + (kb0 + kb) * 32 + hf * 4 - qrow);  // key - query of register 0
+          for (int kb = 0; kb < KBW; kb++) {
+            const KeepFields keep = keep_fields_row_layout(p.pk, (uint32_t)bh, qrow, n0 + (kb0 + kb) * 32, hf);
 #pragma unroll
-          for (int r = 0; r < 16; r++) {
-            const float cr = (float)((r >> 2) * 8 + (r & 3));
-            // under a causal mask every live score has key <= query: -|key - query| = key - query, linear in cr
-            const float bias = kCausal ? __builtin_fmaf(cr, sl2, sl2 * dbase) : -sl2 * __builtin_fabsf(dbase + cr);
-            s[kb][r] = __builtin_fmaf(s[kb][r], cs, bias);
+            for (int r = 0; r < 16; r++)
+              if (!keep.keep_row(r, p.keep_thr)) s[kb][r] = 0.f;
           }
         }
+#pragma unroll
+        for (int kb = 0; kb < KBW; kb++)
+#pragma unroll
+          for (int t = 0; t < 2; t++) {
+            f32x8 pf;
+#pragma unroll
+            for (int i = 0; i < 8; i++) pf[i] = s[kb][8 * t + i];
+            pb[kb][t] = cvt8<T>(pf);
+            if (!kDropout) lt = sum8_acc(pb[kb][t], lt);
+          }
+      };
+      // ---- online softmax (fmha_fprop_kernel_1xN.h:408-454,560-611 restated for a register-resident row).
+      // The reference point m_i of the exponentials only moves when it has to: P may exceed 1 by a factor of up to
+      // 2^kRescaleLog2, which the fp32 accumulators and the fp16/bf16 rounding of P absorb (numerator and denominator carry
+      // the same factor, so the result is unchanged).  Whether it has to move is read off the tile's row sums - if a lane's
+      // share is at most 2^kRescaleLog2, so is every P behind it - so the common tile takes no row maximum at all.  A tile
+      // that fails the test (the first of a row always does: no reference point yet) is redone the long way: scores again,
+      // row maxima, rescaled accumulators, probabilities against the new reference point.
+      scores();
+      bool redo = __any(m_i == -INFINITY && (!kSparse || row_on));
+      if (!redo) {
+        probabilities();
+        redo = __any(!(lt <= kRescaleLimit));  // also catches inf and NaN
+        if (__builtin_expect(redo, 0)) scores();
       }
-      // ---- online softmax (fmha_fprop_kernel_1xN.h:408-454,560-611 restated for a register-resident row)
-      float mt = s[0][0];
+      if (__builtin_expect(redo, 0)) {
+        float mt = s[0][0];
 #pragma unroll
-      for (int kb = 0; kb < KBW; kb++)
+        for (int kb = 0; kb < KBW; kb++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) mt = fmaxf(mt, s[kb][r]);
-      mt = half_max(mt);
-      if (kSparse && !row_on) mt = -INFINITY;  // this lane's row block does not attend the tile
-      // The reference point m_i of the exponentials only moves when some row's maximum has grown by more than
-      // 2^kRescaleLog2 since it was set; until then P may exceed 1 by at most that factor, which the fp32 accumulators and
-      // the fp16/bf16 rounding of P absorb, and the accumulators need no rescaling (numerator and denominator carry the
-      // same factor, so the result is unchanged).
-      if (__builtin_expect(__any((mt - m_i) * cse > kRescaleLog2), 0)) {  // wave-uniform; true on the first tile
+          for (int r = 0; r < 16; r++) mt = fmaxf(mt, s[kb][r]);
+        mt = half_max(mt);
+        if (kSparse && !row_on) mt = -INFINITY;
         const float m_new = fmaxf(m_i, mt);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
         const float alpha = fast_exp2(m_i * cse - m_use * cse);
@@ -242,47 +289,22 @@ __global__ void __launch_bounds__(256, (kSparse && !kDropout && D <= 64) ? 4 : 2
         l_i *= alpha;
 #pragma unroll
         for (int i = 0; i < DV / 32; i++) o_acc[i] = o_acc[i] * alpha;
+        probabilities();
       }
-      float mc = ((m_i == -INFINITY) ? 0.f : m_i) * cse;
-      if (kSparse && !row_on) mc = INFINITY;  // P = exp2(finite - inf) = 0
-      float rsum = 0.f;
-#pragma unroll
-      for (int kb = 0; kb < KBW; kb++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const float pe = fast_exp2(kAlibi ? s[kb][r] - mc : __builtin_fmaf(s[kb][r], cs, -mc));
-          s[kb][r] = pe;
-          if (kDropout) rsum += pe;
-        }
-      if (kDropout) l_i += rsum;  // the sum uses P before dropout (fmha_fprop_kernel_1xN.h:454 vs :471)
-
-      if (kDropout) {
-#pragma unroll
-        for (int kb = 0; kb < KBW; kb++) {
-          const KeepFields keep = keep_fields_row_layout(p.pk, (uint32_t)bh, qrow, n0 + (kb0 + kb) * 32, hf);
-#pragma unroll
-          for (int r = 0; r < 16; r++)
-            if (!keep.keep_row(r, p.keep_thr)) s[kb][r] = 0.f;
-        }
-      }
+      l_i += lt;
 
       // ---- O^T += V^T P^T
 #pragma unroll
       for (int kb = 0; kb < KBW; kb++) {
 #pragma unroll
         for (int t = 0; t < 2; t++) {
-          f32x8 pf;
-#pragma unroll
-          for (int i = 0; i < 8; i++) pf[i] = s[kb][8 * t + i];
-          const vec8 pb = cvt8<T>(pf);
-          if (!kDropout) l_i = sum8_acc(pb, l_i);
 #pragma unroll
           for (int db = 0; db < DV / 32; db++) {
             const T* vp = Vs + ((kb0 + kb) * 32 + 16 * t) * D + voff[db];
             u32x2 lo = lds_read_tr16(vp);
             u32x2 hi = lds_read_tr16(vp + 8 * D);
             u32x4 av = {lo[0], lo[1], hi[0], hi[1]};
-            o_acc[db] = E::mfma32(bitcast<vec8>(av), pb, o_acc[db]);
+            o_acc[db] = E::mfma32(bitcast<vec8>(av), pb[kb][t], o_acc[db]);
           }
         }
       }
