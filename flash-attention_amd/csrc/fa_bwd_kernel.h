@@ -476,7 +476,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
   }
   // For d <= 64 the dP^T accumulator starts from -Dk of this lane's query row (16 registers that save 16 subtractions
   // per 32x32 tile); at d = 128 those registers would push the kernel below two waves per SIMD.
-  constexpr bool kInitNegD = D <= 64;
+  constexpr bool kInitNegD = D <= 64 || !kDropout;
   f32x16 negd;
 #pragma unroll
   for (int r = 0; r < 16; r++) negd[r] = kInitNegD ? -dkv : 0.f;
