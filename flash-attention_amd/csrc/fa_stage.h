@@ -13,7 +13,7 @@
 //   transposed     (ds_read_b64_tr_b16, MFMA A operand of X^T P): 16 lanes read an aligned chunk pair of 4
 //                  consecutive rows;
 //   both.
-// kSwzRow, kSwzTr and kSwzDual are conflict-free for these respectively.  kSwzTr has period 8 rows, the other two
+// kSwzRow, kSwzTr and kSwzDual are conflict-free for these respectively.  kSwzTr has period 2 to 8 rows, the other two
 // period 16 rows.
 #pragma once
 
@@ -29,7 +29,15 @@ FA_DEVICE int tile_swz(int r) {
   constexpr int RPB = CH >= 16 ? 1 : 16 / CH;  // tile rows per 256-byte LDS line
   const int u = (r / RPB) % CH;
   if (KIND == kSwzRow) return u;
-  if (KIND == kSwzTr) return CH >= 4 ? 2 * (u % (CH / 2)) : 0;
+  if (KIND == kSwzTr) {
+    // A transposed read touches 4 consecutive rows, and the two 16-lane groups that the LDS serves together 64 bytes
+    // (4 chunks) of each: the 4 rows must land in 4 distinct 64-byte bank groups of the 256-byte line.  128-element rows
+    // (one per line): chunk ^= 4 * (r % 4); 64-element rows (two per line, the odd row in the upper half anyway): rows r and
+    // r + 2 must differ, chunk ^= 4 * ((r / 2) % 2).  Both have period <= 4 rows, so rows r + 8 and r + 16 keep r's value.
+    if (CH == 16) return 4 * (r % 4);
+    if (CH == 8) return 4 * ((r >> 1) & 1);
+    return CH >= 4 ? 2 * (u % (CH / 2)) : 0;
+  }
   // dual: a bijection of u (row fragments) whose values for the 4 rows of a transposed read fall in distinct pairs
   if (CH == 16) return ((u & 3) << 2) | (u >> 2);
   if (CH == 8) return ((u & 1) << 2) | (u >> 1);
