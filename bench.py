@@ -75,6 +75,16 @@ class Workload:
             self.blockmask = convert_blockmask(blockmask.cuda(), causal=False)  # the entry points' own column-major form
         self.bytes_fwd = 4 * total * H * D * 2 + 4 * B * H * self.max_s          # q,k,v read + o written, lse
         self.bytes_bwd = 8 * total * H * D * 2 + 2 * 4 * B * H * self.max_s      # q,k,v,o,do read + dq,dk,dv written
+        # dropout (dense): the forward leaves its keep decisions, one bit per score, for the backward's two kernels, as
+        # the autograd functions do (flash_attn_interface.py); the buffer is made once, like the tensors
+        self.keep_words = None
+        if p > 0 and blockmask is None:
+            from flash_attn import flash_attn_gfx950 as be
+            self.keep_words = be.new_keep_words(self.q, self.cu, self.max_s, self.max_s, p)
+            if self.keep_words is not None:
+                bits = sum(H * L * L for L in lens) / 8
+                self.bytes_fwd += bits
+                self.bytes_bwd += 2 * bits
 
     def forward(self, be):
         q, k, v = self.q, self.k, self.v
@@ -83,7 +93,7 @@ class Workload:
                                               self.scale, self.causal, False, None)
             return
         self.out, self.lse = be.fwd(q, k, v, self.cu, self.cu, self.max_s, self.max_s, self.p, self.scale, False,
-                                    self.causal, False, None, self.alibi)
+                                    self.causal, False, None, self.alibi, self.keep_words)
 
     def backward(self, be, events=None):
         q, k, v = self.q, self.k, self.v
@@ -97,7 +107,8 @@ class Workload:
                 events[1].record()  # whole backward: the sparse entry point has no per-kernel hook
             return
         be.bwd(self.dout, q, k, v, self.out, self.lse, dq, dk, dv, self.cu, self.cu, self.max_s, self.max_s, self.p,
-               self.scale, False, self.causal, None, main_kernel_events=events, alibi_slopes=self.alibi)
+               self.scale, False, self.causal, None, main_kernel_events=events, alibi_slopes=self.alibi,
+               keep_words=self.keep_words)
 
 
 def time_steps(torch, be, w, steps, warmup, settle_s=0.2):

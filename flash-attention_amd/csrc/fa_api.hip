@@ -223,6 +223,15 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
   p.keep_thr = (uint32_t)std::floor(p_keep * 65535.0);  // fmha_api.cpp:110
   p.pk = make_key(a->philox_seed, a->philox_offset);
   p.alibi = a->alibi_slopes;
+  if (a->keep_words && dropout && !sparse) {
+    FA_REQUIRE(aligned16(a->keep_words), "keep_words must be 16-byte aligned");
+    const size_t kw_need = fa_keep_words_bytes(a->batch, a->nheads, a->max_seqlen_q, a->max_seqlen_k);
+    if (a->keep_words_bytes < kw_need)
+      return fail(FA_ERR_WORKSPACE, "keep_words of %zu bytes needed, %zu given", kw_need, a->keep_words_bytes);
+    p.keep_words = reinterpret_cast<uint32_t*>(a->keep_words);
+    p.kw_q = (int)fa::keep_words_q_extent(a->max_seqlen_q);
+    p.kw_kb = (int)fa::keep_words_key_blocks(a->max_seqlen_k);
+  }
   // short query side, long key side: split the keys over several workgroups if the caller brought the scratch for it
   const SplitPlan sp = split_plan(a->batch, a->nheads, a->head_dim, a->total_q, a->max_seqlen_q, a->max_seqlen_k, r.sq_r,
                                   a->is_causal != 0, sparse);
@@ -326,6 +335,15 @@ int bwd_impl(const fa_bwd_args* a, bool want_block, void* ev_main_start = nullpt
   p.keep_thr = (uint32_t)std::floor(p_keep * 65535.0);
   p.pk = make_key(a->philox_seed, a->philox_offset);
   p.alibi = a->alibi_slopes;
+  if (a->keep_words && dropout && !sparse) {
+    FA_REQUIRE(aligned16(a->keep_words), "keep_words must be 16-byte aligned");
+    const size_t kw_need = fa_keep_words_bytes(a->batch, a->nheads, a->max_seqlen_q, a->max_seqlen_k);
+    if (a->keep_words_bytes < kw_need)
+      return fail(FA_ERR_WORKSPACE, "keep_words of %zu bytes needed, %zu given", kw_need, a->keep_words_bytes);
+    p.keep_words = reinterpret_cast<const uint32_t*>(a->keep_words);
+    p.kw_q = (int)fa::keep_words_q_extent(a->max_seqlen_q);
+    p.kw_kb = (int)fa::keep_words_key_blocks(a->max_seqlen_k);
+  }
 
   // short query side, long key side: the dQ kernel would walk all keys with one workgroup per (batch, head)
   const SplitPlan sp = split_plan(a->batch, a->nheads, a->head_dim, a->total_q, a->max_seqlen_q, a->max_seqlen_k, r.sq_r,
@@ -410,6 +428,11 @@ size_t fa_bwd_workspace_bytes(const fa_bwd_args* a) {
   const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, false);
   return split_plan(a->batch, a->nheads, a->head_dim, a->total_q, a->max_seqlen_q, a->max_seqlen_k, r.sq_r,
                     a->is_causal != 0, false).o_bytes;
+}
+
+size_t fa_keep_words_bytes(int32_t batch, int32_t nheads, int32_t max_seqlen_q, int32_t max_seqlen_k) {
+  if (batch <= 0 || nheads <= 0 || max_seqlen_q <= 0 || max_seqlen_k <= 0) return 0;
+  return (size_t)batch * nheads * fa::keep_words_key_blocks(max_seqlen_k) * fa::keep_words_q_extent(max_seqlen_q) * 4;
 }
 
 void fa_round_seqlens(int32_t head_dim, int32_t max_seqlen_q, int32_t max_seqlen_k, int32_t blocksparse,

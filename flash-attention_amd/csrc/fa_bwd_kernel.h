@@ -62,8 +62,12 @@ struct BwdCfg {
   static constexpr int kMinBlocks = (D == 128 && kDropout) ? 1 : 2;
 };
 
-template <typename T, int D, bool kCausal, bool kDropout, bool kSparse, bool kAlibi = false>
-__global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D, kDropout>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
+// kDrop: 0 = no dropout; 1 = the keep decisions are drawn here (Philox); 2 = they are read from the keep words the dQ
+// kernel left (fa_common.h; dense only): the kernel then has the shape and the registers of the one without dropout.
+template <typename T, int D, bool kCausal, int kDrop, bool kSparse, bool kAlibi = false>
+__global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64) ? 3 : (BwdCfg<T, D, kDrop == 1>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
+  constexpr bool kDropout = kDrop == 1, kStored = kDrop == 2;
+  static_assert(!(kStored && kSparse), "keep words: dense only");
   using Cfg = BwdCfg<T, D, kDropout>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
@@ -139,6 +143,12 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
   // converted when the tile is consumed: arithmetic on a loaded value at this point would make the wave wait for the
   // load - and, memory operations completing in order, for everything issued before it - right away.
   float statpre = 0.f;
+  // kStored: the keep words of a tile's rows and this wave's 32 keys - one per lane, in the order the masks are needed
+  // (fa_common.h) - are fetched with the tile and handed out to the scalar registers by v_readlane, slab by slab.  (Read
+  // straight into scalar registers, 128 bytes a slab, they arrive too late: nothing hides a scalar cache miss here.)
+  uint32_t kwpre = 0;
+  const uint32_t* const kw_wave =
+      kStored ? p.keep_words + ((int64_t)bh * p.kw_kb + (n0 >> 5) + wave) * p.kw_q : nullptr;
   auto stage = [&](int mt, int buf) {
     const int m0 = mt * BM;
     if (tid < BM) {
@@ -150,6 +160,7 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
       statpre = 0.f;
       if (row < Lq) statpre = dsbase[row];
     }
+    if (kStored && (BM == 64 || lane < BM)) kwpre = kw_wave[m0 + lane];
     stager.issue(lds_raw + buf * kBufBytes, m0, Lq);
   };
   // lse scaled to base 2, +inf (row off) where the row saw no key; Dk negated: the dP accumulator starts from -Dk
@@ -237,6 +248,7 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
     float* const lse_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffStat + buf * Cfg::kStatBytes);
     float* const dk_l = lse_l + BM;
     if (tid < 2 * BM) lse_l[tid] = stat_value();
+    const uint32_t kwcur = kwpre;
     __syncthreads();  // the tile is complete, and nobody still reads the other buffer
     if (kSparse) {
       more = next_tile(tn);
@@ -300,6 +312,10 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
         const int mb = 2 * (key & 3) + hf;
         keep = keep_fields_col_layout_q4(p.pk, (uint32_t)bh, (uint32_t)((mb < 4 ? q_lo : q_hi) >> 2) + (mb & 3), key);
       }
+      // -Dk is read a second time where a dropped element needs it; the opaque zero keeps the compiler from holding
+      // the 16 values it read for the accumulator's start in registers until then instead
+      int again = 0;
+      if (kStored) asm volatile("" : "+s"(again));
       if (kCausal && diag) {  // only slabs that straddle the diagonal: scores above it become -inf (P = 0)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
@@ -308,12 +324,21 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
           if (key > qrow) s[r] = -INFINITY;
         }
       }
+      uint64_t km[16];  // kStored: the keep mask of register r over the wave's 64 lanes
+      if (kStored) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)kwcur, (qb * 32 + 2 * r) & 63);
+          const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)kwcur, (qb * 32 + 2 * r + 1) & 63);
+          km[r] = ((uint64_t)hi << 32) | lo;
+        }
+      }
       const float dbase = (float)(key - m0 - qb * 32 - 4 * hf);  // key - query of register 0 (kAlibi; dense only)
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_l + qb * 32 + 8 * j + 4 * hf);
         f32x4 nd4 = {0.f, 0.f, 0.f, 0.f};
-        if (kDropout) nd4 = *reinterpret_cast<const f32x4*>(dk_l + qb * 32 + 8 * j + 4 * hf);
+        if (kDrop != 0) nd4 = *reinterpret_cast<const f32x4*>(dk_l + again + qb * 32 + 8 * j + 4 * hf);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           const int r = 4 * j + i;
@@ -323,6 +348,7 @@ __global__ void __launch_bounds__(256, (!kDropout && D <= 64) ? 3 : (BwdCfg<T, D
           float dpe = dp[r];  // dP - Dk
           float pm = pe;
           if (kDropout && !keep.keep_col(r, p.keep_thr)) { dpe = nd4[i]; pm = 0.f; }  // dropped: M o dP = 0
+          if (kStored && !lane_bit(km[r])) { dpe = nd4[i]; pm = 0.f; }
           s[r] = pm;          // P o M, feeds dV
           dp[r] = pe * dpe;   // dS' = P o (M o dP - Dk), feeds dK
         }
@@ -413,8 +439,11 @@ struct DqCfg {
   static constexpr int CH = D / 8;
 };
 
-template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, bool kAlibi = false, int KS = 1>
-__global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq_kernel(const BwdParams p) {
+// kDrop: as in fa_bwd_dkdv_kernel
+template <typename T, int D, int BN, bool kCausal, int kDrop, bool kSparse, bool kAlibi = false, int KS = 1>
+__global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0) ? 3 : 2) fa_bwd_dq_kernel(const BwdParams p) {
+  constexpr bool kDropout = kDrop == 1, kStored = kDrop == 2;
+  static_assert(!(kStored && kSparse), "keep words: dense only");
   using Cfg = DqCfg<T, D, BN, KS>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
@@ -491,7 +520,17 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
   typename Cfg::Stager stager;
   stager.init(wave, lane, reinterpret_cast<const T*>(p.k) + (int64_t)k_begin * p.k_rs + (int64_t)h * p.k_hs, p.k_rs,
               reinterpret_cast<const T*>(p.v) + (int64_t)k_begin * p.v_rs + (int64_t)h * p.v_hs, p.v_rs);
-  auto stage = [&](int it, int buf) { stager.issue(lds_raw + buf * kBufBytes, it * BN, Lk); };
+  // kStored: the keep words of this lane's query row for the wave's 32-key blocks of a tile travel with the tile
+  uint32_t kwpre[KBW];
+  const uint32_t* const kw_row =
+      kStored ? p.keep_words + ((int64_t)bh * p.kw_kb + kh * KBW) * p.kw_q + mw + (keep_word_slot(c) & 31) : nullptr;
+  auto stage = [&](int it, int buf) {
+    if (kStored) {
+#pragma unroll
+      for (int kbi = 0; kbi < KBW; kbi++) kwpre[kbi] = kw_row[(int64_t)(it * (BN / 32) + kbi) * p.kw_q];
+    }
+    stager.issue(lds_raw + buf * kBufBytes, it * BN, Lk);
+  };
 
   // Sparse: the tile's and this lane's row block's activity bits of 64 consecutive key blocks sit in registers
   uint64_t tile_bits = 0, row_bits = 0;
@@ -552,6 +591,9 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
 #pragma unroll
     for (int i = 0; i < DV / 32; i++) asm volatile("" : "+v"(acc[i]));
     wait_vmem();      // this wave's share of tile `it` is in LDS
+    uint32_t kwcur[KBW];
+#pragma unroll
+    for (int kbi = 0; kbi < KBW; kbi++) kwcur[kbi] = kStored ? kwpre[kbi] >> (4 * hf) : 0u;  // bit 8 (r / 4) + r % 4 <-> register r
     __syncthreads();  // so is everyone else's, and nobody still reads the other buffer
     const int it_next = next_active(it + 1);
     if (it_next < ntiles) stage(it_next, buf ^ 1);
@@ -613,6 +655,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && !kDropout) ? 3 : 2) fa_bwd_dq
           const float pe = fast_exp2(__builtin_fmaf(s[r], cs, e));  // 0 for dead scores and switched-off rows
           float dpe = kInitNegD ? dp[r] : dp[r] - dkv;  // dP - Dk
           if (kDropout && !keep.keep_row(r, p.keep_thr)) dpe = -dkv;
+          if (kStored) dpe = keep_word_select(kwcur[kbi], 8 * (r >> 2) + (r & 3), dpe, -dkv);
           s[r] = pe * dpe;  // dS'
         }
 #pragma unroll

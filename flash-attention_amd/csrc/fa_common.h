@@ -272,4 +272,41 @@ FA_DEVICE KeepFields keep_fields_col_layout(const PhiloxKey& pk, uint32_t bh, in
   return keep_fields_col_layout_q4(pk, bh, ((uint32_t)q0 >> 2) + 2 * (key & 3) + hf, key);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Dropout keep words.  All three kernels decide the same keep bits.  When the caller offers a buffer (one bit per score),
+// the forward - which draws them with Philox - leaves them there and the backward's kernels read them instead of
+// drawing them again:
+// keep_words[(bh * n_key_blocks + kb) * q_extent + keep_word_slot(q)], bit j <=> the score of query q (sequence-local) and
+// key 32 kb + j is kept.
+//   * The dQ kernel (lane -> query row, like the forward) loads its row's word and tests the bits of its 16 keys.
+//   * The dK/dV kernel (lane l owns key l % 32 and, in accumulator register r, query row 8 (r / 4) + 4 (l / 32) + r % 4 of
+//     its 32) needs, for register r, a mask over its 64 lanes = the words of two rows 4 apart: keep_word_slot() makes them
+//     neighbours, the kernel fetches a tile's words one per lane and moves them to scalar registers (v_readlane), where
+//     v_cndmask takes them as they are.
+// ---------------------------------------------------------------------------------------------
+FA_DEVICE int keep_word_slot(int q) { return (q & ~31) | (q & 24) | ((q & 3) << 1) | ((q >> 2) & 1); }
+inline size_t keep_words_q_extent(int max_sq) { return (size_t)((max_sq + 127) & ~127); }
+inline size_t keep_words_key_blocks(int max_sk) { return (size_t)(((max_sk + 127) & ~127) / 32); }
+
+// bit `pos` (a constant) of w ? a : b, as a sign-extended one-bit field and a bitwise select: two instructions
+FA_DEVICE float keep_word_select(uint32_t w, int pos, float a, float b) {
+  const uint32_t m = (uint32_t)((int32_t)(w << (31 - pos)) >> 31);
+  return __uint_as_float((m & __float_as_uint(a)) | (~m & __float_as_uint(b)));
+}
+// w <- 2 w + (this lane's bit of `mask`): one v_addc with the mask as carry-in
+FA_DEVICE uint32_t shift_in_lane_bit(uint32_t w, uint64_t mask) {
+  asm("v_addc_co_u32_e64 %0, vcc, %1, %1, %2" : "=v"(w) : "v"(w), "s"(mask) : "vcc");
+  return w;
+}
+// this lane's bit of a wave-uniform mask, as a condition the compiler selects on with the mask register as it is
+FA_DEVICE bool lane_bit(uint64_t mask) { return __builtin_amdgcn_inverse_ballot_w64(mask); }
+// The 16 keep bits of a lane in the row layout (register r <-> key 8 (r / 4) + 4 hf + r % 4 of a 32-key block), shifted in
+// register by register with shift_in_lane_bit and a 4-bit gap after every fourth: turned into the lane's share of the
+// 32-bit keep word of its query row, then joined with the share of the lane that holds the row's other 16 keys.
+FA_DEVICE uint32_t keep_word_from_shares(uint32_t w, int hf) {
+  w = __builtin_bitreverse32(w) >> (hf ? 0 : 4);  // register r of half hf now sits at bit 8 (r / 4) + 4 hf + r % 4
+  auto r = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+  return r[0] | r[1];
+}
+
 }  // namespace fa

@@ -152,6 +152,22 @@ __global__ void __launch_bounds__(256, (!kDropout && !kAlibi && D <= 64) ? 4 : 2
   for (int ks = 0; ks < D / 16; ks++) koff[ks] = frag_off<D, kSwzRow>(c, ks * 2 + hf);
   int buf = 0;
 
+  // Dropout keep words for the backward (fa_common.h): a tile's words are stored at the top of the next step, ahead of
+  // the next prefetch - stored where they are made, their acknowledgements would still be outstanding when the step
+  // ends and waits for its prefetched tile (one counter serves loads and stores).
+  uint32_t kwout[KBW];
+  int kw_pending = -1;  // first key block (of 32) of the words waiting in kwout
+  auto flush_keep_words = [&]() {
+    if (kDropout && !kSparse && kw_pending >= 0) {
+      if (hf == 0) {
+#pragma unroll
+        for (int kb = 0; kb < KBW; kb++)
+          p.keep_words[((int64_t)bh * p.kw_kb + kw_pending + kb) * p.kw_q + mw + (keep_word_slot(c) & 31)] = kwout[kb];
+      }
+      kw_pending = -1;
+    }
+  };
+
   int it = next_active(tile0);
   bool row_on_cur = row_on_next;
   if (it < ntiles) stage(it, 0);
@@ -162,6 +178,7 @@ __global__ void __launch_bounds__(256, (!kDropout && !kAlibi && D <= 64) ? 4 : 2
 #pragma unroll
     for (int i = 0; i < DV / 32; i++) asm volatile("" : "+v"(o_acc[i]));
     wait_vmem();                         // this wave's share of tile `it` is in LDS
+    flush_keep_words();
     __syncthreads();                     // so is everyone else's, and nobody still reads the other buffer
     const int it_next = next_active(it + 1);
     if (it_next < ntiles) stage(it_next, buf ^ 1);
@@ -244,9 +261,27 @@ __global__ void __launch_bounds__(256, (!kDropout && !kAlibi && D <= 64) ? 4 : 2
 #pragma unroll
           for (int kb = 0; kb < KBW; kb++) {
             const KeepFields keep = keep_fields_row_layout(p.pk, (uint32_t)bh, qrow, n0 + (kb0 + kb) * 32, hf);
+            if (!kSparse && p.keep_words != nullptr) {
+              // the lane's 16 keep bits are gathered into its share of the row's keep word (fa_common.h) for the backward
+              // (dead scores keep whatever bit they drew: their P is 0)
+              uint32_t kw = 0;
 #pragma unroll
-            for (int r = 0; r < 16; r++)
-              if (!keep.keep_row(r, p.keep_thr)) s[kb][r] = 0.f;
+              for (int r = 0; r < 16; r++) {
+                const bool kept = keep.keep_row(r, p.keep_thr);
+                if (!kept) s[kb][r] = 0.f;
+                kw = shift_in_lane_bit(kw, __builtin_amdgcn_ballot_w64(kept));
+                if ((r & 3) == 3 && r != 15) kw <<= 4;
+                // (a compare's 64-bit result is to be used up before the next is made: all sixteen held at once would
+                // overflow the scalar registers into vector ones)
+                if ((r & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+              }
+              kwout[kb] = keep_word_from_shares(kw, hf);
+              kw_pending = (n0 >> 5) + kb0;
+            } else {
+#pragma unroll
+              for (int r = 0; r < 16; r++)
+                if (!keep.keep_row(r, p.keep_thr)) s[kb][r] = 0.f;
+            }
           }
         }
 #pragma unroll
@@ -311,6 +346,7 @@ __global__ void __launch_bounds__(256, (!kDropout && !kAlibi && D <= 64) ? 4 : 2
     }
     it = it_next;
   }
+  flush_keep_words();
 
   // ---- key split: the waves kh > 0 hand their partial (O, maximum, sum) to the wave kh == 0 of their rows, in the
   // accumulator's own register order (word (rs * (16 DV/32 + 2) + j) * 64 + lane: consecutive lanes, no bank conflicts)

@@ -51,6 +51,10 @@ struct FwdParams {
   float* o_part;
   float* lse_part;
   const float* alibi;  // null, or one slope per head: the score of (query i, key j) gets -slope * |i - j| added
+  // Dropout keep words (fa_common.h), or null: the keep decisions of every score, left for the backward
+  uint32_t* keep_words;
+  int kw_q;   // query extent of the buffer (max_seqlen_q rounded up to 128)
+  int kw_kb;  // 32-key blocks (max_seqlen_k rounded up to 128, / 32)
 };
 
 struct DumpParams {  // return_softmax path
@@ -107,6 +111,10 @@ struct BwdParams {
   int n_splits;
   float* dq_part;
   const float* alibi;  // as in FwdParams
+  // Dropout keep words (fa_common.h) as the forward left them, or null: read by both kernels in place of Philox
+  const uint32_t* keep_words;
+  int kw_q;   // query extent of the buffer (max_seqlen_q rounded up to 128)
+  int kw_kb;  // 32-key blocks (max_seqlen_k rounded up to 128, / 32)
 };
 
 // Sequence extent of batch entry b, clamped so that a cu_seqlens array that disagrees with the declared

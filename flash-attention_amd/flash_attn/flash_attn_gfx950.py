@@ -20,9 +20,15 @@ LIB_NAME = "libflash_attn_gfx950.so"
 LIB_PATH = os.path.join(_HERE, LIB_NAME)
 
 FA_FP16, FA_BF16 = 0, 1
-FA_ABI_VERSION = 2
+FA_ABI_VERSION = 3
 
 _c_i32p = ctypes.c_void_p
+
+# Dropout keep words: the forward can leave its keep decisions (one bit per score) in a buffer from which the backward's two
+# kernels read them instead of drawing them again with Philox; results are the same bit for bit.  new_keep_words() makes
+# that buffer unless it would be larger than this many bytes (0: never), in which case every kernel draws its own decisions,
+# as the reference's do, and no memory beyond O(seqlen) is held between forward and backward.
+KEEP_WORDS_MAX_BYTES = 1 << 30
 
 
 class FwdArgs(ctypes.Structure):
@@ -45,6 +51,7 @@ class FwdArgs(ctypes.Structure):
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("stream", ctypes.c_void_p),
         ("alibi_slopes", ctypes.c_void_p),
+        ("keep_words", ctypes.c_void_p), ("keep_words_bytes", ctypes.c_size_t),
     ]
 
 
@@ -74,6 +81,7 @@ class BwdArgs(ctypes.Structure):
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("stream", ctypes.c_void_p),
         ("alibi_slopes", ctypes.c_void_p),
+        ("keep_words", ctypes.c_void_p), ("keep_words_bytes", ctypes.c_size_t),
     ]
 
 
@@ -95,6 +103,7 @@ EXPORTED_SYMBOLS = (
     "fa_fwd", "fa_bwd", "fa_bwd_profiled", "fa_fwd_block", "fa_bwd_block", "fa_fwd_block_noalloc", "fa_fwd_workspace_bytes", "fa_bwd_workspace_bytes",
     "fa_round_seqlens", "fa_philox_offset_increment", "fa_last_error", "fa_abi_version",
     "fa_gather_rows", "fa_scatter_rows", "fa_scatter_rows_workspace_bytes", "fa_rotary", "fa_set_launch_policy",
+    "fa_keep_words_bytes",
 )
 
 _lib = None
@@ -128,6 +137,8 @@ def load_library():
         lib.fa_fwd_workspace_bytes.restype = ctypes.c_size_t
         lib.fa_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdArgs)]
         lib.fa_bwd_workspace_bytes.restype = ctypes.c_size_t
+        lib.fa_keep_words_bytes.argtypes = [ctypes.c_int32] * 4
+        lib.fa_keep_words_bytes.restype = ctypes.c_size_t
         lib.fa_round_seqlens.argtypes = [ctypes.c_int32] * 4 + [ctypes.POINTER(ctypes.c_int32)] * 2
         lib.fa_round_seqlens.restype = None
         lib.fa_philox_offset_increment.argtypes = []
@@ -254,8 +265,27 @@ def _check_alibi(alibi_slopes, nheads, device, sparse):
     return alibi_slopes.data_ptr()
 
 
+def new_keep_words(q, cu_seqlens_q, max_seqlen_q, max_seqlen_k, p_dropout):
+    """Buffer for the dropout keep words of one forward call (argument keep_words of fwd and bwd), or None if there is no
+    dropout or the buffer would exceed KEEP_WORDS_MAX_BYTES."""
+    if not p_dropout > 0:
+        return None
+    n = load_library().fa_keep_words_bytes(cu_seqlens_q.numel() - 1, q.shape[1], int(max_seqlen_q), int(max_seqlen_k))
+    if n == 0 or n > KEEP_WORDS_MAX_BYTES:
+        return None
+    return torch.empty((n,), dtype=torch.uint8, device=q.device)
+
+
+def _keep_words_arg(a, keep_words, dev, sparse):
+    if keep_words is None or sparse:
+        return
+    _check(keep_words.device == dev and keep_words.dtype == torch.uint8 and keep_words.is_contiguous(),
+           "keep_words must be a contiguous uint8 tensor on the tensors' device (see new_keep_words)")
+    a.keep_words, a.keep_words_bytes = keep_words.data_ptr(), keep_words.numel()
+
+
 def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
-              zero_tensors, is_causal, return_softmax, gen, alibi_slopes=None):
+              zero_tensors, is_causal, return_softmax, gen, alibi_slopes=None, keep_words=None):
     lib = load_library()
     code = _dtype_code(q)
     _check(q.dim() == 3, "q must be (total_q, nheads, head_size)")
@@ -307,6 +337,7 @@ def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_
         a.workspace_bytes = ws_bytes
         a.stream = _stream_handle(dev)
         a.alibi_slopes = _check_alibi(alibi_slopes, nheads, dev, sparse)
+        _keep_words_arg(a, keep_words, dev, sparse)
         rc = (lib.fa_fwd_block if sparse else lib.fa_fwd)(ctypes.byref(a))
         if rc != 0:
             _raise(rc, lib)
@@ -315,7 +346,7 @@ def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_
 
 def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q,
               max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen, main_kernel_events=None,
-              alibi_slopes=None):
+              alibi_slopes=None, keep_words=None):
     lib = load_library()
     code = _dtype_code(q)
     _check(q.dim() == 3, "q must be (total_q, nheads, head_size)")
@@ -375,6 +406,7 @@ def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seql
         a.workspace_bytes = ws_bytes
         a.stream = _stream_handle(dev)
         a.alibi_slopes = _check_alibi(alibi_slopes, nheads, dev, sparse)
+        _keep_words_arg(a, keep_words, dev, sparse)
         if main_kernel_events is not None and not sparse:  # (start, stop) torch.cuda.Event created with enable_timing=True
             for ev in main_kernel_events:
                 if not ev.cuda_event:  # torch creates the HIP event lazily, on first record
@@ -388,20 +420,24 @@ def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seql
 
 
 def fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors,
-        is_causal, return_softmax, gen=None, alibi_slopes=None):
+        is_causal, return_softmax, gen=None, alibi_slopes=None, keep_words=None):
     """mha_fwd (fmha_api.cpp:173-299): returns [o, softmax_lse] or [o, softmax_lse, s].
-    alibi_slopes (extension, not in the reference): nheads fp32 slopes; scores get -slope * |i - j| added."""
+    alibi_slopes (extension, not in the reference): nheads fp32 slopes; scores get -slope * |i - j| added.
+    keep_words (extension): a buffer from new_keep_words() in which the dropout keep decisions are left for bwd."""
     return _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, None, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
-                     zero_tensors, is_causal, return_softmax, gen, alibi_slopes)
+                     zero_tensors, is_causal, return_softmax, gen, alibi_slopes, keep_words)
 
 
 def bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-        p_dropout, softmax_scale, zero_tensors, is_causal, gen=None, main_kernel_events=None, alibi_slopes=None):
+        p_dropout, softmax_scale, zero_tensors, is_causal, gen=None, main_kernel_events=None, alibi_slopes=None,
+        keep_words=None):
     """mha_bwd (fmha_api.cpp:302-449): fills dq, dk, dv in place, returns [dq, dk, dv, softmax_d].
     main_kernel_events: optional (start, stop) timing events recorded around the dq/dk/dv kernel alone.
-    alibi_slopes: the slopes the forward was given (extension, not in the reference)."""
+    alibi_slopes: the slopes the forward was given (extension, not in the reference).
+    keep_words (extension): the buffer the forward of this call filled; the kernels then read the dropout decisions."""
     return _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, None, max_seqlen_q,
-                     max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen, main_kernel_events, alibi_slopes)
+                     max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen, main_kernel_events, alibi_slopes,
+                     keep_words)
 
 
 def fwd_block(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,

@@ -16,17 +16,18 @@ def _get_block_size(device, head_dim, is_dropout):
 
 
 def _flash_attn_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-                        softmax_scale, causal, return_softmax, alibi_slopes=None):
+                        softmax_scale, causal, return_softmax, alibi_slopes=None, keep_words=None):
     res = _backend.fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale,
-                       False, causal, return_softmax, None, alibi_slopes)
+                       False, causal, return_softmax, None, alibi_slopes, keep_words)
     return res[0], res[1], (res[2] if return_softmax else None)
 
 
 def _flash_attn_backward(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
-                         max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal, alibi_slopes=None):
+                         max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal, alibi_slopes=None,
+                         keep_words=None):
     _, _, _, softmax_d = _backend.bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
                                       max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, False, causal, None,
-                                      alibi_slopes=alibi_slopes)
+                                      alibi_slopes=alibi_slopes, keep_words=keep_words)
     return dq, dk, dv, softmax_d
 
 
@@ -48,9 +49,16 @@ def _forward(ctx, packing, tensors, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, ma
     rng_state = torch.cuda.get_rng_state(q.device) if dropout_p > 0 else None
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
+    # with a backward to come, the forward leaves its dropout decisions (one bit per score) for it to read instead of
+    # drawing them twice more; None (no dropout, no gradient wanted, or too large: _backend.KEEP_WORDS_MAX_BYTES) = redraw
+    keep_words = None
+    if dropout_p > 0 and any(ctx.needs_input_grad[:len(tensors)]):
+        keep_words = _backend.new_keep_words(q, cu_seqlens_q, max_seqlen_q, max_seqlen_k, dropout_p)
     out, softmax_lse, S_dmask = _flash_attn_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-                                                    dropout_p, softmax_scale, causal, return_softmax, alibi_slopes)
+                                                    dropout_p, softmax_scale, causal, return_softmax, alibi_slopes,
+                                                    keep_words)
     ctx.save_for_backward(*tensors, out, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state)
+    ctx.keep_words = keep_words
     ctx.alibi_slopes = alibi_slopes  # fixed slopes, not differentiated
     ctx.packing = packing
     ctx.n_in = len(tensors)
@@ -74,7 +82,7 @@ def _backward(ctx, dout):
         torch.cuda.set_rng_state(rng_state, dev)
     _flash_attn_backward(dout.contiguous(), q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
                          ctx.max_seqlen_q, ctx.max_seqlen_k, ctx.dropout_p, ctx.softmax_scale, ctx.causal,
-                         ctx.alibi_slopes)
+                         ctx.alibi_slopes, ctx.keep_words)
     if rng_state is not None:
         torch.cuda.set_rng_state(cur_rng_state, dev)
     return grads

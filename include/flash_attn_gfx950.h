@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FA_ABI_VERSION 2
+#define FA_ABI_VERSION 3
 
 enum fa_dtype { FA_FP16 = 0, FA_BF16 = 1 };
 
@@ -74,6 +74,13 @@ typedef struct fa_fwd_args {
    * planned, README.md:49-50).  NULL, or a device array of nheads fp32 slopes: softmax_scale * q.k - slope[h] * |i - j|
    * is what the softmax sees, i and j being the positions of query and key in their sequences.  Not with a blockmask. */
   const float* alibi_slopes;
+  /* Dropout keep words (no counterpart in the reference, whose backward kernels draw every keep decision again,
+   * fmha_dgrad_kernel_1xN_loop.h:337).  NULL, or 16-byte aligned device memory of keep_words_bytes >=
+   * fa_keep_words_bytes() bytes: with p_dropout > 0 and no blockmask the forward then also leaves the keep decision of
+   * every score there, one bit each, for fa_bwd (fa_bwd_args.keep_words).  o, softmax_lse and s_dmask are what they are
+   * without it.  Ignored with p_dropout == 0 or a blockmask. */
+  void* keep_words;
+  size_t keep_words_bytes;
 } fa_fwd_args;
 
 /* Arguments of the backward pass.  Mirrors mha_bwd (fmha_api.cpp:302-321) and, when `blockmask`
@@ -117,6 +124,12 @@ typedef struct fa_bwd_args {
   size_t workspace_bytes;
   void* stream;
   const float* alibi_slopes; /* as in fa_fwd_args: the slopes the forward was given */
+  /* NULL, or the keep words the forward of this very call (same shapes, cu_seqlens, p_dropout, seed and offset) left in
+   * fa_fwd_args.keep_words: with p_dropout > 0 and no blockmask neither backward kernel then runs Philox, they read the
+   * decisions (the dropout variants of these kernels spend more than half of their vector instructions drawing them).
+   * dq, dk, dv are bit for bit what they are without it.  Ignored with p_dropout == 0 or a blockmask. */
+  const void* keep_words;
+  size_t keep_words_bytes;
 } fa_bwd_args;
 
 /* replaces flash_attn_cuda.fwd -> mha_fwd, csrc/flash_attn/fmha_api.cpp:173-299 */
@@ -156,6 +169,9 @@ int fa_fwd_block_noalloc(const fa_fwd_args* args);
  * are read. */
 size_t fa_fwd_workspace_bytes(const fa_fwd_args* args);
 size_t fa_bwd_workspace_bytes(const fa_bwd_args* args);
+/* Size of fa_fwd_args.keep_words / fa_bwd_args.keep_words: one bit per (batch, head, query, key) with both sequence
+ * lengths rounded up to 128. */
+size_t fa_keep_words_bytes(int32_t batch, int32_t nheads, int32_t max_seqlen_q, int32_t max_seqlen_k);
 
 /* Seqlen rounding used for the shapes of softmax_lse / s_dmask / softmax_d / blockmask
  * (fmha_api.cpp:232-241 dense, :509-514 block-sparse).  Writes the rounded values. */

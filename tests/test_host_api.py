@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol(lib):
     assert declared == set(be.EXPORTED_SYMBOLS)
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.fa_abi_version() == be.FA_ABI_VERSION == 2
+    assert lib.fa_abi_version() == be.FA_ABI_VERSION == 3
 
 
 def test_struct_layout_matches_library(lib):
@@ -113,6 +113,11 @@ def test_workspace_sizes(lib):
     assert lib.fa_bwd_workspace_bytes(ctypes.byref(g)) == 0  # nor the dense backward (no fp32 dq_tmp)
     g.blockmask = 0x1000
     assert lib.fa_bwd_workspace_bytes(ctypes.byref(g)) > 0   # block-sparse: room for the block activity maps
+    # dropout keep words: one bit per (batch, head, query, key), both lengths rounded up to 128
+    assert lib.fa_keep_words_bytes(8, 12, 512, 512) == 8 * 12 * 512 * 512 // 8
+    assert lib.fa_keep_words_bytes(1, 1, 100, 300) == 128 * 384 // 8
+    assert lib.fa_keep_words_bytes(2, 3, 129, 1) == 2 * 3 * 256 * 128 // 8
+    assert lib.fa_keep_words_bytes(0, 3, 129, 1) == 0 and lib.fa_keep_words_bytes(2, 3, 0, 1) == 0
 
 
 @pytest.mark.parametrize("d,sq,sk,sparse,want", [
@@ -181,7 +186,7 @@ def test_public_signatures_match_the_reference():
     from flash_attn import flash_attn_gfx950 as be
     assert list(inspect.signature(be.fwd).parameters) == [
         "q", "k", "v", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k", "p_dropout", "softmax_scale",
-        "zero_tensors", "is_causal", "return_softmax", "gen", "alibi_slopes"]      # fmha_api.cpp:173-186 + extension
+        "zero_tensors", "is_causal", "return_softmax", "gen", "alibi_slopes", "keep_words"]  # fmha_api.cpp:173-186 + extensions
     assert list(inspect.signature(be.bwd_block).parameters) == [
         "dout", "q", "k", "v", "out", "softmax_lse", "dq", "dk", "dv", "cu_seqlens_q", "cu_seqlens_k", "blockmask",
         "max_seqlen_q", "max_seqlen_k", "p_dropout", "softmax_scale", "is_causal", "gen"]  # fmha_api.cpp:575-594

@@ -54,20 +54,23 @@ def test_d64_kernels_keep_their_waves_per_simd():
         assert k["Occupancy"] >= want and k["VGPRs Spill"] <= (2 if flags == plain else 0), ("forward", flags, k)
         k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags + "Li2EEEv")  # half-size tiles
         assert k["Occupancy"] >= 4 and k["VGPRs Spill"] == 0, ("forward, key split", flags, k)
-    for flags, want in ((plain, 3), (causal, 3), (dropout, 3)):
+    # backward kernels: <..., causal, dropout mode (0 none, 1 drawn with Philox, 2 read from the forward's keep words),
+    # sparse, alibi, ...>
+    bplain, bcausal, bdrawn, bread = "Lb0ELi0ELb0ELb0E", "Lb1ELi0ELb0ELb0E", "Lb0ELi1ELb0ELb0E", "Lb0ELi2ELb0ELb0E"
+    for flags, want in ((bplain, 3), (bcausal, 3), (bdrawn, 3), (bread, 3)):
         k = _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", flags + full)
         assert k["Occupancy"] >= want and k["VGPRs Spill"] == 0, ("dq", flags, k)
         k = _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", flags + "Li2EEEv")
         assert k["Occupancy"] >= 3 and k["VGPRs Spill"] == 0, ("dq, key split", flags, k)
-    for flags, want, spill in ((plain, 3, 2), (causal, 3, 2), (dropout, 2, 0)):
+    for flags, want, spill in ((bplain, 3, 2), (bcausal, 3, 2), (bdrawn, 2, 0), (bread, 2, 0)):
         k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", flags)
         assert k["Occupancy"] >= want and k["VGPRs Spill"] <= spill, ("dkdv", flags, k)
     # the ALiBi variants (fourth flag set) keep the waves per SIMD of their plain counterparts in the backward
-    for flags in ("Lb0ELb0ELb0ELb1E", "Lb1ELb0ELb0ELb1E"):
+    for flags, bflags in (("Lb0ELb0ELb0ELb1E", "Lb0ELi0ELb0ELb1E"), ("Lb1ELb0ELb0ELb1E", "Lb1ELi0ELb0ELb1E")):
         assert _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags + full)["Occupancy"] >= 3, flags  # (the bias costs the fourth)
-        assert _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", flags + full)["Occupancy"] >= 3, flags
-        k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", flags)
-        assert k["Occupancy"] >= 3 and k["VGPRs Spill"] <= 4, (flags, k)
+        assert _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", bflags + full)["Occupancy"] >= 3, bflags
+        k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", bflags)
+        assert k["Occupancy"] >= 3 and k["VGPRs Spill"] <= 4, (bflags, k)
 
 
 @pytest.mark.timeout(600)
@@ -76,7 +79,9 @@ def test_d128_backward_keeps_two_waves_per_simd():
     (two waves per SIMD, nothing spilled: a spill's scratch load would wait behind the tile prefetch on every step)."""
     bwd = _resources("fa_bwd_d128.hip")
     for dt in ("IDF16_", "IDF16b"):
-        for flags in ("Lb0ELb0ELb0ELb0E", "Lb1ELb0ELb0ELb0E", "Lb0ELb0ELb1ELb0E", "Lb1ELb0ELb1ELb0E"):
+        # plain, causal, both with a block layout, and the two without that read the dropout decisions from keep words
+        for flags in ("Lb0ELi0ELb0ELb0E", "Lb1ELi0ELb0ELb0E", "Lb0ELi0ELb1ELb0E", "Lb1ELi0ELb1ELb0E", "Lb0ELi2ELb0ELb0E",
+                      "Lb1ELi2ELb0ELb0E"):
             k = _pick(bwd, "fa_bwd_dkdv_kernel%sLi128E" % dt, flags)
             assert k["Occupancy"] >= 2 and k["VGPRs Spill"] == 0 and k["LDS Size"] <= 80 * 1024, (dt, flags, k)
             k = _pick(bwd, "fa_bwd_dq_kernel%sLi128E" % dt, flags + "Li1EEEv")

@@ -57,6 +57,17 @@ def full_size_tiles():
     be.set_launch_policy(0)
 
 
+@pytest.fixture(params=[1 << 30, 0], ids=["keep words", "redrawn"])
+def dropout_path(request):
+    """Runs a dropout test both ways: the forward leaves its keep decisions for the backward to read (the default when
+    the buffer is small enough), or every kernel draws them again (flash_attn_gfx950.KEEP_WORDS_MAX_BYTES = 0)."""
+    from flash_attn import flash_attn_gfx950 as be
+    old = be.KEEP_WORDS_MAX_BYTES
+    be.KEEP_WORDS_MAX_BYTES = request.param
+    yield request.param
+    be.KEEP_WORDS_MAX_BYTES = old
+
+
 def _cu(lens, device="cuda"):
     return torch.tensor([0] + list(np.cumsum(lens)), dtype=torch.int32, device=device)
 
@@ -351,7 +362,7 @@ def _gen_state():
 
 
 @pytest.mark.parametrize("D,dtype,causal", [(64, torch.float16, False), (32, torch.bfloat16, True), (128, torch.float16, False)])
-def test_dropout_mask_is_the_defined_one_and_is_applied(D, dtype, causal, tile_shape):
+def test_dropout_mask_is_the_defined_one_and_is_applied(D, dtype, causal, tile_shape, dropout_path):
     p = 0.17
     lens_q, lens_k, H = [70, 130], [70, 130], 3
     q, k, v, do = _inputs(lens_q, lens_k, H, D, dtype, 21)
@@ -378,7 +389,7 @@ def test_dropout_mask_is_the_defined_one_and_is_applied(D, dtype, causal, tile_s
     check_against_oracle(ours, ref, half, dtype, what="dropout D%d" % D)
 
 
-def test_dropout_random_shapes_sweep(tile_shape):
+def test_dropout_random_shapes_sweep(tile_shape, dropout_path):
     """Eight seeded random dropout cases (rates, head dims, ragged self- and cross-attention lengths, packings): the
     returned mask equals its definition bit for bit and out / gradients equal the closed form with that mask."""
     rng = np.random.default_rng(77)
@@ -433,7 +444,7 @@ def test_dropout_keep_rate_and_rng_semantics():
     assert (per_head - kp).abs().max() < 5e-3
 
 
-def test_dropout_backward_reuses_the_forward_mask_without_probs():
+def test_dropout_backward_reuses_the_forward_mask_without_probs(dropout_path):
     """production path (no S_dmask): gradients must match the closed form under the mask defined by the state the
     generator had when the forward ran, even after other draws moved the generator on."""
     p, lens, H, D = 0.25, [96, 200], 2, 64
@@ -454,6 +465,98 @@ def test_dropout_backward_reuses_the_forward_mask_without_probs():
     half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu.tolist(), cu.tolist(), D ** -0.5, False, masks, p, dout=do.cuda())
     ours = {"out": out.detach(), "dq": qkv.grad[:, 0], "dk": qkv.grad[:, 1], "dv": qkv.grad[:, 2]}
     check_against_oracle(ours, ref, half, torch.float16, what="dropout production path")
+
+
+@pytest.mark.parametrize("D,dtype,causal,lens_q,lens_k,alibi", [
+    (64, torch.float16, False, [300, 129, 512, 77], None, False),
+    (64, torch.bfloat16, True, [405, 435, 303, 318], None, False),
+    (32, torch.float16, True, [300, 129, 512, 77], None, False),
+    (16, torch.bfloat16, False, [200, 100], [333, 1000], False),
+    (128, torch.float16, False, [300, 129, 512], None, False),
+    (128, torch.bfloat16, True, [1024, 77], None, False),
+    (64, torch.float16, False, [64, 100], [2048, 1500], False),   # short query side: the key-split dQ
+    (64, torch.float16, True, [300, 129], None, True),
+])
+def test_keep_words_hold_the_defined_mask_and_give_the_same_results(D, dtype, causal, lens_q, lens_k, alibi, tile_shape):
+    """The forward's keep words (one bit per score) equal the oracle's mask bit for bit in their documented layout, the
+    forward's outputs do not depend on whether it leaves them, and the backward that reads them gives the gradients of the
+    backward that draws the decisions again: bit for bit (at head dim 128 dq within one rounding: there the two dQ variants
+    subtract Dk from dP at different points)."""
+    from flash_attn import flash_attn_gfx950 as be
+    lens_k = lens_k or lens_q
+    p, H = 0.17, 3
+    q, k, v, do = (x.cuda() for x in _inputs(lens_q, lens_k, H, D, dtype, 77))
+    cq, ck = _cu(lens_q), _cu(lens_k)
+    mq, mk = max(lens_q), max(lens_k)
+    sl = (torch.rand(H, device="cuda") * 0.3) if alibi else None
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    st = g.get_state()
+    seed, offset = g.initial_seed(), g.get_offset()
+    o0, lse0 = be.fwd(q, k, v, cq, ck, mq, mk, p, D ** -0.5, False, causal, False, g, alibi_slopes=sl)
+    g.set_state(st)
+    kw = be.new_keep_words(q, cq, mq, mk, p)
+    assert kw is not None and kw.numel() == len(lens_q) * H * ((mq + 127) // 128 * 128) * ((mk + 127) // 128 * 128) // 8
+    kw.fill_(0xA5)
+    o1, lse1 = be.fwd(q, k, v, cq, ck, mq, mk, p, D ** -0.5, False, causal, False, g, alibi_slopes=sl, keep_words=kw)
+    assert torch.equal(o0, o1)
+    for b, L in enumerate(lens_q):
+        assert torch.equal(lse0[b, :, :L], lse1[b, :, :L])
+    # layout: word [(b H + h) * key_blocks + key / 32][slot(q)], bit key % 32; slot swaps q's bits so that rows q and q + 4 are neighbours
+    q_ext, kbs = (mq + 127) // 128 * 128, (mk + 127) // 128 * 128 // 32
+    words = kw.view(torch.int32).view(len(lens_q) * H, kbs, q_ext).cpu().numpy().astype(np.uint32)
+    for b, (Lq, Lk) in enumerate(zip(lens_q, lens_k)):
+        for h in range(H):
+            want = orc.dropout_keep_mask(seed, offset, b * H + h, Lq, Lk, p)          # [Lq, Lk] bool
+            qs = np.arange(Lq)
+            slot = (qs & ~31) | (qs & 24) | ((qs & 3) << 1) | ((qs >> 2) & 1)
+            keys = np.arange(Lk)
+            got = (words[b * H + h][keys[None, :] // 32, slot[:, None]] >> (keys[None, :] % 32).astype(np.uint32)) & 1
+            valid = orc._score_mask(Lq, Lk, causal, None).numpy()
+            assert np.array_equal(got.astype(bool)[valid], want[valid]), "keep words differ from the mask's definition"
+    grads = []
+    for words_arg in (None, kw):
+        g.set_state(st)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        be.bwd(do, q, k, v, o1, lse1, dq, dk, dv, cq, ck, mq, mk, p, D ** -0.5, False, causal, g, alibi_slopes=sl,
+               keep_words=words_arg)
+        grads.append((dq, dk, dv))
+    torch.cuda.synchronize()
+    assert torch.equal(grads[0][1], grads[1][1]) and torch.equal(grads[0][2], grads[1][2])
+    if D <= 64:
+        assert torch.equal(grads[0][0], grads[1][0])
+    else:
+        a, b_ = grads[0][0].float(), grads[1][0].float()
+        assert (a - b_).abs().max() <= 2.0 ** (-10 if dtype == torch.float16 else -7) * a.abs().max()
+
+
+def test_keep_words_argument_checks():
+    from flash_attn import flash_attn_gfx950 as be
+    lens, H, D, p = [100, 60], 2, 64, 0.1
+    q, k, v, do = (x.cuda() for x in _inputs(lens, lens, H, D, torch.float16, 3))
+    cu = _cu(lens)
+    need = be.load_library().fa_keep_words_bytes(2, H, 100, 100)
+    assert need == 2 * H * (128 // 32) * 128 * 4
+    small = torch.empty(need - 16, dtype=torch.uint8, device="cuda")
+    with pytest.raises(RuntimeError, match="keep_words of"):
+        be.fwd(q, k, v, cu, cu, 100, 100, p, D ** -0.5, False, False, False, None, keep_words=small)
+    odd = torch.empty(need + 16, dtype=torch.uint8, device="cuda")[4:]
+    with pytest.raises(RuntimeError, match="16-byte aligned"):
+        be.fwd(q, k, v, cu, cu, 100, 100, p, D ** -0.5, False, False, False, None, keep_words=odd)
+    with pytest.raises(RuntimeError, match="uint8"):
+        be.fwd(q, k, v, cu, cu, 100, 100, p, D ** -0.5, False, False, False, None, keep_words=small.view(torch.int16))
+    # without dropout the buffer is ignored, whatever its size
+    be.fwd(q, k, v, cu, cu, 100, 100, 0.0, D ** -0.5, False, False, False, None, keep_words=small)
+    old = be.KEEP_WORDS_MAX_BYTES
+    try:
+        be.KEEP_WORDS_MAX_BYTES = need - 1
+        assert be.new_keep_words(q, cu, 100, 100, p) is None
+        be.KEEP_WORDS_MAX_BYTES = need
+        assert be.new_keep_words(q, cu, 100, 100, p).numel() == need
+        assert be.new_keep_words(q, cu, 100, 100, 0.0) is None
+    finally:
+        be.KEEP_WORDS_MAX_BYTES = old
+    torch.cuda.synchronize()
 
 
 def test_element_offsets_beyond_int32():
@@ -916,7 +1019,7 @@ def _full_size_check(lens, H, D, dtype, causal, p=0.0, seed=0):
     return q, k, v, do, cu, ours
 
 
-def test_config_bert_varlen_dropout(tile_shape):
+def test_config_bert_varlen_dropout(tile_shape, dropout_path):
     """BASELINE config 2: fp16, B=8, H=12, d=64, lengths uniform in [256, 512], p=0.1."""
     g = torch.Generator().manual_seed(0)
     lens = torch.randint(256, 513, (8,), generator=g).tolist()
