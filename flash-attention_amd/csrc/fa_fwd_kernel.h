@@ -47,8 +47,11 @@ struct FwdCfg {
 
 // kAlibi: the score of (query i, key j) gets -slope[head] * |i - j| added after scaling.  The scores are then moved to the
 // softmax's own units (base-2 exponent) before the row maximum is taken, and the running maximum is kept in those units.
-template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, bool kAlibi = false, int KS = 1>
+// kWords (dropout, dense): the keep decisions are also left in p.keep_words for the backward (fa_common.h)
+template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, bool kAlibi = false, int KS = 1,
+          bool kWords = false>
 __global__ void __launch_bounds__(256, (!kDropout && !kAlibi && D <= 64) ? 4 : 2) fa_fwd_kernel(const FwdParams p) {
+  static_assert(!kWords || (kDropout && !kSparse), "keep words: dense dropout variants only");
   using Cfg = FwdCfg<T, D, BN, KS>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
@@ -158,7 +161,7 @@ __global__ void __launch_bounds__(256, (!kDropout && !kAlibi && D <= 64) ? 4 : 2
   uint32_t kwout[KBW];
   int kw_pending = -1;  // first key block (of 32) of the words waiting in kwout
   auto flush_keep_words = [&]() {
-    if (kDropout && !kSparse && kw_pending >= 0) {
+    if (kWords && kw_pending >= 0) {
       if (hf == 0) {
 #pragma unroll
         for (int kb = 0; kb < KBW; kb++)
@@ -261,7 +264,7 @@ __global__ void __launch_bounds__(256, (!kDropout && !kAlibi && D <= 64) ? 4 : 2
 #pragma unroll
           for (int kb = 0; kb < KBW; kb++) {
             const KeepFields keep = keep_fields_row_layout(p.pk, (uint32_t)bh, qrow, n0 + (kb0 + kb) * 32, hf);
-            if (!kSparse && p.keep_words != nullptr) {
+            if (kWords) {
               // the lane's 16 keep bits are gathered into its share of the row's keep word (fa_common.h) for the backward
               // (dead scores keep whatever bit they drew: their P is 0)
               uint32_t kw = 0;

@@ -48,12 +48,17 @@ def test_d64_kernels_keep_their_waves_per_simd():
     # (the dK/dV kernel has no key-split parameter)
     plain, causal, dropout = "Lb0ELb0ELb0ELb0E", "Lb1ELb0ELb0ELb0E", "Lb0ELb1ELb0ELb0E"
     full = "Li1EEEv"
+    # (the forward's last parameter: the dropout variant that also leaves its keep decisions for the backward)
     for flags, want in ((plain, 4), (causal, 4), (dropout, 3)):
-        k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags + full)
+        k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags + "Li1ELb0EEEv")
         # (the plain variant parks one register pair in scratch across its main loop: stored before, reloaded after)
         assert k["Occupancy"] >= want and k["VGPRs Spill"] <= (2 if flags == plain else 0), ("forward", flags, k)
-        k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags + "Li2EEEv")  # half-size tiles
+        k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags + "Li2ELb0EEEv")  # half-size tiles
         assert k["Occupancy"] >= 4 and k["VGPRs Spill"] == 0, ("forward, key split", flags, k)
+    k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", dropout + "Li1ELb1EEEv")
+    assert k["Occupancy"] >= 3 and k["VGPRs Spill"] == 0, ("forward, keep words", k)
+    k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", dropout + "Li2ELb1EEEv")
+    assert k["Occupancy"] >= 4 and k["VGPRs Spill"] == 0 and k["SGPRs Spill"] == 0, ("forward, keep words, key split", k)
     # backward kernels: <..., causal, dropout mode (0 none, 1 drawn with Philox, 2 read from the forward's keep words),
     # sparse, alibi, ...>
     bplain, bcausal, bdrawn, bread = "Lb0ELi0ELb0ELb0E", "Lb1ELi0ELb0ELb0E", "Lb0ELi1ELb0ELb0E", "Lb0ELi2ELb0ELb0E"
@@ -67,7 +72,7 @@ def test_d64_kernels_keep_their_waves_per_simd():
         assert k["Occupancy"] >= want and k["VGPRs Spill"] <= spill, ("dkdv", flags, k)
     # the ALiBi variants (fourth flag set) keep the waves per SIMD of their plain counterparts in the backward
     for flags, bflags in (("Lb0ELb0ELb0ELb1E", "Lb0ELi0ELb0ELb1E"), ("Lb1ELb0ELb0ELb1E", "Lb1ELi0ELb0ELb1E")):
-        assert _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags + full)["Occupancy"] >= 3, flags  # (the bias costs the fourth)
+        assert _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags + "Li1ELb0EEEv")["Occupancy"] >= 3, flags  # (the bias costs the fourth)
         assert _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", bflags + full)["Occupancy"] >= 3, bflags
         k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", bflags)
         assert k["Occupancy"] >= 3 and k["VGPRs Spill"] <= 4, (bflags, k)
