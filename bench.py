@@ -339,6 +339,9 @@ def main():
     ap.add_argument("--cpu-budget", type=float, default=20.0)
     ap.add_argument("--settle", type=float, default=0.2,
                     help="seconds of untimed steps before the warm-up (0 for counter-collection runs)")
+    ap.add_argument("--redraw-dropout", action="store_true",
+                    help="dropout configurations: every kernel draws its keep decisions with Philox (the reference's scheme) "
+                         "instead of the backward reading those the forward left (flash_attn_gfx950.KEEP_WORDS_MAX_BYTES = 0)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     a = ap.parse_args()
@@ -348,6 +351,8 @@ def main():
     import torch
     from flash_attn import flash_attn_gfx950 as be
     be.load_library()  # fails loudly if the HIP library is not built
+    if a.redraw_dropout:
+        be.KEEP_WORDS_MAX_BYTES = 0
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
 
