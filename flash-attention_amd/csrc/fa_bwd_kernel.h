@@ -62,8 +62,8 @@ struct BwdCfg {
   static constexpr int kMinBlocks = (D == 128 && kDropout) ? 1 : 2;
 };
 
-// kDrop: 0 = no dropout; 1 = the keep decisions are drawn here (Philox); 2 = they are read from the keep words the dQ
-// kernel left (fa_common.h; dense only): the kernel then has the shape and the registers of the one without dropout.
+// kDrop: 0 = no dropout; 1 = the keep decisions are drawn here (Philox); 2 = they are read from the keep words the
+// forward left (fa_common.h; dense only): the kernel then has the tile shape of the one without dropout.
 template <typename T, int D, bool kCausal, int kDrop, bool kSparse, bool kAlibi = false>
 __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64) ? 3 : (BwdCfg<T, D, kDrop == 1>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
   constexpr bool kDropout = kDrop == 1, kStored = kDrop == 2;
