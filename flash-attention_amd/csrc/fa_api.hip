@@ -509,6 +509,7 @@ int fa_rotary(const fa_rotary_args* a) {
   p.dst_row_stride = a->dst_row_stride; p.dst_part_stride = a->dst_part_stride; p.dst_head_stride = a->dst_head_stride;
   p.n_parts = a->n_parts; p.n_rotated = a->n_rotated; p.n_heads = a->n_heads; p.head_dim = a->head_dim;
   p.seqlen = a->seqlen; p.table_rows = a->table_rows; p.conjugate = a->conjugate;
+  p.row_offset = 0;
   FA_LAUNCH(fa::launch_rotary(p, a->dtype, reinterpret_cast<hipStream_t>(a->stream)));
   return FA_OK;
 }

@@ -199,6 +199,7 @@ struct RotaryParams {
   int64_t src_row_stride, src_part_stride, src_head_stride;  // elements
   int64_t dst_row_stride, dst_part_stride, dst_head_stride;
   int n_parts, n_rotated, n_heads, head_dim, seqlen, table_rows, conjugate;
+  int64_t row_offset;  // set by launch_rotary: index of this launch's first row in the caller's tensor (position = row % seqlen)
 };
 hipError_t launch_rotary(const RotaryParams& p, int dtype, hipStream_t stream);
 hipError_t launch_gather_rows(const void* src, void* dst, const int64_t* idx, int64_t n_idx, int64_t n_src,
