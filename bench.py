@@ -294,6 +294,32 @@ def sustained_mfma(torch, n=8192, iters=20):
     return out
 
 
+def graph_replay_ms(torch, fn, calls=20, replays=5):
+    """Milliseconds per call of fn, with `calls` of them captured in a HIP graph and the replays timed: for kernels that
+    run shorter than their Python call takes (argument checks, ctypes), a loop of calls would time the host.  The C ABI
+    neither allocates nor synchronises, so its calls can be captured."""
+    for _ in range(5):
+        fn()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(calls):
+                fn()
+    torch.cuda.current_stream().wait_stream(side)
+    graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(replays):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / (calls * replays)
+
+
 TRAFFIC_PROFILE = os.path.join("profiles", "headline_fp16_b8_h12_d64_n2048_hbm_traffic.md")
 
 
@@ -447,16 +473,7 @@ def main():
         for name, fn, nbytes in (
                 ("unpad_input (gather)", lambda: be.gather_rows(hidden.view(Bp * Sp, dim), idx), 2 * nnz * dim * 2 + nnz * 8),
                 ("pad_input (scatter)", lambda: be.scatter_rows(rows, idx, Bp * Sp), (nnz + Bp * Sp) * dim * 2 + nnz * 8)):
-            for _ in range(20):
-                fn()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(50):
-                fn()
-            e1.record()
-            torch.cuda.synchronize()
-            ms = e0.elapsed_time(e1) / 50
+            ms = graph_replay_ms(torch, fn)
             print("%-28s %9.4f ms  %8.1f GB/s of %d (%.1f %% of HBM peak)  [B=%d S=%d dim=%d fp16, %d of %d tokens valid]"
                   % (name, ms, nbytes / ms / 1e6, HBM_PEAK_GBS, 100 * nbytes / ms / 1e6 / HBM_PEAK_GBS, Bp, Sp, dim, nnz, Bp * Sp),
                   file=sys.stderr)
@@ -466,28 +483,7 @@ def main():
         ang = torch.outer(torch.arange(Sr, device="cuda", dtype=torch.float32),
                           1.0 / (10000 ** (torch.arange(0, Dr, 2, device="cuda").float() / Dr)))
         cos_h, sin_h = torch.cos(ang).half().contiguous(), torch.sin(ang).half().contiguous()
-        for _ in range(20):
-            be.rotary(qkv_r, qkv_r, cos_h, sin_h, n_rotated=2)
-        torch.cuda.synchronize()
-        # the Python call (argument checks, ctypes) takes longer than this kernel runs, so a loop of calls would time the
-        # host: 20 calls are captured in a HIP graph (the C ABI neither allocates nor synchronises) and the replay is timed
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.stream(side):
-            with torch.cuda.graph(graph, stream=side):
-                for _ in range(20):
-                    be.rotary(qkv_r, qkv_r, cos_h, sin_h, n_rotated=2)
-        torch.cuda.current_stream().wait_stream(side)
-        graph.replay()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(5):
-            graph.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / 100
+        ms = graph_replay_ms(torch, lambda: be.rotary(qkv_r, qkv_r, cos_h, sin_h, n_rotated=2))
         nbytes = 2 * 2 * Br * Sr * Hr * Dr * 2   # q and k read and written; v is not touched in place
         print("%-28s %9.4f ms  %8.1f GB/s of %d (%.1f %% of HBM peak)  [B=%d S=%d H=%d d=%d fp16 packed qkv, in place]"
               % ("rotary q,k (fa_rotary)", ms, nbytes / ms / 1e6, HBM_PEAK_GBS, 100 * nbytes / ms / 1e6 / HBM_PEAK_GBS,
