@@ -38,8 +38,17 @@ __global__ void __launch_bounds__(256) dq_combine_kernel(const BwdParams p, int 
   int q_begin, Lq;
   if (!seq_extent(p.cu_q, b, p.total_q, p.max_sq, &q_begin, &Lq) || row >= Lq) return;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < p.n_splits; s++)
-    acc = acc + *reinterpret_cast<const f32x4*>(p.dq_part + (((int64_t)s * p.total_q + q_begin + row) * p.H + h) * D + ch * 4);
+  constexpr int U = 8;  // eight splits' loads in flight at a time (see fwd_combine_kernel)
+  const float* part = p.dq_part + ((int64_t)(q_begin + row) * p.H + h) * D + ch * 4;
+  const int64_t step = (int64_t)p.total_q * p.H * D;
+  for (int s0 = 0; s0 < p.n_splits; s0 += U) {
+    f32x4 x[U];
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      x[u] = s0 + u < p.n_splits ? *reinterpret_cast<const f32x4*>(part + (s0 + u) * step) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < U; u++) acc = acc + x[u];
+  }
   T* op = reinterpret_cast<T*>(p.dq) + (int64_t)(q_begin + row) * p.dq_rs + (int64_t)h * p.dq_hs + ch * 4;
   *reinterpret_cast<typename Elem<T>::vec4*>(op) = cvt4<T>(acc);
 }

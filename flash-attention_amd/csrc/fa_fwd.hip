@@ -37,16 +37,39 @@ __global__ void __launch_bounds__(256) fwd_combine_kernel(const FwdParams p, int
   const int b = (int)(t / cpr / p.max_sq / p.H);
   int q_begin, Lq;
   if (!seq_extent(p.cu_q, b, p.total_q, p.max_sq, &q_begin, &Lq) || row >= Lq) return;
+  // The splits are read eight at a time, all loads of a group in flight together: with few query rows (decoding) the
+  // kernel has a handful of workgroups and its time is the latency of this loop, not bandwidth.
+  constexpr int U = 8;
+  const float* lp = p.lse_part + ((int64_t)b * p.H + h) * p.sq_r + row;
+  const int64_t lstep = (int64_t)p.B * p.H * p.sq_r;
+  const float* opart = p.o_part + ((int64_t)(q_begin + row) * p.H + h) * D + ch * 4;
+  const int64_t ostep = (int64_t)p.total_q * p.H * D;
   float m = -INFINITY;
-  for (int s = 0; s < p.n_splits; s++) m = fmaxf(m, p.lse_part[(((int64_t)s * p.B + b) * p.H + h) * p.sq_r + row]);
+  for (int s0 = 0; s0 < p.n_splits; s0 += U) {
+    float l[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) l[u] = s0 + u < p.n_splits ? lp[(s0 + u) * lstep] : -INFINITY;
+#pragma unroll
+    for (int u = 0; u < U; u++) m = fmaxf(m, l[u]);
+  }
   float sum = 0.f;
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   if (m > -INFINITY) {
-    for (int s = 0; s < p.n_splits; s++) {
-      const float w = __expf(p.lse_part[(((int64_t)s * p.B + b) * p.H + h) * p.sq_r + row] - m);
-      sum += w;
-      const f32x4 o = *reinterpret_cast<const f32x4*>(p.o_part + (((int64_t)s * p.total_q + q_begin + row) * p.H + h) * D + ch * 4);
-      acc = acc + o * w;
+    for (int s0 = 0; s0 < p.n_splits; s0 += U) {
+      float l[U];
+      f32x4 o[U];
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        const bool in = s0 + u < p.n_splits;
+        l[u] = in ? lp[(s0 + u) * lstep] : -INFINITY;
+        o[u] = in ? *reinterpret_cast<const f32x4*>(opart + (s0 + u) * ostep) : f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int u = 0; u < U; u++) {
+        const float w = __expf(l[u] - m);  // 0 for a split past the end or without keys
+        sum += w;
+        acc = acc + o[u] * w;
+      }
     }
     acc = acc * (1.f / sum);
   }
