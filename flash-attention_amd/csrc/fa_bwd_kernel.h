@@ -97,35 +97,44 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64) ? 3 : (BwdCfg<T, 
   // ---- K and V fragments of this wave's 32 keys (B operands), registers for the whole kernel (V: LDS with kVLds).
   // Keys past the end are zero: their P is finite, their dK / dV rows are never stored.
   constexpr bool kVLds = Cfg::kVLds;
+  // The loads are only issued here; what they bring is looked at after the first tile has been asked for (finish_kv below):
+  // a select or an LDS write on a loaded value at this point would hold the first tile back by a global load's latency.
   vec8 kreg[D / 16], vreg[kVLds ? 1 : D / 16];
+  u32x4 kraw[D / 16], vraw[kVLds ? BN * CH / 256 : D / 16];
+  T* const Vl = reinterpret_cast<T*>(lds_raw + Cfg::kOffV);
   {
     const int kr = key < Lk ? key : Lk - 1;
     const T* kp = reinterpret_cast<const T*>(p.k) + (int64_t)(k_begin + kr) * p.k_rs + (int64_t)h * p.k_hs + hf * 8;
     const T* vp = reinterpret_cast<const T*>(p.v) + (int64_t)(k_begin + kr) * p.v_rs + (int64_t)h * p.v_hs + hf * 8;
 #pragma unroll
     for (int ks = 0; ks < D / 16; ks++) {
-      u32x4 a = ld_global16(kp + ks * 16);
-      if (key >= Lk) a = u32x4{0, 0, 0, 0};
-      kreg[ks] = bitcast<vec8>(a);
-      if (!kVLds) {
-        u32x4 bb = ld_global16(vp + ks * 16);
-        if (key >= Lk) bb = u32x4{0, 0, 0, 0};
-        vreg[ks] = bitcast<vec8>(bb);
+      kraw[ks] = ld_global16(kp + ks * 16);
+      if (!kVLds) vraw[ks] = ld_global16(vp + ks * 16);
+    }
+    if (kVLds) {
+      const T* vt = reinterpret_cast<const T*>(p.v) + (int64_t)k_begin * p.v_rs + (int64_t)h * p.v_hs;
+#pragma unroll
+      for (int i = 0; i < BN * CH / 256; i++) {
+        const int row = (tid + i * 256) / CH, ch = (tid + i * 256) % CH;
+        const int vr = n0 + row < Lk ? n0 + row : Lk - 1;
+        vraw[i] = ld_global16(vt + (int64_t)vr * p.v_rs + ch * 8);
       }
     }
   }
-  T* const Vl = reinterpret_cast<T*>(lds_raw + Cfg::kOffV);
-  if (kVLds) {  // the first barrier of the main loop orders these writes before the first read
-    const T* vt = reinterpret_cast<const T*>(p.v) + (int64_t)k_begin * p.v_rs + (int64_t)h * p.v_hs;
+  auto finish_kv = [&]() {
 #pragma unroll
-    for (int i = 0; i < BN * CH / 256; i++) {
-      const int id = tid + i * 256;
-      const int row = id / CH, ch = id % CH;
-      u32x4 x = {0, 0, 0, 0};
-      if (n0 + row < Lk) x = ld_global16(vt + (int64_t)(n0 + row) * p.v_rs + ch * 8);
-      *reinterpret_cast<u32x4*>(Vl + row * Cfg::VS + ch * 8) = x;
+    for (int ks = 0; ks < D / 16; ks++) {
+      kreg[ks] = bitcast<vec8>(key < Lk ? kraw[ks] : u32x4{0, 0, 0, 0});
+      if (!kVLds) vreg[ks] = bitcast<vec8>(key < Lk ? vraw[ks] : u32x4{0, 0, 0, 0});
     }
-  }
+    if (kVLds) {  // the first barrier of the main loop orders these writes before the first read
+#pragma unroll
+      for (int i = 0; i < BN * CH / 256; i++) {
+        const int row = (tid + i * 256) / CH, ch = (tid + i * 256) % CH;
+        *reinterpret_cast<u32x4*>(Vl + row * Cfg::VS + ch * 8) = n0 + row < Lk ? vraw[i] : u32x4{0, 0, 0, 0};
+      }
+    }
+  };
   const T* const Vfrag = Vl + (wave * 32 + c) * Cfg::VS + hf * 8;  // this lane's V fragments: + 16 * ks elements
   int mt_begin = 0;
   if (kCausal) mt_begin = n0 / BM;  // query rows above the tile's first key see none of its keys
@@ -242,6 +251,7 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64) ? 3 : (BwdCfg<T, 
     if (kSparse) stage_blocks(tc, 0);
     else stage(mt, 0);
   }
+  finish_kv();
   while (more) {
     const int m0 = mt * BM;
     wait_vmem();  // this thread's share of the tile has arrived (LDS) / is in statpre
@@ -477,38 +487,29 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0) ? 3 : 2) fa_bwd_d
   // ---- Q and dO fragments (B operands), lse and Dk of this lane's query row.  Dk = keep * rowsum(dO o O) is computed
   // here (fmha_dgrad_kernel_1xN_loop.h:15-30 does it on the first column block) and stored to softmax_d, which the
   // dK/dV kernel, launched after this one, reads.
+  // The loads are only issued here; what they bring is looked at after the first key tile has been asked for (below):
+  // arithmetic on a loaded value at this point would hold that tile back by a global load's latency.
   vec8 qreg[D / 16], doreg[D / 16];
-  float lse2 = INFINITY, dkv = 0.f;  // +inf switches the row off
+  u32x4 qraw[D / 16], doraw[D / 16], oraw[D / 16];
+  float lse_raw = 0.f;
   {
     const int qr = qrow < Lq ? qrow : Lq - 1;
     const T* qp = reinterpret_cast<const T*>(p.q) + (int64_t)(q_begin + qr) * p.q_rs + (int64_t)h * p.q_hs + hf * 8;
     const T* dp_ = reinterpret_cast<const T*>(p.dout) + (int64_t)(q_begin + qr) * p.do_rs + (int64_t)h * p.do_hs + hf * 8;
     const T* op = reinterpret_cast<const T*>(p.out) + (int64_t)(q_begin + qr) * p.o_rs + (int64_t)h * p.o_hs + hf * 8;
-    float dsum = 0.f;
 #pragma unroll
     for (int ks = 0; ks < D / 16; ks++) {
-      u32x4 a = ld_global16(qp + ks * 16), bb = ld_global16(dp_ + ks * 16);
-      const vec8 ov = bitcast<vec8>(ld_global16(op + ks * 16));
-      if (qrow >= Lq) { a = u32x4{0, 0, 0, 0}; bb = u32x4{0, 0, 0, 0}; }
-      qreg[ks] = bitcast<vec8>(a);
-      doreg[ks] = bitcast<vec8>(bb);
-#pragma unroll
-      for (int i = 0; i < 8; i++) dsum = __builtin_fmaf((float)doreg[ks][i], (float)ov[i], dsum);
+      qraw[ks] = ld_global16(qp + ks * 16);
+      doraw[ks] = ld_global16(dp_ + ks * 16);
+      oraw[ks] = ld_global16(op + ks * 16);
     }
-    dsum = half_sum(dsum) * p.p_keep;  // lanes l and l^32 hold the two halves of each 16-element group of the row
-    if (qrow < Lq) {
-      const float x = p.lse[((int64_t)b * p.H + h) * p.lse_stride + qrow];
-      lse2 = (x == -INFINITY) ? INFINITY : x * kLog2e;
-      dkv = dsum;
-      if (hf == 0 && split == 0 && kh == 0) p.dsoftmax[((int64_t)b * p.H + h) * p.sq_r + qrow] = dsum;
-    }
+    lse_raw = p.lse[((int64_t)b * p.H + h) * p.lse_stride + qr];
   }
   // For d <= 64 the dP^T accumulator starts from -Dk of this lane's query row (16 registers that save 16 subtractions
   // per 32x32 tile); at d = 128 those registers would push the kernel below two waves per SIMD.
   constexpr bool kInitNegD = D <= 64 || !kDropout;
   f32x16 negd;
-#pragma unroll
-  for (int r = 0; r < 16; r++) negd[r] = kInitNegD ? -dkv : 0.f;
+  float lse2 = INFINITY, dkv = 0.f;  // +inf switches the row off
   int n_end = Lk;
   if (kCausal) n_end = n_end < m0 + BM ? n_end : m0 + BM;
   const int ntiles_all = (n_end + BN - 1) / BN;
@@ -585,6 +586,26 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0) ? 3 : 2) fa_bwd_d
   int it = next_active(tile0);
   bool row_on_cur = row_on_next;
   if (it < ntiles) stage(it, 0);
+  // ---- now the fragments: rows past the end are zero; Dk and -Dk, lse in base-2 units (+inf switches a row off)
+  {
+    float dsum = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ks++) {
+      const vec8 ov = bitcast<vec8>(oraw[ks]);
+      qreg[ks] = bitcast<vec8>(qrow < Lq ? qraw[ks] : u32x4{0, 0, 0, 0});
+      doreg[ks] = bitcast<vec8>(qrow < Lq ? doraw[ks] : u32x4{0, 0, 0, 0});
+#pragma unroll
+      for (int i = 0; i < 8; i++) dsum = __builtin_fmaf((float)doreg[ks][i], (float)ov[i], dsum);
+    }
+    dsum = half_sum(dsum) * p.p_keep;  // lanes l and l^32 hold the two halves of each 16-element group of the row
+    if (qrow < Lq) {
+      lse2 = (lse_raw == -INFINITY) ? INFINITY : lse_raw * kLog2e;
+      dkv = dsum;
+      if (hf == 0 && split == 0 && kh == 0) p.dsoftmax[((int64_t)b * p.H + h) * p.sq_r + qrow] = dsum;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 16; r++) negd[r] = kInitNegD ? -dkv : 0.f;
   while (it < ntiles) {
     const int n0 = it * BN;
     // Opaque redefinition of the accumulators (keeps the register allocator from copying them around the loop)
