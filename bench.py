@@ -368,6 +368,9 @@ def main():
     ap.add_argument("--redraw-dropout", action="store_true",
                     help="dropout configurations: every kernel draws its keep decisions with Philox (the reference's scheme) "
                          "instead of the backward reading those the forward left (flash_attn_gfx950.KEEP_WORDS_MAX_BYTES = 0)")
+    ap.add_argument("--only", default=None, metavar="TEXT",
+                    help="time only the BASELINE configurations whose name contains TEXT and print their table rows "
+                         "(no JSON line): for collecting rocprofv3 counters of one configuration")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     a = ap.parse_args()
@@ -388,6 +391,21 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+
+    if a.only is not None:
+        for name, kw in config_list(torch):
+            if a.only.lower() not in name.lower():
+                continue
+            wl = Workload(torch, **kw)
+            tt = time_steps(torch, be, wl, a.steps, a.warmup, a.settle)
+            fb = 3.5 * wl.fwd_flops / ((tt["fwd_ms"] + tt["bwd_ms"]) * 1e-3) / 1e12
+            gbs = (wl.bytes_fwd + wl.bytes_bwd) / ((tt["fwd_ms"] + tt["bwd_ms"]) * 1e-3) / 1e9
+            print("%-31s fwd %.4f ms  bwd %.4f ms  fwd+bwd %.1f TFLOP/s (%.2f %% of MFMA peak)  %.1f GB/s of algorithmic bytes "
+                  "(fwd %.1f MB, bwd %.1f MB)" % (name.strip(), tt["fwd_ms"], tt["bwd_ms"], fb, 100 * fb / MFMA_PEAK_TFLOPS, gbs,
+                                                   wl.bytes_fwd / 1e6, wl.bytes_bwd / 1e6), file=sys.stderr)
+            del wl
+            torch.cuda.empty_cache()
+        return
 
     B, H, D, N = 8, 12, 64, 2048
     w = Workload(torch, B, H, D, N, torch.float16)
