@@ -177,7 +177,9 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
   FA_REQUIRE(out_stride_ok(a->o_row_stride, a->head_dim) && out_stride_ok(a->o_head_stride, a->head_dim),
              "row and head strides of o must be at least head_dim (the output's rows and heads may not overlap)");
 
-  if (sparse && a->alibi_slopes) return fail(FA_ERR_UNSUPPORTED, "alibi_slopes are not supported together with a blockmask");
+  if (sparse && (a->alibi_slopes || a->attn_bias))
+    return fail(FA_ERR_UNSUPPORTED, "alibi_slopes and attn_bias are not supported together with a blockmask");
+  if (a->alibi_slopes && a->attn_bias) return fail(FA_ERR_UNSUPPORTED, "alibi_slopes and attn_bias are not supported together");
 
   const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, sparse);
   // the probability dump puts the rounded query length and batch * heads into grid dimensions: refuse what does not fit
@@ -223,6 +225,15 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
   p.keep_thr = (uint32_t)std::floor(p_keep * 65535.0);  // fmha_api.cpp:110
   p.pk = make_key(a->philox_seed, a->philox_offset);
   p.alibi = a->alibi_slopes;
+  if (a->attn_bias) {
+    FA_REQUIRE(aligned16(a->attn_bias) && a->bias_row_stride % 8 == 0 && a->bias_row_stride >= a->max_seqlen_k &&
+                   a->bias_batch_stride >= 0 && a->bias_head_stride >= 0,
+               "attn_bias must be 16-byte aligned with a row stride that is a multiple of 8 and at least max_seqlen_k");
+    if ((int64_t)a->max_seqlen_q * a->bias_row_stride >= ((int64_t)1 << 31))
+      return fail(FA_ERR_UNSUPPORTED, "attn_bias: a (batch, head) slice is limited to 2^31 elements");
+    p.bias = a->attn_bias;
+    p.bias_bs = a->bias_batch_stride; p.bias_hs = a->bias_head_stride; p.bias_rs = a->bias_row_stride;
+  }
   if (a->keep_words && dropout && !sparse) {
     FA_REQUIRE(aligned16(a->keep_words), "keep_words must be 16-byte aligned");
     const size_t kw_need = fa_keep_words_bytes(a->batch, a->nheads, a->max_seqlen_q, a->max_seqlen_k);
@@ -257,6 +268,7 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
     d.scale = a->softmax_scale;
     d.causal = a->is_causal != 0; d.dropout = dropout; d.sparse = sparse;
     d.keep_thr = p.keep_thr; d.pk = p.pk; d.sp = p.sp; d.alibi = p.alibi;
+    d.bias = p.bias; d.bias_bs = p.bias_bs; d.bias_hs = p.bias_hs; d.bias_rs = p.bias_rs;
     FA_LAUNCH(fa::launch_dump_probs(d, a->dtype, stream));
   }
   return FA_OK;
@@ -269,7 +281,9 @@ int bwd_impl(const fa_bwd_args* a, bool want_block, void* ev_main_start = nullpt
   if (rc) return rc;
   const bool sparse = a->blockmask != nullptr;
   FA_REQUIRE(sparse == want_block, want_block ? "fa_bwd_block needs a blockmask" : "fa_bwd takes no blockmask; call fa_bwd_block");
-  if (sparse && a->alibi_slopes) return fail(FA_ERR_UNSUPPORTED, "alibi_slopes are not supported together with a blockmask");
+  if (sparse && (a->alibi_slopes || a->attn_bias))
+    return fail(FA_ERR_UNSUPPORTED, "alibi_slopes and attn_bias are not supported together with a blockmask");
+  if (a->alibi_slopes && a->attn_bias) return fail(FA_ERR_UNSUPPORTED, "alibi_slopes and attn_bias are not supported together");
   FA_REQUIRE(a->dout && a->q && a->k && a->v && a->out && a->softmax_lse && a->dq && a->dk && a->dv && a->softmax_d &&
                  a->cu_seqlens_q && a->cu_seqlens_k, "NULL tensor pointer");
   FA_REQUIRE(aligned16(a->dout) && aligned16(a->q) && aligned16(a->k) && aligned16(a->v) && aligned16(a->out) &&
@@ -335,6 +349,24 @@ int bwd_impl(const fa_bwd_args* a, bool want_block, void* ev_main_start = nullpt
   p.keep_thr = (uint32_t)std::floor(p_keep * 65535.0);
   p.pk = make_key(a->philox_seed, a->philox_offset);
   p.alibi = a->alibi_slopes;
+  if (a->attn_bias) {
+    FA_REQUIRE(aligned16(a->attn_bias) && a->bias_row_stride % 8 == 0 && a->bias_row_stride >= a->max_seqlen_k &&
+                   a->bias_batch_stride >= 0 && a->bias_head_stride >= 0,
+               "attn_bias must be 16-byte aligned with a row stride that is a multiple of 8 and at least max_seqlen_k");
+    if ((int64_t)a->max_seqlen_q * a->bias_row_stride >= ((int64_t)1 << 31))
+      return fail(FA_ERR_UNSUPPORTED, "attn_bias: a (batch, head) slice is limited to 2^31 elements");
+    p.bias = a->attn_bias;
+    p.bias_bs = a->bias_batch_stride; p.bias_hs = a->bias_head_stride; p.bias_rs = a->bias_row_stride;
+  }
+  if (a->dbias) {
+    FA_REQUIRE(a->attn_bias, "dbias without attn_bias");
+    FA_REQUIRE(a->dbias_row_stride >= a->max_seqlen_k && a->dbias_head_stride > 0 && (a->dbias_batch_stride > 0 || a->batch == 1),
+               "dbias needs its own slice for every (batch, head) and rows of at least max_seqlen_k elements");
+    if ((int64_t)a->max_seqlen_q * a->dbias_row_stride >= ((int64_t)1 << 31))
+      return fail(FA_ERR_UNSUPPORTED, "dbias: a (batch, head) slice is limited to 2^31 elements");
+    p.dbias = a->dbias;
+    p.dbias_bs = a->dbias_batch_stride; p.dbias_hs = a->dbias_head_stride; p.dbias_rs = a->dbias_row_stride;
+  }
   if (a->keep_words && dropout && !sparse) {
     FA_REQUIRE(aligned16(a->keep_words), "keep_words must be 16-byte aligned");
     const size_t kw_need = fa_keep_words_bytes(a->batch, a->nheads, a->max_seqlen_q, a->max_seqlen_k);

@@ -71,6 +71,8 @@ __global__ void __launch_bounds__(256) dump_probs_kernel(const DumpParams p) {
     const float lse = p.lse[((int64_t)b * p.H + h) * p.sq_r + qrow];
     float x = s * p.scale;
     if (p.alibi) x -= p.alibi[h] * fabsf((float)(key - qrow));
+    if (p.bias)
+      x += (float)reinterpret_cast<const T*>(p.bias)[(int64_t)b * p.bias_bs + (int64_t)h * p.bias_hs + (int64_t)qrow * p.bias_rs + key];
     val = __expf(x - lse);
     if (p.dropout) {
       const uint32_t bits = dropout_keep_bits16(p.pk, (uint32_t)bh, (uint32_t)qrow >> 2, (uint32_t)key >> 2, p.keep_thr);

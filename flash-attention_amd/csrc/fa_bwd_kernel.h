@@ -64,10 +64,13 @@ struct BwdCfg {
 
 // kDrop: 0 = no dropout; 1 = the keep decisions are drawn here (Philox); 2 = they are read from the keep words the
 // forward left (fa_common.h; dense only): the kernel then has the tile shape of the one without dropout.
-template <typename T, int D, bool kCausal, int kDrop, bool kSparse, bool kAlibi = false>
-__global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64) ? 3 : (BwdCfg<T, D, kDrop == 1>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
+// kBias: as in fa_fwd_kernel; with a bias tensor the kernel also leaves d(loss)/d(bias) in p.dbias if that is not null
+template <typename T, int D, bool kCausal, int kDrop, bool kSparse, int kBias = 0>
+__global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasTensor) ? 3 : ((D == 128 && kBias == kBiasTensor) ? 1 : BwdCfg<T, D, kDrop == 1>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
   constexpr bool kDropout = kDrop == 1, kStored = kDrop == 2;
+  constexpr bool kAlibi = kBias == kBiasAlibi, kTensorBias = kBias == kBiasTensor;
   static_assert(!(kStored && kSparse), "keep words: dense only");
+  static_assert(kBias == 0 || !kSparse, "score bias: dense variants only");
   using Cfg = BwdCfg<T, D, kDropout>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
@@ -233,6 +236,14 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64) ? 3 : (BwdCfg<T, 
 
   const float cs = p.scale_log2;
   const float sl2 = kAlibi ? p.alibi[h] * kLog2e : 0.f;  // ALiBi slope in base-2 exponent units (see fa_fwd_kernel)
+  // kTensorBias: this lane's column (key) of the bias and of its gradient; row q is q * stride further
+  // (wave-uniform bases and 32-bit element offsets: a (batch, head) slice holds fewer than 2^31 elements, the front end checks)
+  const T* const bias_bh =
+      kTensorBias ? reinterpret_cast<const T*>(p.bias) + (int64_t)b * p.bias_bs + (int64_t)h * p.bias_hs : nullptr;
+  T* const dbias_bh =
+      (kTensorBias && p.dbias) ? reinterpret_cast<T*>(p.dbias) + (int64_t)b * p.dbias_bs + (int64_t)h * p.dbias_hs : nullptr;
+  const uint32_t bias_key = (uint32_t)(key < Lk ? key : Lk - 1);
+  const uint32_t bias_rs = (uint32_t)p.bias_rs, dbias_rs = (uint32_t)p.dbias_rs;
   // element offsets inside a tile of this lane's row fragments and of its transposed reads (rows +0 and +8)
   int foff[D / 16], tlo[DV / 32], thi[DV / 32];
 #pragma unroll
@@ -294,7 +305,7 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64) ? 3 : (BwdCfg<T, 
     for (int qb = 0; qb < BM / 32; qb++) {
       // dropout: the two slabs' Philox streams are not to be interleaved by the scheduler (it would, for the sake of
       // instruction-level parallelism, and need 70 more registers: one wave per SIMD fewer)
-      if (kDropout) __builtin_amdgcn_sched_barrier(0);
+      if (kDropout || kTensorBias) __builtin_amdgcn_sched_barrier(0);  // (kTensorBias: nor the two slabs' bias loads)
       // first query rows of the slab's two 16-row halves (sparse: of the two listed blocks; ascending)
       const int q_lo = kSparse ? tc.rb[2 * qb] * 16 : m0 + qb * 32;
       const int q_hi = kSparse ? tc.rb[2 * qb + 1] * 16 : q_lo + 16;
@@ -308,6 +319,17 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64) ? 3 : (BwdCfg<T, 
         const f32x4 nd4 = *reinterpret_cast<const f32x4*>(dk_l + qb * 32 + 8 * j + 4 * hf);
 #pragma unroll
         for (int i = 0; i < 4; i++) { s[4 * j + i] = 0.f; dp[4 * j + i] = nd4[i]; }
+      }
+      // kTensorBias: the bias of this lane's key for the slab's 16 query rows of the lane (register r <-> row
+      // 8 (r / 4) + 4 hf + r % 4), asked for before the MFMAs; rows past the end read the last row (their P is 0)
+      T braw[kTensorBias ? 16 : 1];
+      if (kTensorBias) {
+        const uint32_t q0 = (uint32_t)(q_lo + 4 * hf), qlast = (uint32_t)(Lq - 1);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const uint32_t qr = q0 + 8 * (r >> 2) + (r & 3);
+          braw[r] = bias_bh[(qr < qlast ? qr : qlast) * bias_rs + bias_key];
+        }
       }
       vec8 aq[D / 16], ad[D / 16];
       load_rows(qb, aq, ad);
@@ -354,6 +376,7 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64) ? 3 : (BwdCfg<T, 
           const int r = 4 * j + i;
           float e = -lse4[i];
           if (kAlibi) e = __builtin_fmaf(__builtin_fabsf(dbase - (float)(8 * j + i)), -sl2, -lse4[i]);
+          if (kTensorBias) e = __builtin_fmaf((float)braw[r], kLog2e, -lse4[i]);
           const float pe = fast_exp2(__builtin_fmaf(s[r], cs, e));
           float dpe = dp[r];  // dP - Dk
           float pm = pe;
@@ -361,6 +384,14 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64) ? 3 : (BwdCfg<T, 
           if (kStored && !lane_bit(km[r])) { dpe = nd4[i]; pm = 0.f; }
           s[r] = pm;          // P o M, feeds dV
           dp[r] = pe * dpe;   // dS' = P o (M o dP - Dk), feeds dK
+        }
+      }
+      if (kTensorBias && dbias_bh != nullptr && key < Lk) {  // d(loss)/d(bias) = dS = dS' / keep
+        const uint32_t q0 = (uint32_t)(q_lo + 4 * hf);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const uint32_t qr = q0 + 8 * (r >> 2) + (r & 3);
+          if (qr < (uint32_t)Lq) dbias_bh[qr * dbias_rs + (uint32_t)key] = (T)(dp[r] * p.rp_keep);
         }
       }
       // ---- dV^T += dO^T P; dK^T += Q^T dS'
@@ -450,9 +481,11 @@ struct DqCfg {
 };
 
 // kDrop: as in fa_bwd_dkdv_kernel
-template <typename T, int D, int BN, bool kCausal, int kDrop, bool kSparse, bool kAlibi = false, int KS = 1>
-__global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0) ? 3 : 2) fa_bwd_dq_kernel(const BwdParams p) {
+template <typename T, int D, int BN, bool kCausal, int kDrop, bool kSparse, int kBias = 0, int KS = 1>
+__global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasTensor) ? 3 : 2) fa_bwd_dq_kernel(const BwdParams p) {
   constexpr bool kDropout = kDrop == 1, kStored = kDrop == 2;
+  constexpr bool kAlibi = kBias == kBiasAlibi, kTensorBias = kBias == kBiasTensor;
+  static_assert(kBias == 0 || !kSparse, "score bias: dense variants only");
   static_assert(!(kStored && kSparse), "keep words: dense only");
   using Cfg = DqCfg<T, D, BN, KS>;
   using E = Elem<T>;
@@ -569,6 +602,11 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0) ? 3 : 2) fa_bwd_d
 
   const float cs = p.scale_log2;
   const float sl2 = kAlibi ? p.alibi[h] * kLog2e : 0.f;  // ALiBi slope in base-2 exponent units (see fa_fwd_kernel)
+  // kTensorBias: this lane's row of the bias (rows past the end read the last row, like Q)
+  const T* const bias_row =
+      kTensorBias ? reinterpret_cast<const T*>(p.bias) + (int64_t)b * p.bias_bs + (int64_t)h * p.bias_hs +
+                        (int64_t)(qrow < Lq ? qrow : Lq - 1) * p.bias_rs
+                  : nullptr;
   // element offsets inside a tile: row fragments of K (dual swizzle) and V, transposed reads of K (rows +0, +8)
   int kfoff[D / 16], vfoff[D / 16], tlo[DV / 32], thi[DV / 32];
 #pragma unroll
@@ -643,6 +681,16 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0) ? 3 : 2) fa_bwd_d
         f32x16 s, dp = negd;
 #pragma unroll
         for (int r = 0; r < 16; r++) s[r] = 0.f;
+        // kTensorBias: as in the forward kernel - 4 x 4 consecutive values per 32-key block, groups past the last key not read
+        typename E::vec4 bv[4];
+        if (kTensorBias) {
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            const int k0 = n0 + kb * 32 + 8 * j + 4 * hf;
+            bv[j] = typename E::vec4{0, 0, 0, 0};
+            if (k0 < Lk) bv[j] = *reinterpret_cast<const typename E::vec4*>(bias_row + k0);
+          }
+        }
 #pragma unroll
         for (int ks = 0; ks < D / 16; ks++) {
           vec8 a = *reinterpret_cast<const vec8*>(Ks + kb * 32 * D + kfoff[ks]);
@@ -673,6 +721,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0) ? 3 : 2) fa_bwd_d
             e = kCausal ? __builtin_fmaf(cr, sl2, __builtin_fmaf(dbase, sl2, -lse_t))
                         : __builtin_fmaf(__builtin_fabsf(dbase + cr), -sl2, -lse_t);
           }
+          if (kTensorBias) e = (s[r] == -INFINITY) ? 0.f : __builtin_fmaf((float)bv[r >> 2][r & 3], kLog2e, -lse_t);
           const float pe = fast_exp2(__builtin_fmaf(s[r], cs, e));  // 0 for dead scores and switched-off rows
           float dpe = kInitNegD ? dp[r] : dp[r] - dkv;  // dP - Dk
           if (kDropout && !keep.keep_row(r, p.keep_thr)) dpe = -dkv;

@@ -45,13 +45,16 @@ struct FwdCfg {
   static constexpr int CH = D / 8;
 };
 
-// kAlibi: the score of (query i, key j) gets -slope[head] * |i - j| added after scaling.  The scores are then moved to the
-// softmax's own units (base-2 exponent) before the row maximum is taken, and the running maximum is kept in those units.
+// kBias (fa_params.h): 1 = ALiBi, the score of (query i, key j) gets -slope[head] * |i - j| added after scaling; 2 = it gets
+// bias[b, h, i, j] of a tensor added.  The scores are then moved to the softmax's own units (base-2 exponent) before the row
+// maximum is taken, and the running maximum is kept in those units.
 // kWords (dropout, dense): the keep decisions are also left in p.keep_words for the backward (fa_common.h)
-template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, bool kAlibi = false, int KS = 1,
+template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, int kBias = 0, int KS = 1,
           bool kWords = false>
-__global__ void __launch_bounds__(256, (!kDropout && !kAlibi && D <= 64) ? 4 : 2) fa_fwd_kernel(const FwdParams p) {
+__global__ void __launch_bounds__(256, (!kDropout && kBias == 0 && D <= 64) ? 4 : 2) fa_fwd_kernel(const FwdParams p) {
+  constexpr bool kAlibi = kBias == kBiasAlibi, kTensorBias = kBias == kBiasTensor;
   static_assert(!kWords || (kDropout && !kSparse), "keep words: dense dropout variants only");
+  static_assert(kBias == 0 || !kSparse, "score bias: dense variants only");
   using Cfg = FwdCfg<T, D, BN, KS>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
@@ -145,8 +148,13 @@ __global__ void __launch_bounds__(256, (!kDropout && !kAlibi && D <= 64) ? 4 : 2
   float l_i = 0.f;        // this lane's share of the running row sum (other share in lane^32)
 
   const float cs = p.scale_log2;
-  const float cse = kAlibi ? 1.f : cs;                           // units of the scores the softmax works on
+  const float cse = kBias != 0 ? 1.f : cs;                       // units of the scores the softmax works on
   const float sl2 = kAlibi ? p.alibi[h] * kLog2e : 0.f;          // slope in base-2 exponent units
+  // kTensorBias: this lane's row of the bias (rows past the end read the last row, like Q)
+  const T* const bias_row =
+      kTensorBias ? reinterpret_cast<const T*>(p.bias) + (int64_t)b * p.bias_bs + (int64_t)h * p.bias_hs +
+                        (int64_t)(qrow < Lq ? qrow : Lq - 1) * p.bias_rs
+                  : nullptr;
   int voff[DV / 32];  // element offsets of this lane's transposed V reads and K row fragments inside a tile
 #pragma unroll
   for (int db = 0; db < DV / 32; db++) voff[db] = tr_off<D, kSwzTr>(0, db * 4, lane);
@@ -205,6 +213,19 @@ __global__ void __launch_bounds__(256, (!kDropout && !kAlibi && D <= 64) ? 4 : 2
       f32x16 s[KBW];
       // ---- S^T = K Q^T, dead scores set to -inf, bias added
       auto scores = [&]() {
+        // kTensorBias: the lane's 4 x 4 consecutive bias values per 32-key block (registers 4 j .. 4 j + 3 <-> keys
+        // 8 j + 4 hf ..), asked for before the MFMAs; groups that begin past the last key are not read
+        typename E::vec4 bv[kTensorBias ? KBW : 1][4];
+        if (kTensorBias) {
+#pragma unroll
+          for (int kb = 0; kb < KBW; kb++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+              const int k0 = n0 + (kb0 + kb) * 32 + 8 * j + 4 * hf;
+              bv[kb][j] = typename E::vec4{0, 0, 0, 0};
+              if (k0 < Lk) bv[kb][j] = *reinterpret_cast<const typename E::vec4*>(bias_row + k0);
+            }
+        }
 #pragma unroll
         for (int kb = 0; kb < KBW; kb++) {
 #pragma unroll
@@ -227,6 +248,15 @@ __global__ void __launch_bounds__(256, (!kDropout && !kAlibi && D <= 64) ? 4 : 2
               bool dead = key >= Lk;
               if (kCausal) dead = dead || key > qrow;
               if (dead) s[kb][r] = -INFINITY;
+            }
+        }
+        if (kTensorBias) {  // s <- s * scale * log2(e) + bias * log2(e); dead scores stay -inf whatever lies behind them
+#pragma unroll
+          for (int kb = 0; kb < KBW; kb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+              const float bf = (s[kb][r] == -INFINITY) ? 0.f : (float)bv[kb][r >> 2][r & 3] * kLog2e;
+              s[kb][r] = __builtin_fmaf(s[kb][r], cs, bf);
             }
         }
         if (kAlibi) {  // s <- s * scale * log2(e) - slope2 * |key - query|; dead scores stay -inf
@@ -256,7 +286,7 @@ __global__ void __launch_bounds__(256, (!kDropout && !kAlibi && D <= 64) ? 4 : 2
         for (int kb = 0; kb < KBW; kb++)
 #pragma unroll
           for (int r = 0; r < 16; r++) {
-            const float pe = fast_exp2(kAlibi ? s[kb][r] - mc : __builtin_fmaf(s[kb][r], cs, -mc));
+            const float pe = fast_exp2(kBias != 0 ? s[kb][r] - mc : __builtin_fmaf(s[kb][r], cs, -mc));
             s[kb][r] = pe;
             if (kDropout) lt += pe;
           }

@@ -24,6 +24,11 @@ struct SparseMaps {
   int nrw;   // 64-bit words per row of cbits
 };
 
+// What is added to the scaled scores before the softmax (template parameter kBias of the kernels)
+constexpr int kBiasNone = 0;    // nothing
+constexpr int kBiasAlibi = 1;   // -slope[head] * |query - key| (alibi)
+constexpr int kBiasTensor = 2;  // bias[b, h, query, key] (bias, strides in elements; batch and head stride may be 0)
+
 struct FwdParams {
   const void* q;
   const void* k;
@@ -51,6 +56,8 @@ struct FwdParams {
   float* o_part;
   float* lse_part;
   const float* alibi;  // null, or one slope per head: the score of (query i, key j) gets -slope * |i - j| added
+  const void* bias;    // null, or a tensor of the element type added to the scaled scores: [b, h, query, key]
+  int64_t bias_bs, bias_hs, bias_rs;  // its batch, head (0: shared) and row strides in elements; keys are contiguous
   // Dropout keep words (fa_common.h), or null: the keep decisions of every score, left for the backward
   uint32_t* keep_words;
   int kw_q;   // query extent of the buffer (max_seqlen_q rounded up to 128)
@@ -75,6 +82,8 @@ struct DumpParams {  // return_softmax path
   PhiloxKey pk;
   SparseMaps sp;
   const float* alibi;
+  const void* bias;  // as in FwdParams
+  int64_t bias_bs, bias_hs, bias_rs;
 };
 
 struct BwdParams {
@@ -111,6 +120,10 @@ struct BwdParams {
   int n_splits;
   float* dq_part;
   const float* alibi;  // as in FwdParams
+  const void* bias;    // as in FwdParams
+  int64_t bias_bs, bias_hs, bias_rs;
+  void* dbias;         // null, or where the dK/dV kernel leaves d(loss)/d(bias) = dS / keep: [b, h, query, key], written for the
+  int64_t dbias_bs, dbias_hs, dbias_rs;  // (query, key) tiles it visits (the caller clears the tensor)
   // Dropout keep words (fa_common.h) as the forward left them, or null: read by both kernels in place of Philox
   const uint32_t* keep_words;
   int kw_q;   // query extent of the buffer (max_seqlen_q rounded up to 128)

@@ -20,7 +20,7 @@ LIB_NAME = "libflash_attn_gfx950.so"
 LIB_PATH = os.path.join(_HERE, LIB_NAME)
 
 FA_FP16, FA_BF16 = 0, 1
-FA_ABI_VERSION = 3
+FA_ABI_VERSION = 4
 
 _c_i32p = ctypes.c_void_p
 
@@ -52,6 +52,8 @@ class FwdArgs(ctypes.Structure):
         ("stream", ctypes.c_void_p),
         ("alibi_slopes", ctypes.c_void_p),
         ("keep_words", ctypes.c_void_p), ("keep_words_bytes", ctypes.c_size_t),
+        ("attn_bias", ctypes.c_void_p), ("bias_batch_stride", ctypes.c_int64), ("bias_head_stride", ctypes.c_int64),
+        ("bias_row_stride", ctypes.c_int64),
     ]
 
 
@@ -82,6 +84,10 @@ class BwdArgs(ctypes.Structure):
         ("stream", ctypes.c_void_p),
         ("alibi_slopes", ctypes.c_void_p),
         ("keep_words", ctypes.c_void_p), ("keep_words_bytes", ctypes.c_size_t),
+        ("attn_bias", ctypes.c_void_p), ("bias_batch_stride", ctypes.c_int64), ("bias_head_stride", ctypes.c_int64),
+        ("bias_row_stride", ctypes.c_int64),
+        ("dbias", ctypes.c_void_p), ("dbias_batch_stride", ctypes.c_int64), ("dbias_head_stride", ctypes.c_int64),
+        ("dbias_row_stride", ctypes.c_int64),
     ]
 
 
@@ -265,6 +271,37 @@ def _check_alibi(alibi_slopes, nheads, device, sparse):
     return alibi_slopes.data_ptr()
 
 
+def prepare_attn_bias(attn_bias, q, batch, nheads, max_seqlen_q, max_seqlen_k):
+    """The tensor the kernels read for attn_bias (an extension: the reference only plans attention bias, README.md:50):
+    attn_bias itself if it already is what they need - 4-D, (1 or batch, 1 or nheads, >= max_seqlen_q, >= max_seqlen_k) in
+    q's dtype on q's device, keys contiguous, 16-byte aligned, row stride a multiple of 8 - else a copy with padded rows."""
+    _check(attn_bias.dim() == 4 and attn_bias.shape[0] in (1, batch) and attn_bias.shape[1] in (1, nheads) and
+           attn_bias.shape[2] >= max_seqlen_q and attn_bias.shape[3] >= max_seqlen_k,
+           "attn_bias must be (1 or batch, 1 or nheads, >= max_seqlen_q, >= max_seqlen_k), got %s" % (tuple(attn_bias.shape),))
+    _check(attn_bias.device == q.device and attn_bias.dtype == q.dtype, "attn_bias must have q's dtype and device")
+    ok = (attn_bias.stride(3) == 1 and attn_bias.stride(2) % 8 == 0 and attn_bias.stride(2) >= max_seqlen_k and
+          attn_bias.data_ptr() % 16 == 0 and all(attn_bias.stride(i) % 8 == 0 for i in (0, 1)))
+    if not ok:
+        sk8 = (attn_bias.shape[3] + 7) // 8 * 8
+        padded = torch.zeros(attn_bias.shape[:3] + (sk8,), dtype=attn_bias.dtype, device=attn_bias.device)
+        padded[..., :attn_bias.shape[3]] = attn_bias
+        attn_bias = padded
+    return attn_bias
+
+
+def _bias_arg(a, attn_bias, q, batch, nheads, max_seqlen_q, max_seqlen_k, sparse):
+    """Fills the attn_bias fields of a FwdArgs / BwdArgs; returns the tensor they point into (to be kept alive)."""
+    if attn_bias is None:
+        return None
+    _check(not sparse, "attn_bias is not supported together with a blockmask")
+    t = prepare_attn_bias(attn_bias, q, batch, nheads, int(max_seqlen_q), int(max_seqlen_k))
+    a.attn_bias = t.data_ptr()
+    a.bias_batch_stride = 0 if t.shape[0] == 1 else t.stride(0)
+    a.bias_head_stride = 0 if t.shape[1] == 1 else t.stride(1)
+    a.bias_row_stride = t.stride(2)
+    return t
+
+
 def new_keep_words(q, cu_seqlens_q, max_seqlen_q, max_seqlen_k, p_dropout):
     """Buffer for the dropout keep words of one forward call (argument keep_words of fwd and bwd), or None if there is no
     dropout or the buffer would exceed KEEP_WORDS_MAX_BYTES."""
@@ -285,7 +322,7 @@ def _keep_words_arg(a, keep_words, dev, sparse):
 
 
 def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
-              zero_tensors, is_causal, return_softmax, gen, alibi_slopes=None, keep_words=None):
+              zero_tensors, is_causal, return_softmax, gen, alibi_slopes=None, keep_words=None, attn_bias=None):
     lib = load_library()
     code = _dtype_code(q)
     _check(q.dim() == 3, "q must be (total_q, nheads, head_size)")
@@ -338,6 +375,7 @@ def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_
         a.stream = _stream_handle(dev)
         a.alibi_slopes = _check_alibi(alibi_slopes, nheads, dev, sparse)
         _keep_words_arg(a, keep_words, dev, sparse)
+        bias_t = _bias_arg(a, attn_bias, q, batch, nheads, max_seqlen_q, max_seqlen_k, sparse)  # noqa: F841 (kept alive)
         rc = (lib.fa_fwd_block if sparse else lib.fa_fwd)(ctypes.byref(a))
         if rc != 0:
             _raise(rc, lib)
@@ -346,7 +384,7 @@ def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_
 
 def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q,
               max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen, main_kernel_events=None,
-              alibi_slopes=None, keep_words=None):
+              alibi_slopes=None, keep_words=None, attn_bias=None, dbias=None):
     lib = load_library()
     code = _dtype_code(q)
     _check(q.dim() == 3, "q must be (total_q, nheads, head_size)")
@@ -407,6 +445,14 @@ def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seql
         a.stream = _stream_handle(dev)
         a.alibi_slopes = _check_alibi(alibi_slopes, nheads, dev, sparse)
         _keep_words_arg(a, keep_words, dev, sparse)
+        bias_t = _bias_arg(a, attn_bias, q, batch, nheads, max_seqlen_q, max_seqlen_k, sparse)  # noqa: F841 (kept alive)
+        if dbias is not None:
+            _check(attn_bias is not None, "dbias without attn_bias")
+            _check(dbias.dim() == 4 and tuple(dbias.shape[:2]) == (batch, nheads) and dbias.shape[2] >= max_seqlen_q and
+                   dbias.shape[3] >= max_seqlen_k and dbias.stride(3) == 1 and dbias.dtype == q.dtype and dbias.device == dev,
+                   "dbias must be (batch, nheads, >= max_seqlen_q, >= max_seqlen_k) in q's dtype, keys contiguous")
+            a.dbias = dbias.data_ptr()
+            a.dbias_batch_stride, a.dbias_head_stride, a.dbias_row_stride = dbias.stride(0), dbias.stride(1), dbias.stride(2)
         if main_kernel_events is not None and not sparse:  # (start, stop) torch.cuda.Event created with enable_timing=True
             for ev in main_kernel_events:
                 if not ev.cuda_event:  # torch creates the HIP event lazily, on first record
@@ -420,24 +466,28 @@ def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seql
 
 
 def fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors,
-        is_causal, return_softmax, gen=None, alibi_slopes=None, keep_words=None):
+        is_causal, return_softmax, gen=None, alibi_slopes=None, keep_words=None, attn_bias=None):
     """mha_fwd (fmha_api.cpp:173-299): returns [o, softmax_lse] or [o, softmax_lse, s].
     alibi_slopes (extension, not in the reference): nheads fp32 slopes; scores get -slope * |i - j| added.
-    keep_words (extension): a buffer from new_keep_words() in which the dropout keep decisions are left for bwd."""
+    keep_words (extension): a buffer from new_keep_words() in which the dropout keep decisions are left for bwd.
+    attn_bias (extension): (1 or batch, 1 or nheads, max_seqlen_q, max_seqlen_k) in q's dtype, added to the scaled scores
+    (positions counted inside the sequences; -inf masks); see prepare_attn_bias."""
     return _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, None, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
-                     zero_tensors, is_causal, return_softmax, gen, alibi_slopes, keep_words)
+                     zero_tensors, is_causal, return_softmax, gen, alibi_slopes, keep_words, attn_bias)
 
 
 def bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
         p_dropout, softmax_scale, zero_tensors, is_causal, gen=None, main_kernel_events=None, alibi_slopes=None,
-        keep_words=None):
+        keep_words=None, attn_bias=None, dbias=None):
     """mha_bwd (fmha_api.cpp:302-449): fills dq, dk, dv in place, returns [dq, dk, dv, softmax_d].
+    attn_bias: the bias the forward was given; dbias: None, or a zero-filled (batch, nheads, max_seqlen_q, max_seqlen_k)
+    tensor of q's dtype in which the gradient of the bias is left (per batch entry and head: sum for a shared bias).
     main_kernel_events: optional (start, stop) timing events recorded around the dq/dk/dv kernel alone.
     alibi_slopes: the slopes the forward was given (extension, not in the reference).
     keep_words (extension): the buffer the forward of this call filled; the kernels then read the dropout decisions."""
     return _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, None, max_seqlen_q,
                      max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen, main_kernel_events, alibi_slopes,
-                     keep_words)
+                     keep_words, attn_bias, dbias)
 
 
 def fwd_block(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,

@@ -16,18 +16,18 @@ def _get_block_size(device, head_dim, is_dropout):
 
 
 def _flash_attn_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-                        softmax_scale, causal, return_softmax, alibi_slopes=None, keep_words=None):
+                        softmax_scale, causal, return_softmax, alibi_slopes=None, keep_words=None, attn_bias=None):
     res = _backend.fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale,
-                       False, causal, return_softmax, None, alibi_slopes, keep_words)
+                       False, causal, return_softmax, None, alibi_slopes, keep_words, attn_bias)
     return res[0], res[1], (res[2] if return_softmax else None)
 
 
 def _flash_attn_backward(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
                          max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal, alibi_slopes=None,
-                         keep_words=None):
+                         keep_words=None, attn_bias=None, dbias=None):
     _, _, _, softmax_d = _backend.bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
                                       max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, False, causal, None,
-                                      alibi_slopes=alibi_slopes, keep_words=keep_words)
+                                      alibi_slopes=alibi_slopes, keep_words=keep_words, attn_bias=attn_bias, dbias=dbias)
     return dq, dk, dv, softmax_d
 
 
@@ -43,7 +43,7 @@ def _split(packing, tensors):
 
 
 def _forward(ctx, packing, tensors, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-             softmax_scale, causal, return_softmax, alibi_slopes=None):
+             softmax_scale, causal, return_softmax, alibi_slopes=None, attn_bias=None):
     q, k, v = _split(packing, tensors)
     # the dropout mask is a function of the generator state at this point; the backward rewinds to it
     rng_state = torch.cuda.get_rng_state(q.device) if dropout_p > 0 else None
@@ -52,12 +52,19 @@ def _forward(ctx, packing, tensors, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, ma
     # with a backward to come, the forward leaves its dropout decisions (one bit per score) for it to read instead of
     # drawing them twice more; None (no dropout, no gradient wanted, or too large: _backend.KEEP_WORDS_MAX_BYTES) = redraw
     keep_words = None
-    if dropout_p > 0 and any(ctx.needs_input_grad[:len(tensors)]):
+    if dropout_p > 0 and any(ctx.needs_input_grad):
         keep_words = _backend.new_keep_words(q, cu_seqlens_q, max_seqlen_q, max_seqlen_k, dropout_p)
+    # the bias in the form the kernels read (the caller's tensor itself if its layout allows, else a padded copy)
+    bias_t = None
+    if attn_bias is not None:
+        bias_t = _backend.prepare_attn_bias(attn_bias.detach(), q, cu_seqlens_q.numel() - 1, q.shape[1], int(max_seqlen_q),
+                                            int(max_seqlen_k))
     out, softmax_lse, S_dmask = _flash_attn_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
                                                     dropout_p, softmax_scale, causal, return_softmax, alibi_slopes,
-                                                    keep_words)
-    ctx.save_for_backward(*tensors, out, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state)
+                                                    keep_words, bias_t)
+    ctx.save_for_backward(*tensors, out, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state, bias_t)
+    ctx.bias_shape = tuple(attn_bias.shape) if attn_bias is not None else None
+    ctx.bias_needs_grad = attn_bias is not None and attn_bias.requires_grad
     ctx.keep_words = keep_words
     ctx.alibi_slopes = alibi_slopes  # fixed slopes, not differentiated
     ctx.packing = packing
@@ -72,34 +79,57 @@ def _forward(ctx, packing, tensors, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, ma
 def _backward(ctx, dout):
     saved = ctx.saved_tensors
     tensors = saved[:ctx.n_in]
-    out, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state = saved[ctx.n_in:]
+    out, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state, bias_t = saved[ctx.n_in:]
     q, k, v = _split(ctx.packing, tensors)
     grads = tuple(torch.empty_like(t) for t in tensors)
     dq, dk, dv = _split(ctx.packing, grads)
     dev = q.device
+    dbias = None
+    if ctx.bias_needs_grad:  # per (batch, head); only the tiles the kernels visit are written
+        dbias = torch.zeros((cu_seqlens_q.numel() - 1, q.shape[1], ctx.max_seqlen_q, (ctx.max_seqlen_k + 7) // 8 * 8),
+                            dtype=q.dtype, device=dev)
     if rng_state is not None:
         cur_rng_state = torch.cuda.get_rng_state(dev)
         torch.cuda.set_rng_state(rng_state, dev)
     _flash_attn_backward(dout.contiguous(), q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
                          ctx.max_seqlen_q, ctx.max_seqlen_k, ctx.dropout_p, ctx.softmax_scale, ctx.causal,
-                         ctx.alibi_slopes, ctx.keep_words)
+                         ctx.alibi_slopes, ctx.keep_words, bias_t, dbias)
     if rng_state is not None:
         torch.cuda.set_rng_state(cur_rng_state, dev)
+    ctx.dbias = None
+    if dbias is not None:  # back to the shape the caller's bias has: summed over the batch entries / heads that shared it
+        g = dbias[:, :, :, :ctx.max_seqlen_k]
+        shp = ctx.bias_shape
+        if shp[0] == 1 and g.shape[0] > 1:
+            g = g.float().sum(0, keepdim=True)
+        if shp[1] == 1 and g.shape[1] > 1:
+            g = g.float().sum(1, keepdim=True)
+        full = torch.zeros(shp, dtype=q.dtype, device=dev)  # rows / keys beyond max_seqlen get no gradient
+        full[:, :, :ctx.max_seqlen_q, :ctx.max_seqlen_k] = g.to(q.dtype)
+        ctx.dbias = full
     return grads
 
 
+def _extra_grads(ctx, grads):
+    """grads of the tensors, then None for every other argument - but the bias gradient for attn_bias, the last one."""
+    extra = [None] * ctx.n_extra
+    if ctx.dbias is not None:
+        extra[-1] = ctx.dbias
+    return grads + tuple(extra)
+
+
 class FlashAttnQKVPackedFunc(torch.autograd.Function):
-    """apply(qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal, return_softmax[, alibi_slopes])"""
+    """apply(qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal, return_softmax[, alibi_slopes[, attn_bias]])"""
 
     @staticmethod
-    def forward(ctx, qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal, return_softmax, *alibi_slopes):
-        ctx.n_extra = 6 + len(alibi_slopes)  # the reference's six non-tensor arguments (:72), plus the optional slopes
+    def forward(ctx, qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal, return_softmax, *bias):
+        ctx.n_extra = 6 + len(bias)  # the reference's six non-tensor arguments (:72), plus the optional alibi_slopes, attn_bias
         return _forward(ctx, "qkv", (qkv,), cu_seqlens, cu_seqlens, max_seqlen, max_seqlen, dropout_p, softmax_scale,
-                        causal, return_softmax, *alibi_slopes)
+                        causal, return_softmax, *bias)
 
     @staticmethod
     def backward(ctx, dout, *args):
-        return _backward(ctx, dout) + (None,) * ctx.n_extra
+        return _extra_grads(ctx, _backward(ctx, dout))
 
 
 class FlashAttnKVPackedFunc(torch.autograd.Function):
@@ -108,14 +138,14 @@ class FlashAttnKVPackedFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, kv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal,
-                return_softmax, *alibi_slopes):
-        ctx.n_extra = 8 + len(alibi_slopes)  # :111
+                return_softmax, *bias):
+        ctx.n_extra = 8 + len(bias)  # :111
         return _forward(ctx, "kv", (q, kv), cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-                        softmax_scale, causal, return_softmax, *alibi_slopes)
+                        softmax_scale, causal, return_softmax, *bias)
 
     @staticmethod
     def backward(ctx, dout, *args):
-        return _backward(ctx, dout) + (None,) * ctx.n_extra
+        return _extra_grads(ctx, _backward(ctx, dout))
 
 
 class FlashAttnFunc(torch.autograd.Function):
@@ -124,14 +154,14 @@ class FlashAttnFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal,
-                return_softmax, *alibi_slopes):
-        ctx.n_extra = 8 + len(alibi_slopes)  # :148
+                return_softmax, *bias):
+        ctx.n_extra = 8 + len(bias)  # :148
         return _forward(ctx, "sep", (q, k, v), cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-                        softmax_scale, causal, return_softmax, *alibi_slopes)
+                        softmax_scale, causal, return_softmax, *bias)
 
     @staticmethod
     def backward(ctx, dout, *args):
-        return _backward(ctx, dout) + (None,) * ctx.n_extra
+        return _extra_grads(ctx, _backward(ctx, dout))
 
 
 _COMMON_DOC = """
@@ -148,6 +178,10 @@ _COMMON_DOC = """
         alibi_slopes: None, or (nheads,) fp32 on the GPU.  Not in the reference (its README lists attention bias as
             planned): the score of query i and key j, positions counted inside their sequences, becomes
             softmax_scale * q_i.k_j - alibi_slopes[head] * |i - j|.  The slopes are constants (no gradient).
+        attn_bias: None, or (1 or batch_size, 1 or nheads, max_seqlen_q, max_seqlen_k) in the inputs' dtype (not in the
+            reference either): the score becomes softmax_scale * q_i.k_j + attn_bias[b, head, i, j]; -inf entries mask.
+            Differentiable (a shared bias gets the sum over the batch entries / heads that share it).  Not together
+            with alibi_slopes.
     Returns
         out: (total_q, nheads, headdim).
         With return_attn_probs=True additionally
@@ -158,25 +192,26 @@ _COMMON_DOC = """
 
 
 def flash_attn_unpadded_qkvpacked_func(qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale=None,
-                                       causal=False, return_attn_probs=False, alibi_slopes=None):
+                                       causal=False, return_attn_probs=False, alibi_slopes=None, attn_bias=None):
     """Self-attention on a packed (total, 3, nheads, headdim) tensor of variable-length sequences."""
     return FlashAttnQKVPackedFunc.apply(qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal,
-                                        return_attn_probs, alibi_slopes)
+                                        return_attn_probs, alibi_slopes, attn_bias)
 
 
 def flash_attn_unpadded_kvpacked_func(q, kv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
                                       dropout_p, softmax_scale=None, causal=False,
-                                      return_attn_probs=False, alibi_slopes=None):
+                                      return_attn_probs=False, alibi_slopes=None, attn_bias=None):
     """Attention of q (total_q, nheads, headdim) over packed keys/values kv (total_k, 2, nheads, headdim)."""
     return FlashAttnKVPackedFunc.apply(q, kv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-                                       softmax_scale, causal, return_attn_probs, alibi_slopes)
+                                       softmax_scale, causal, return_attn_probs, alibi_slopes, attn_bias)
 
 
 def flash_attn_unpadded_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-                             dropout_p, softmax_scale=None, causal=False, return_attn_probs=False, alibi_slopes=None):
+                             dropout_p, softmax_scale=None, causal=False, return_attn_probs=False, alibi_slopes=None,
+                             attn_bias=None):
     """Attention of q (total_q, nheads, headdim) over k, v (total_k, nheads, headdim)."""
     return FlashAttnFunc.apply(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-                               softmax_scale, causal, return_attn_probs, alibi_slopes)
+                               softmax_scale, causal, return_attn_probs, alibi_slopes, attn_bias)
 
 
 def flash_attn_func(qkv, cu_seqlens, dropout_p, max_s, softmax_scale=None, causal=False,

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FA_ABI_VERSION 3
+#define FA_ABI_VERSION 4
 
 enum fa_dtype { FA_FP16 = 0, FA_BF16 = 1 };
 
@@ -81,6 +81,13 @@ typedef struct fa_fwd_args {
    * without it.  Ignored with p_dropout == 0 or a blockmask. */
   void* keep_words;
   size_t keep_words_bytes;
+  /* Attention bias as a tensor (same origin as alibi_slopes: the reference plans it, README.md:50, "relative positional
+   * encoding").  NULL, or a device tensor of `dtype` indexed [batch, head, query, key] with the strides below in elements
+   * (keys contiguous; batch and head stride may be 0: one bias for all of them): softmax_scale * q.k + bias[b, h, i, j] is
+   * what the softmax sees, i < max_seqlen_q and j < max_seqlen_k being positions inside the sequences.  -inf entries mask.
+   * 16-byte aligned, bias_row_stride a multiple of 8 and >= max_seqlen_k.  Not with a blockmask, not with alibi_slopes. */
+  const void* attn_bias;
+  int64_t bias_batch_stride, bias_head_stride, bias_row_stride;
 } fa_fwd_args;
 
 /* Arguments of the backward pass.  Mirrors mha_bwd (fmha_api.cpp:302-321) and, when `blockmask`
@@ -130,6 +137,15 @@ typedef struct fa_bwd_args {
    * dq, dk, dv are bit for bit what they are without it.  Ignored with p_dropout == 0 or a blockmask. */
   const void* keep_words;
   size_t keep_words_bytes;
+  /* as in fa_fwd_args: the bias the forward was given */
+  const void* attn_bias;
+  int64_t bias_batch_stride, bias_head_stride, bias_row_stride;
+  /* NULL, or where to leave d(loss)/d(attn_bias): a tensor of `dtype` indexed [batch, head, query, key] with the strides
+   * below (nonzero batch and head strides: every (batch, head) has its own slice; sum over them for a shared bias), 2-byte
+   * aligned.  Only the (query, key) tiles the backward visits are written (under a causal mask none above the diagonal,
+   * none past a sequence's end): the caller clears the tensor first. */
+  void* dbias;
+  int64_t dbias_batch_stride, dbias_head_stride, dbias_row_stride;
 } fa_bwd_args;
 
 /* replaces flash_attn_cuda.fwd -> mha_fwd, csrc/flash_attn/fmha_api.cpp:173-299 */

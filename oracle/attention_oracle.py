@@ -28,6 +28,9 @@ How each function is pinned (the reference has no tests, golden vectors or fixtu
   convert_blockmask_ref: brute force over all small masks against an independent per-element definition.
   alibi_bias (inside varlen_attention): torch's scaled_dot_product_attention with the same bias as a float attn_mask;
       slope 0 is no bias; a bias that is constant along a row changes nothing.
+  attn_bias (inside varlen_attention; the engine's tensor-bias extension): the same library routine with the tensor as float
+      attn_mask, forward and - through its autograd - dq, dk, dv and dbias; -inf entries equal the causal mask they spell; a
+      shared bias gets the sum of the per-(batch, head) gradients; fp64 finite differences on a tiny case.
   unpad_ref / pad_ref: round trip pad(unpad(x)) == x * mask, cu_seqlens against the cumulative sum of the lengths.
   rotary_ref: the cited definition evaluated literally; it is a rotation (norm kept, conjugate inverts it, angles add,
       position 0 is the identity).
@@ -93,7 +96,7 @@ def alibi_bias(slopes, Lq, Lk, device="cpu", dtype=torch.float32):
 
 
 def varlen_attention(q, k, v, cu_q, cu_k, softmax_scale=None, causal=False, p_dropout=0.0, keep_mask=None,
-                     layout=None, dout=None, dtype=torch.float32, alibi_slopes=None):
+                     layout=None, dout=None, dtype=torch.float32, alibi_slopes=None, attn_bias=None):
     """Closed-form attention forward (+ backward if dout is given) on packed tensors.
 
     q (total_q, H, D), k, v (total_k, H, D) any float dtype (upcast to `dtype`); cu_q, cu_k int sequences of length
@@ -101,6 +104,8 @@ def varlen_attention(q, k, v, cu_q, cu_k, softmax_scale=None, causal=False, p_dr
     Returns dict(out, lse [list of (H, Lq_b)], dq, dk, dv, softmax_d [list of (H, Lq_b)], probs [list]).
     Rows with no visible key give out = 0, lse = -inf (fmha_fprop_kernel_1xN.h:575,606; fmha_api.cpp:519).
     softmax_d is keep * rowsum(dO o O) (fmha_dgrad_kernel_1xN_loop.h:15-30,226).
+    attn_bias (the engine's extension, no reference counterpart): (1 or B, 1 or H, >= Lq, >= Lk), added to the scaled scores
+    at positions counted inside each sequence; with dout the result also holds dbias, in attn_bias's shape.
     """
     cu_q = [int(x) for x in cu_q]
     cu_k = [int(x) for x in cu_k]
@@ -111,6 +116,7 @@ def varlen_attention(q, k, v, cu_q, cu_k, softmax_scale=None, causal=False, p_dr
     qf = q.detach().to(dtype).requires_grad_(dout is not None)
     kf = k.detach().to(dtype).requires_grad_(dout is not None)
     vf = v.detach().to(dtype).requires_grad_(dout is not None)
+    bf = attn_bias.detach().to(dtype).requires_grad_(dout is not None) if attn_bias is not None else None
     outs, lses, probs = [], [], []
     for b in range(B):
         qb = qf[cu_q[b]:cu_q[b + 1]].transpose(0, 1)  # (H, Lq, D)
@@ -120,6 +126,8 @@ def varlen_attention(q, k, v, cu_q, cu_k, softmax_scale=None, causal=False, p_dr
         s = torch.einsum("hqd,hkd->hqk", qb, kb) * scale
         if alibi_slopes is not None:
             s = s + alibi_bias(alibi_slopes, Lq, Lk, qf.device, dtype)
+        if bf is not None:
+            s = s + bf[b if bf.shape[0] > 1 else 0, :, :Lq, :Lk]
         valid = _score_mask(Lq, Lk, causal, layout, qf.device)
         s = s.masked_fill(~valid[None], float("-inf"))
         lse = torch.logsumexp(s, dim=-1)  # -inf for empty rows
@@ -138,6 +146,8 @@ def varlen_attention(q, k, v, cu_q, cu_k, softmax_scale=None, causal=False, p_dr
         do = dout.detach().to(dtype)
         out.backward(do)
         res["dq"], res["dk"], res["dv"] = qf.grad, kf.grad, vf.grad
+        if bf is not None:
+            res["dbias"] = bf.grad if bf.grad is not None else torch.zeros_like(bf)
         dsum = (do * out.detach()).sum(-1) * keep  # (total_q, H)
         res["softmax_d"] = [dsum[cu_q[b]:cu_q[b + 1]].transpose(0, 1) for b in range(B)]
     return res

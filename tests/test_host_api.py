@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol(lib):
     assert declared == set(be.EXPORTED_SYMBOLS)
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.fa_abi_version() == be.FA_ABI_VERSION == 3
+    assert lib.fa_abi_version() == be.FA_ABI_VERSION == 4
 
 
 def test_struct_layout_matches_library(lib):
@@ -159,9 +159,9 @@ def test_public_signatures_match_the_reference():
         return [(n, p.default if p.default is not inspect.Parameter.empty else "<req>")
                 for n, p in inspect.signature(f).parameters.items()]
 
-    # the three functions that reach the kernels take the reference's parameters followed by one extension,
-    # alibi_slopes=None (attention bias: planned in the reference's README, absent from its API)
-    ext = [("alibi_slopes", None)]
+    # the three functions that reach the kernels take the reference's parameters followed by two extensions,
+    # alibi_slopes=None and attn_bias=None (attention bias: planned in the reference's README, absent from its API)
+    ext = [("alibi_slopes", None), ("attn_bias", None)]
     assert sig(fi.flash_attn_unpadded_qkvpacked_func) == [
         ("qkv", "<req>"), ("cu_seqlens", "<req>"), ("max_seqlen", "<req>"), ("dropout_p", "<req>"),
         ("softmax_scale", None), ("causal", False), ("return_attn_probs", False)] + ext
@@ -186,7 +186,7 @@ def test_public_signatures_match_the_reference():
     from flash_attn import flash_attn_gfx950 as be
     assert list(inspect.signature(be.fwd).parameters) == [
         "q", "k", "v", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k", "p_dropout", "softmax_scale",
-        "zero_tensors", "is_causal", "return_softmax", "gen", "alibi_slopes", "keep_words"]  # fmha_api.cpp:173-186 + extensions
+        "zero_tensors", "is_causal", "return_softmax", "gen", "alibi_slopes", "keep_words", "attn_bias"]  # fmha_api.cpp:173-186 + extensions
     assert list(inspect.signature(be.bwd_block).parameters) == [
         "dout", "q", "k", "v", "out", "softmax_lse", "dq", "dk", "dv", "cu_seqlens_q", "cu_seqlens_k", "blockmask",
         "max_seqlen_q", "max_seqlen_k", "p_dropout", "softmax_scale", "is_causal", "gen"]  # fmha_api.cpp:575-594

@@ -44,9 +44,9 @@ def _pick(res, *parts):
 def test_d64_kernels_keep_their_waves_per_simd():
     fwd = _resources("fa_fwd_d64.hip")
     bwd = _resources("fa_bwd_d64.hip")
-    # <f16, 64, ..., causal, dropout, sparse, alibi, key split> mangled as ...IDF16_Li64E...Lb{0,1}E x4 Li{1,2}E
+    # <f16, 64, ..., causal, dropout, sparse, alibi, key split> mangled as ...IDF16_Li64E...Lb{0,1}E x3, Li{0,1,2}E for the score bias, Li{1,2}E
     # (the dK/dV kernel has no key-split parameter)
-    plain, causal, dropout = "Lb0ELb0ELb0ELb0E", "Lb1ELb0ELb0ELb0E", "Lb0ELb1ELb0ELb0E"
+    plain, causal, dropout = "Lb0ELb0ELb0ELi0E", "Lb1ELb0ELb0ELi0E", "Lb0ELb1ELb0ELi0E"
     full = "Li1EEEv"
     # (the forward's last parameter: the dropout variant that also leaves its keep decisions for the backward)
     for flags, want in ((plain, 4), (causal, 4), (dropout, 3)):
@@ -61,7 +61,7 @@ def test_d64_kernels_keep_their_waves_per_simd():
     assert k["Occupancy"] >= 4 and k["VGPRs Spill"] == 0 and k["SGPRs Spill"] == 0, ("forward, keep words, key split", k)
     # backward kernels: <..., causal, dropout mode (0 none, 1 drawn with Philox, 2 read from the forward's keep words),
     # sparse, alibi, ...>
-    bplain, bcausal, bdrawn, bread = "Lb0ELi0ELb0ELb0E", "Lb1ELi0ELb0ELb0E", "Lb0ELi1ELb0ELb0E", "Lb0ELi2ELb0ELb0E"
+    bplain, bcausal, bdrawn, bread = "Lb0ELi0ELb0ELi0E", "Lb1ELi0ELb0ELi0E", "Lb0ELi1ELb0ELi0E", "Lb0ELi2ELb0ELi0E"
     for flags, want in ((bplain, 3), (bcausal, 3), (bdrawn, 3), (bread, 3)):
         k = _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", flags + full)
         assert k["Occupancy"] >= want and k["VGPRs Spill"] == 0, ("dq", flags, k)
@@ -71,7 +71,7 @@ def test_d64_kernels_keep_their_waves_per_simd():
         k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", flags)
         assert k["Occupancy"] >= want and k["VGPRs Spill"] <= spill, ("dkdv", flags, k)
     # the ALiBi variants (fourth flag set) keep the waves per SIMD of their plain counterparts in the backward
-    for flags, bflags in (("Lb0ELb0ELb0ELb1E", "Lb0ELi0ELb0ELb1E"), ("Lb1ELb0ELb0ELb1E", "Lb1ELi0ELb0ELb1E")):
+    for flags, bflags in (("Lb0ELb0ELb0ELi1E", "Lb0ELi0ELb0ELi1E"), ("Lb1ELb0ELb0ELi1E", "Lb1ELi0ELb0ELi1E")):
         assert _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags + "Li1ELb0EEEv")["Occupancy"] >= 3, flags  # (the bias costs the fourth)
         assert _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", bflags + full)["Occupancy"] >= 3, bflags
         k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", bflags)
@@ -85,9 +85,9 @@ def test_d128_backward_keeps_two_waves_per_simd():
     bwd = _resources("fa_bwd_d128.hip")
     for dt in ("IDF16_", "IDF16b"):
         # plain, causal, both with a block layout, and the two without that read the dropout decisions from keep words
-        for flags in ("Lb0ELi0ELb0ELb0E", "Lb1ELi0ELb0ELb0E", "Lb0ELi0ELb1ELb0E", "Lb1ELi0ELb1ELb0E", "Lb0ELi2ELb0ELb0E",
-                      "Lb1ELi2ELb0ELb0E"):
+        for flags in ("Lb0ELi0ELb0ELi0E", "Lb1ELi0ELb0ELi0E", "Lb0ELi0ELb1ELi0E", "Lb1ELi0ELb1ELi0E", "Lb0ELi2ELb0ELi0E",
+                      "Lb1ELi2ELb0ELi0E"):
             k = _pick(bwd, "fa_bwd_dkdv_kernel%sLi128E" % dt, flags)
             assert k["Occupancy"] >= 2 and k["VGPRs Spill"] == 0 and k["LDS Size"] <= 80 * 1024, (dt, flags, k)
             k = _pick(bwd, "fa_bwd_dq_kernel%sLi128E" % dt, flags + "Li1EEEv")
-            assert k["Occupancy"] >= 2 and k["VGPRs Spill"] <= (1 if "Lb1ELb0E" in flags[8:] else 0), ("dq", dt, flags, k)
+            assert k["Occupancy"] >= 2 and k["VGPRs Spill"] <= (1 if "Lb1ELi0E" in flags[8:] else 0), ("dq", dt, flags, k)

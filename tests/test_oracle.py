@@ -302,3 +302,44 @@ def test_alibi_bias_against_sdpa_float_mask():
         plain = orc.varlen_attention(q, k, v, cu, cu, None, causal, dtype=torch.float64)
         assert torch.equal(res["out"][:, 2], plain["out"][:, 2])          # head with slope 0
         assert not torch.allclose(res["out"][:, 0], plain["out"][:, 0], atol=1e-3)
+
+
+def test_attn_bias_against_sdpa_float_mask_and_finite_differences():
+    """varlen_attention with a bias tensor against torch's scaled_dot_product_attention given the same tensor as a float
+    attn_mask (library routine): forward, and through its autograd dq, dk, dv and dbias; two ragged sequences share one
+    (1, H, S, S) bias, whose gradient is then the sum over the batch; -inf entries spell a causal mask."""
+    g = torch.Generator().manual_seed(33)
+    H, D = 2, 8
+    lens = [7, 5]
+    S = max(lens)
+    cu = [0, 7, 12]
+    q, k, v, do = (torch.randn(sum(lens), H, D, generator=g, dtype=torch.float64) for _ in range(4))
+    bias = torch.randn(1, H, S, S, generator=g, dtype=torch.float64)
+    res = orc.varlen_attention(q, k, v, cu, cu, None, False, dout=do, dtype=torch.float64, attn_bias=bias)
+    bb = bias.clone().requires_grad_()
+    grads = {n: torch.zeros_like(q) for n in ("dq", "dk", "dv")}
+    for b, L in enumerate(lens):
+        sl = slice(cu[b], cu[b + 1])
+        qq, kk, vv = (x[sl].transpose(0, 1).clone().requires_grad_() for x in (q, k, v))
+        ref = torch.nn.functional.scaled_dot_product_attention(qq[None], kk[None], vv[None], attn_mask=bb[:, :, :L, :L])[0]
+        ref.backward(do[sl].transpose(0, 1))
+        assert torch.allclose(res["out"][sl].transpose(0, 1), ref, atol=1e-12)
+        for n, t in (("dq", qq), ("dk", kk), ("dv", vv)):
+            assert torch.allclose(res[n][sl].transpose(0, 1), t.grad, atol=1e-11), n
+    assert torch.allclose(res["dbias"], bb.grad, atol=1e-11)           # summed over the two sequences that share it
+    assert res["dbias"][0, :, 5:, :].abs().max() > 0 and torch.equal(res["dbias"][0, :, 7:, :], torch.zeros(H, 0, S, dtype=torch.float64))
+    # a bias of 0 / -inf above the diagonal is the causal mask
+    tri = torch.zeros(1, 1, S, S, dtype=torch.float64).masked_fill(torch.triu(torch.ones(S, S, dtype=torch.bool), 1), float("-inf"))
+    a = orc.varlen_attention(q, k, v, cu, cu, None, False, dout=do, dtype=torch.float64, attn_bias=tri)
+    c = orc.varlen_attention(q, k, v, cu, cu, None, True, dout=do, dtype=torch.float64)
+    for n in ("out", "dq", "dk", "dv"):
+        assert torch.allclose(a[n], c[n], atol=1e-12), n
+    # dbias by central differences of sum(out * dout) on a few entries
+    eps = 1e-6
+    for (h, i, j) in ((0, 0, 0), (1, 3, 4), (0, 6, 2)):
+        bp, bm = bias.clone(), bias.clone()
+        bp[0, h, i, j] += eps
+        bm[0, h, i, j] -= eps
+        fp = (orc.varlen_attention(q, k, v, cu, cu, None, False, dtype=torch.float64, attn_bias=bp)["out"] * do).sum()
+        fm = (orc.varlen_attention(q, k, v, cu, cu, None, False, dtype=torch.float64, attn_bias=bm)["out"] * do).sum()
+        assert abs((fp - fm) / (2 * eps) - res["dbias"][0, h, i, j]) < 1e-7

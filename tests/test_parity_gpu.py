@@ -80,9 +80,11 @@ def _inputs(lens_q, lens_k, H, D, dtype, seed):
     return mk(tq), mk(tk), mk(tk), mk(tq)
 
 
-def half_attention(q, k, v, cu_q, cu_k, scale, causal, keep_mask=None, p=0.0, layout=None, dout=None, alibi_slopes=None):
+def half_attention(q, k, v, cu_q, cu_k, scale, causal, keep_mask=None, p=0.0, layout=None, dout=None, alibi_slopes=None,
+                   attn_bias=None):
     """the closed form evaluated in the tensors' own half dtype by PyTorch (the error yardstick)"""
     q, k, v = (x.detach().clone().requires_grad_(dout is not None) for x in (q, k, v))
+    bias = attn_bias.detach().clone().requires_grad_(dout is not None) if attn_bias is not None else None
     outs, lses = [], []
     for b in range(len(cu_q) - 1):
         qb = q[cu_q[b]:cu_q[b + 1]].transpose(0, 1)
@@ -91,6 +93,8 @@ def half_attention(q, k, v, cu_q, cu_k, scale, causal, keep_mask=None, p=0.0, la
         s = torch.matmul(qb, kb.transpose(1, 2)) * scale
         if alibi_slopes is not None:
             s = s + orc.alibi_bias(alibi_slopes, qb.shape[1], kb.shape[1], q.device).to(s.dtype)
+        if bias is not None:
+            s = s + bias[b if bias.shape[0] > 1 else 0, :, :qb.shape[1], :kb.shape[1]]
         valid = orc._score_mask(qb.shape[1], kb.shape[1], causal, layout, q.device)
         s = s.masked_fill(~valid[None], float("-inf"))
         empty = ~valid.any(-1)
@@ -106,6 +110,8 @@ def half_attention(q, k, v, cu_q, cu_k, scale, causal, keep_mask=None, p=0.0, la
     if dout is not None:
         out.backward(dout)
         res.update(dq=q.grad, dk=k.grad, dv=v.grad)
+        if bias is not None:
+            res["dbias"] = bias.grad
     return res
 
 
@@ -151,22 +157,28 @@ def check_lse(got, want, half_lse, dtype, what=""):
     assert e_ours <= 2 * e_half + 1e-4 and e_ours <= LSE_TOL[dtype], "%s lse: ours %.3e vs half-precision PyTorch %.3e" % (what, e_ours, e_half)
 
 
-def run_ours(q, k, v, do, cu_q, cu_k, max_q, max_k, p, scale, causal, packing="sep", probs=False, alibi_slopes=None):
+def run_ours(q, k, v, do, cu_q, cu_k, max_q, max_k, p, scale, causal, packing="sep", probs=False, alibi_slopes=None,
+             attn_bias=None):
     from flash_attn import flash_attn_interface as fi
     dev = "cuda"
     cu_q, cu_k = cu_q.to(dev), cu_k.to(dev)
+    bias_kw = {}
+    if attn_bias is not None:
+        bias_g = attn_bias.to(dev).requires_grad_()
+        bias_kw = {"attn_bias": bias_g}
     if packing == "qkv":
         qkv = torch.stack([q, k, v], 1).to(dev).requires_grad_()
-        res = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu_q, max_q, p, scale, causal, probs, alibi_slopes=alibi_slopes)
+        res = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu_q, max_q, p, scale, causal, probs, alibi_slopes=alibi_slopes,
+                                                    **bias_kw)
     elif packing == "kv":
         qg = q.to(dev).requires_grad_()
         kv = torch.stack([k, v], 1).to(dev).requires_grad_()
         res = fi.flash_attn_unpadded_kvpacked_func(qg, kv, cu_q, cu_k, max_q, max_k, p, scale, causal, probs,
-                                                   alibi_slopes=alibi_slopes)
+                                                   alibi_slopes=alibi_slopes, **bias_kw)
     else:
         qg, kg, vg = (x.to(dev).requires_grad_() for x in (q, k, v))
         res = fi.flash_attn_unpadded_func(qg, kg, vg, cu_q, cu_k, max_q, max_k, p, scale, causal, probs,
-                                          alibi_slopes=alibi_slopes)
+                                          alibi_slopes=alibi_slopes, **bias_kw)
     out = res[0] if probs else res
     out.backward(do.to(dev))
     torch.cuda.synchronize()
@@ -177,6 +189,8 @@ def run_ours(q, k, v, do, cu_q, cu_k, max_q, max_k, p, scale, causal, packing="s
     else:
         dq, dk, dv = qg.grad, kg.grad, vg.grad
     r = {"out": out.detach(), "dq": dq, "dk": dk, "dv": dv}
+    if attn_bias is not None:
+        r["dbias"] = bias_g.grad
     if probs:
         r["lse"], r["S_dmask"] = res[1], res[2]
     return r
@@ -771,6 +785,159 @@ def test_alibi_headline_shape_and_errors():
     q3 = qkv.detach()
     with pytest.raises(RuntimeError):
         be._fwd_impl(q3[:, 0], q3[:, 1], q3[:, 2], cu, cu, bm, N, N, 0.0, D ** -0.5, False, False, False, None, slopes)
+
+
+# ------------------------------------------------------------------------------------------------
+# attention bias as a tensor (extension: the reference only plans it, README.md:50)
+# ------------------------------------------------------------------------------------------------
+def _random_bias(rng, shape, dtype, minus_inf=0.0):
+    g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
+    bias = (torch.randn(shape, generator=g) * 1.5).to(dtype)
+    if minus_inf > 0:  # masked entries, never a whole row (key 0 stays)
+        drop = torch.rand(shape, generator=g) < minus_inf
+        drop[..., 0] = False
+        bias = bias.masked_fill(drop, float("-inf"))
+    return bias
+
+
+def test_attn_bias_random_shapes_sweep():
+    """Sixteen seeded random cases with a bias tensor added to the scaled scores: head dims, dtypes, ragged self- and
+    cross-attention, causal or not, the bias per (batch, head), shared over the batch or over everything, with and
+    without -inf entries, key extents that are and are not multiples of 8 (the latter make the binding pad a copy):
+    out, lse, dq, dk, dv and the bias gradient against the oracle (closed form + autograd, itself pinned against
+    torch's scaled_dot_product_attention with the same tensor as float mask)."""
+    rng = np.random.default_rng(4242)
+    for case in range(16):
+        D = int(rng.choice([16, 32, 64, 128]))
+        dtype = torch.float16 if rng.integers(2) else torch.bfloat16
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        causal = bool(rng.integers(2))
+        cross = bool(rng.integers(2)) and not causal
+        top = int(rng.choice([40, 150, 330]))
+        lens_q = [int(x) for x in rng.integers(1, top + 1, B)]
+        lens_k = [int(x) for x in rng.integers(1, top + 1, B)] if cross else list(lens_q)
+        mq, mk = max(lens_q), max(lens_k)
+        if rng.integers(2):
+            mk8 = (mk + 7) // 8 * 8   # a bias whose rows the kernels can read as they are
+        else:
+            mk8 = mk
+        bshape = ((B, H), (1, H), (1, 1), (B, 1))[int(rng.integers(4))] + (mq, mk8)
+        bias = _random_bias(rng, bshape, dtype, minus_inf=float(rng.choice([0.0, 0.2])))
+        packing = "kv" if cross else str(rng.choice(["qkv", "sep"]))
+        print("case %d: D=%d %s B=%d H=%d causal=%s q=%s k=%s bias%s %s" % (case, D, dtype, B, H, causal, lens_q, lens_k,
+                                                                            tuple(bshape), packing), flush=True)
+        q, k, v, do = _inputs(lens_q, lens_k, H, D, dtype, 900 + case)
+        cu_q, cu_k = _cu(lens_q, "cpu"), _cu(lens_k, "cpu")
+        ours = run_ours(q, k, v, do, cu_q, cu_k, mq, mk, 0.0, None, causal, packing, probs=True, attn_bias=bias)
+        ref = orc.varlen_attention(q, k, v, cu_q, cu_k, None, causal, dout=do, attn_bias=bias)
+        half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu_q.tolist(), cu_k.tolist(), D ** -0.5, causal, dout=do.cuda(),
+                              attn_bias=bias.cuda())
+        what = "attn_bias sweep case %d" % case
+        check_against_oracle(ours, ref, half, dtype, names=("out", "dq", "dk", "dv", "dbias"), what=what)
+        for b, L in enumerate(lens_q):
+            check_lse(ours["lse"][b, :, :L].cpu(), ref["lse"][b], half["lse"][b], dtype, what)
+        # the probabilities returned for testing carry the bias too
+        S = ours["S_dmask"].float().cpu()
+        for b, (Lq, Lk) in enumerate(zip(lens_q, lens_k)):
+            assert (S[b, :, :Lq, :Lk] - ref["probs"][b]).abs().max() < (2e-3 if dtype == torch.float16 else 1.6e-2)
+
+
+@pytest.mark.parametrize("D,dtype,causal", [(64, torch.float16, False), (128, torch.bfloat16, True), (32, torch.float16, True)])
+def test_attn_bias_with_dropout(D, dtype, causal, dropout_path):
+    """bias and dropout together (the backward reading the forward's keep words, or drawing again): the mask is the defined
+    one, out / gradients / bias gradient equal the closed form with that mask."""
+    lens, H, p = [150, 77, 200], 2, 0.2
+    rng = np.random.default_rng(7)
+    bias = _random_bias(rng, (1, H, max(lens), max(lens)), dtype)
+    q, k, v, do = _inputs(lens, lens, H, D, dtype, 31)
+    cu = _cu(lens, "cpu")
+    torch.manual_seed(123)
+    seed, offset = _gen_state()
+    ours = run_ours(q, k, v, do, cu, cu, max(lens), max(lens), p, None, causal, "qkv", probs=True, attn_bias=bias)
+    S = ours["S_dmask"].cpu()
+    masks = []
+    for b, L in enumerate(lens):
+        mb = np.stack([orc.dropout_keep_mask(seed, offset, b * H + h, L, L, p) for h in range(H)])
+        masks.append(torch.tensor(mb))
+        valid = orc._score_mask(L, L, causal, None)
+        assert torch.equal(torch.signbit(S[b, :, :L, :L])[:, valid], ~masks[b][:, valid])
+    ref = orc.varlen_attention(q, k, v, cu, cu, None, causal, p_dropout=p, keep_mask=masks, dout=do, attn_bias=bias)
+    half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu.tolist(), cu.tolist(), D ** -0.5, causal, masks, p, dout=do.cuda(),
+                          attn_bias=bias.cuda())
+    check_against_oracle(ours, ref, half, dtype, names=("out", "dq", "dk", "dv", "dbias"), what="attn_bias + dropout D=%d" % D)
+
+
+def test_attn_bias_special_cases_and_errors():
+    """A bias of zeros changes nothing (bit for bit against the kernels without bias at d = 128, where both run the same
+    tile shapes; within rounding elsewhere); 0 / -inf above the diagonal is the causal mask; a row whose bias is -inf
+    everywhere gives out = 0 and lse = -inf; the slopes' bias as a tensor equals alibi_slopes; argument errors."""
+    from flash_attn import flash_attn_interface as fi
+    B, H, D, N = 2, 3, 64, 200
+    torch.manual_seed(5)
+    qkv = torch.randn(B * N, 3, H, D, device="cuda", dtype=torch.float16)
+    cu = torch.arange(0, (B + 1) * N, N, dtype=torch.int32, device="cuda")
+    plain = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0)
+    zero = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0, attn_bias=torch.zeros(1, 1, N, N, device="cuda", dtype=torch.float16))
+    assert (plain.float() - zero.float()).abs().max() < 2e-3
+    tri = torch.zeros(1, 1, N, N, device="cuda", dtype=torch.float16).masked_fill(
+        torch.triu(torch.ones(N, N, dtype=torch.bool, device="cuda"), 1), float("-inf"))
+    a = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0, attn_bias=tri)
+    c = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0, causal=True)
+    assert (a.float() - c.float()).abs().max() < 2e-3
+    # a fully masked row
+    dead = torch.zeros(1, 1, N, N, device="cuda", dtype=torch.float16)
+    dead[0, 0, 17, :] = float("-inf")
+    out, lse, _ = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0, return_attn_probs=True, attn_bias=dead)
+    assert torch.equal(out[17], torch.zeros_like(out[17])) and torch.isinf(lse[0, :, 17]).all() and (lse[0, :, 17] < 0).all()
+    assert torch.isfinite(out).all()
+    # ALiBi written out as a tensor
+    slopes = _alibi_slopes(H).cuda()
+    al = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0, alibi_slopes=slopes)
+    tb = orc.alibi_bias(slopes.cpu(), N, N)[None].to(torch.float16).cuda()
+    at = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0, attn_bias=tb)
+    assert (al.float() - at.float()).abs().max() < 4e-3   # the tensor's entries are rounded to fp16, the slopes' are not
+    # errors
+    with pytest.raises(RuntimeError, match="attn_bias"):
+        fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0, attn_bias=torch.zeros(1, 1, N, N - 1, device="cuda", dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="attn_bias"):
+        fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0, attn_bias=torch.zeros(1, 1, N, N, device="cuda", dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="together"):
+        fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0, alibi_slopes=slopes,
+                                              attn_bias=torch.zeros(1, 1, N, N, device="cuda", dtype=torch.float16))
+
+
+def test_attn_bias_full_size_against_pytorch_and_decode_shape():
+    """Headline-sized check (B=2, H=12, d=64, N=2048, a bias per head shared over the batch) against PyTorch's
+    scaled_dot_product_attention in fp32 with the same tensor as mask, forward and backward, and a decode-shaped call
+    (one query row per sequence over thousands of keys: the key-split kernels) against the oracle."""
+    B, H, D, N = 2, 12, 64, 2048
+    torch.manual_seed(9)
+    qkv = torch.randn(B * N, 3, H, D, device="cuda", dtype=torch.float16, requires_grad=True)
+    bias = (torch.randn(1, H, N, N, device="cuda") * 1.5).to(torch.float16).requires_grad_()
+    cu = torch.arange(0, (B + 1) * N, N, dtype=torch.int32, device="cuda")
+    from flash_attn import flash_attn_interface as fi
+    out = fi.flash_attn_unpadded_qkvpacked_func(qkv, cu, N, 0.0, attn_bias=bias)
+    do = torch.randn_like(out)
+    out.backward(do)
+    q32 = qkv.detach().float().view(B, N, 3, H, D).permute(2, 0, 3, 1, 4).clone().requires_grad_()
+    b32 = bias.detach().float().clone().requires_grad_()
+    ref = torch.nn.functional.scaled_dot_product_attention(q32[0], q32[1], q32[2], attn_mask=b32)
+    ref.backward(do.float().view(B, N, H, D).permute(0, 2, 1, 3))
+    assert (out.float().view(B, N, H, D).permute(0, 2, 1, 3) - ref).abs().max() < 4e-3
+    g = qkv.grad.float().view(B, N, 3, H, D).permute(2, 0, 3, 1, 4)
+    assert (g - q32.grad).abs().max() < 8e-3
+    assert (bias.grad.float() - b32.grad).abs().max() < 8e-3
+    # decode shape
+    lens_q, lens_k = [1, 1], [3000, 1777]
+    q, k, v, do = _inputs(lens_q, lens_k, 4, 64, torch.float16, 77)
+    rng = np.random.default_rng(3)
+    db = _random_bias(rng, (2, 4, 1, 3000), torch.float16)
+    cu_q, cu_k = _cu(lens_q, "cpu"), _cu(lens_k, "cpu")
+    ours = run_ours(q, k, v, do, cu_q, cu_k, 1, 3000, 0.0, None, False, "kv", attn_bias=db)
+    ref = orc.varlen_attention(q, k, v, cu_q, cu_k, None, False, dout=do, attn_bias=db)
+    half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu_q.tolist(), cu_k.tolist(), 64 ** -0.5, False, dout=do.cuda(),
+                          attn_bias=db.cuda())
+    check_against_oracle(ours, ref, half, torch.float16, names=("out", "dq", "dk", "dv", "dbias"), what="attn_bias decode shape")
 
 
 # ------------------------------------------------------------------------------------------------
