@@ -22,10 +22,12 @@ class FlashAttention(nn.Module):
         self.dropout_p = attention_dropout
 
     def forward(self, qkv, attn_mask=None, key_padding_mask=None, causal=False, cu_seqlens=None, max_s=None,
-                need_weights=False, alibi_slopes=None):
+                need_weights=False, alibi_slopes=None, attn_bias=None):
         """qkv is (B, S, 3, H, D) when cu_seqlens is None, else already packed (nnz, 3, H, D) with cu_seqlens / max_s.
         key_padding_mask, if given, is an object whose `.bool_matrix` is a (B, S) bool tensor, True = keep.
         alibi_slopes (not in the reference): (H,) fp32 slopes of the in-kernel attention bias -slope * |i - j|.
+        attn_bias (not in the reference): (1 or B, 1 or H, S, S) in qkv's dtype, added to the scaled scores; positions are
+        counted inside each sequence (so with a key_padding_mask, among the tokens that are kept); differentiable.
         Returns (output, None); output has the layout of the input's token dimensions."""
         assert not need_weights
         assert attn_mask is None
@@ -36,7 +38,7 @@ class FlashAttention(nn.Module):
         if cu_seqlens is not None:
             assert max_s is not None
             out = flash_attn_unpadded_qkvpacked_func(qkv, cu_seqlens, max_s, p, softmax_scale=self.softmax_scale,
-                                                     causal=causal, alibi_slopes=alibi_slopes)
+                                                     causal=causal, alibi_slopes=alibi_slopes, attn_bias=attn_bias)
             return out, None
 
         batch, seqlen = qkv.shape[0], qkv.shape[1]
@@ -44,7 +46,7 @@ class FlashAttention(nn.Module):
             packed = qkv.reshape(batch * seqlen, *qkv.shape[2:])
             cu = torch.arange(0, (batch + 1) * seqlen, step=seqlen, dtype=torch.int32, device=qkv.device)
             out = flash_attn_unpadded_qkvpacked_func(packed, cu, seqlen, p, softmax_scale=self.softmax_scale,
-                                                     causal=causal, alibi_slopes=alibi_slopes)
+                                                     causal=causal, alibi_slopes=alibi_slopes, attn_bias=attn_bias)
             return out.reshape(batch, seqlen, *out.shape[1:]), None
 
         nheads, headdim = qkv.shape[-2], qkv.shape[-1]
@@ -52,7 +54,7 @@ class FlashAttention(nn.Module):
         x_unpad, indices, cu, max_len = unpad_input(x, key_padding_mask.bool_matrix)
         out_unpad = flash_attn_unpadded_qkvpacked_func(x_unpad.reshape(-1, 3, nheads, headdim), cu, max_len, p,
                                                        softmax_scale=self.softmax_scale, causal=causal,
-                                                       alibi_slopes=alibi_slopes)
+                                                       alibi_slopes=alibi_slopes, attn_bias=attn_bias)
         out = pad_input(out_unpad.reshape(-1, nheads * headdim), indices, batch, seqlen)
         return out.reshape(batch, seqlen, nheads, headdim), None
 

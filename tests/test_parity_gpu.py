@@ -1133,6 +1133,13 @@ def test_flash_attention_module_three_input_modes():
         L = int(lens[b])
         r = orc.varlen_attention(qkv[b, :L, 0], qkv[b, :L, 1], qkv[b, :L, 2], [0, L], [0, L], None, True, alibi_slopes=slopes)
         assert (out_al[b, :L].float().cpu() - r["out"]).abs().max() < 2e-3
+    # a bias tensor through the module (shared over the batch, per head; padded input: positions inside each sequence)
+    tb = (torch.randn(1, H, S, S, generator=g) * 1.5).half()
+    out_tb, _ = m(qkv.cuda(), key_padding_mask=KPM(), attn_bias=tb.cuda())
+    for b in range(B):
+        L = int(lens[b])
+        r = orc.varlen_attention(qkv[b, :L, 0], qkv[b, :L, 1], qkv[b, :L, 2], [0, L], [0, L], None, False, attn_bias=tb)
+        assert (out_tb[b, :L].float().cpu() - r["out"]).abs().max() < 2e-3
     ref = orc.attention_ref(qkv, mask, 0.0, upcast=True, causal=True).float()
     out_pad, _ = m(qkv.cuda(), key_padding_mask=KPM(), causal=True)
     assert tuple(out_pad.shape) == (B, S, H, D)
