@@ -493,7 +493,9 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
   constexpr int BM = Cfg::BM, DV = Cfg::DV, CH = Cfg::CH, kBufBytes = Cfg::kBufBytes, KBW = Cfg::KBW;
   static_assert(KS == 1 || !kSparse, "the block-sparse maps are built for 128-row query tiles");
 
-  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
+  // kTensorBias: behind the tiles, per wave 32 rows x BN keys of bias, rows padded by 8 bytes (as in fa_fwd_kernel)
+  constexpr int kBiasRowBytes = BN * 2 + 8, kBiasWaveBytes = 32 * kBiasRowBytes;
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes + (kBias == kBiasTensor ? 4 * kBiasWaveBytes : 0)];
 
   int bh, rank;
   const int n_splits = p.n_splits > 1 ? p.n_splits : 1;  // key splits per query tile (see BwdParams)
@@ -602,11 +604,26 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
 
   const float cs = p.scale_log2;
   const float sl2 = kAlibi ? p.alibi[h] * kLog2e : 0.f;  // ALiBi slope in base-2 exponent units (see fa_fwd_kernel)
-  // kTensorBias: this lane's row of the bias (rows past the end read the last row, like Q)
-  const T* const bias_row =
-      kTensorBias ? reinterpret_cast<const T*>(p.bias) + (int64_t)b * p.bias_bs + (int64_t)h * p.bias_hs +
-                        (int64_t)(qrow < Lq ? qrow : Lq - 1) * p.bias_rs
-                  : nullptr;
+  // kTensorBias: as in the forward kernel - whole rows of the wave's 32 x BN bias values fetched 16 bytes a lane one tile ahead,
+  // turned into the MFMA layout through a wave-private piece of LDS
+  constexpr int kBiasCPR = BN / 8, kBiasRPI = 64 / kBiasCPR, kBiasNLD = 32 / kBiasRPI;
+  const T* const bias_bh =
+      kTensorBias ? reinterpret_cast<const T*>(p.bias) + (int64_t)b * p.bias_bs + (int64_t)h * p.bias_hs : nullptr;
+  unsigned char* const bias_lds = lds_raw + Cfg::kLdsBytes + wave * kBiasWaveBytes;
+  u32x4 braw[kTensorBias ? kBiasNLD : 1];
+  auto load_bias = [&](int tile) {
+#pragma unroll
+    for (int i = 0; i < kBiasNLD; i++) {
+      const int row = mw + i * kBiasRPI + lane / kBiasCPR, k0 = tile * BN + (lane % kBiasCPR) * 8;
+      braw[i] = u32x4{0, 0, 0, 0};
+      if (k0 < Lk) braw[i] = ld_global16(bias_bh + (uint32_t)(row < Lq ? row : Lq - 1) * (uint32_t)p.bias_rs + (uint32_t)k0);
+    }
+  };
+  auto bias_to_lds = [&]() {
+#pragma unroll
+    for (int i = 0; i < kBiasNLD; i++)
+      *reinterpret_cast<u32x4*>(bias_lds + (i * kBiasRPI + lane / kBiasCPR) * kBiasRowBytes + (lane % kBiasCPR) * 16) = braw[i];
+  };
   // element offsets inside a tile: row fragments of K (dual swizzle) and V, transposed reads of K (rows +0, +8)
   int kfoff[D / 16], vfoff[D / 16], tlo[DV / 32], thi[DV / 32];
 #pragma unroll
@@ -623,7 +640,10 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
 
   int it = next_active(tile0);
   bool row_on_cur = row_on_next;
-  if (it < ntiles) stage(it, 0);
+  if (it < ntiles) {
+    stage(it, 0);
+    if (kTensorBias) load_bias(it);
+  }
   // ---- now the fragments: rows past the end are zero; Dk and -Dk, lse in base-2 units (+inf switches a row off)
   {
     float dsum = 0.f;
@@ -656,6 +676,10 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
     __syncthreads();  // so is everyone else's, and nobody still reads the other buffer
     const int it_next = next_active(it + 1);
     if (it_next < ntiles) stage(it_next, buf ^ 1);
+    if (kTensorBias) {
+      bias_to_lds();
+      if (it_next < ntiles) load_bias(it_next);
+    }
     const T* const Ks = reinterpret_cast<const T*>(lds_raw + buf * kBufBytes);
     const T* const Vs = Ks + BN * D;
     buf ^= 1;
@@ -681,15 +705,11 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
         f32x16 s, dp = negd;
 #pragma unroll
         for (int r = 0; r < 16; r++) s[r] = 0.f;
-        // kTensorBias: as in the forward kernel - 4 x 4 consecutive values per 32-key block, groups past the last key not read
-        typename E::vec4 bv[4];
+        typename E::vec4 bv[4];  // kTensorBias: the lane's 4 x 4 consecutive values of this 32-key block
         if (kTensorBias) {
 #pragma unroll
-          for (int j = 0; j < 4; j++) {
-            const int k0 = n0 + kb * 32 + 8 * j + 4 * hf;
-            bv[j] = typename E::vec4{0, 0, 0, 0};
-            if (k0 < Lk) bv[j] = *reinterpret_cast<const typename E::vec4*>(bias_row + k0);
-          }
+          for (int j = 0; j < 4; j++)
+            bv[j] = *reinterpret_cast<const typename E::vec4*>(bias_lds + c * kBiasRowBytes + (kb * 32 + 8 * j + 4 * hf) * 2);
         }
 #pragma unroll
         for (int ks = 0; ks < D / 16; ks++) {
@@ -721,7 +741,11 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
             e = kCausal ? __builtin_fmaf(cr, sl2, __builtin_fmaf(dbase, sl2, -lse_t))
                         : __builtin_fmaf(__builtin_fabsf(dbase + cr), -sl2, -lse_t);
           }
-          if (kTensorBias) e = (s[r] == -INFINITY) ? 0.f : __builtin_fmaf((float)bv[r >> 2][r & 3], kLog2e, -lse_t);
+          if (kTensorBias) {  // (past the last key the caller's rows may hold anything: +inf and NaN are cut off there)
+            float bf = (float)bv[r >> 2][r & 3];
+            if (need_mask) bf = fminf(bf, 3.0e38f);
+            e = __builtin_fmaf(bf, kLog2e, -lse_t);
+          }
           const float pe = fast_exp2(__builtin_fmaf(s[r], cs, e));  // 0 for dead scores and switched-off rows
           float dpe = kInitNegD ? dp[r] : dp[r] - dkv;  // dP - Dk
           if (kDropout && !keep.keep_row(r, p.keep_thr)) dpe = -dkv;

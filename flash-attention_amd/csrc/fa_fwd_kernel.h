@@ -51,7 +51,7 @@ struct FwdCfg {
 // kWords (dropout, dense): the keep decisions are also left in p.keep_words for the backward (fa_common.h)
 template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, int kBias = 0, int KS = 1,
           bool kWords = false>
-__global__ void __launch_bounds__(256, (!kDropout && kBias == 0 && D <= 64) ? 4 : 2) fa_fwd_kernel(const FwdParams p) {
+__global__ void __launch_bounds__(256, (!kDropout && kBias == 0 && D <= 64) ? 4 : ((!kDropout && kBias == kBiasTensor && D <= 64) ? 3 : 2)) fa_fwd_kernel(const FwdParams p) {
   constexpr bool kAlibi = kBias == kBiasAlibi, kTensorBias = kBias == kBiasTensor;
   static_assert(!kWords || (kDropout && !kSparse), "keep words: dense dropout variants only");
   static_assert(kBias == 0 || !kSparse, "score bias: dense variants only");
@@ -61,7 +61,9 @@ __global__ void __launch_bounds__(256, (!kDropout && kBias == 0 && D <= 64) ? 4 
   constexpr int BM = Cfg::BM, DV = Cfg::DV, CH = Cfg::CH, kBufBytes = Cfg::kBufBytes, KBW = Cfg::KBW;
   static_assert(KS == 1 || !kSparse, "the block-sparse maps are built for 128-row query tiles");
 
-  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
+  // kTensorBias: behind the tiles, per wave 32 rows x BN keys of bias, rows padded by 8 bytes (see load_bias below)
+  constexpr int kBiasRowBytes = BN * 2 + 8, kBiasWaveBytes = 32 * kBiasRowBytes;
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes + (kTensorBias ? 4 * kBiasWaveBytes : 0)];
 
   // Workgroup -> (batch, head, query tile), XCD-aware (see map_tile): the query tiles of one (batch, head) share
   // one XCD's L2 copy of K and V.
@@ -150,11 +152,30 @@ __global__ void __launch_bounds__(256, (!kDropout && kBias == 0 && D <= 64) ? 4 
   const float cs = p.scale_log2;
   const float cse = kBias != 0 ? 1.f : cs;                       // units of the scores the softmax works on
   const float sl2 = kAlibi ? p.alibi[h] * kLog2e : 0.f;          // slope in base-2 exponent units
-  // kTensorBias: this lane's row of the bias (rows past the end read the last row, like Q)
-  const T* const bias_row =
-      kTensorBias ? reinterpret_cast<const T*>(p.bias) + (int64_t)b * p.bias_bs + (int64_t)h * p.bias_hs +
-                        (int64_t)(qrow < Lq ? qrow : Lq - 1) * p.bias_rs
-                  : nullptr;
+  // kTensorBias: the wave's 32 rows x BN keys of the bias come in as whole rows - BN / 8 lanes fetch the BN * 2 contiguous
+  // bytes of one row, 16 bytes each, so that an instruction touches 8 (16) rows and not 32: read lane by lane in the MFMA
+  // layout (every lane another row) the requests, one per row and instruction, took as long as the whole kernel without a
+  // bias - and are turned into that layout through LDS (wave-private, rows padded by 8 bytes: 32 lanes reading 8 bytes at the
+  // same column of 32 rows hit 32 distinct bank pairs).  Asked for one tile ahead; chunks that begin past the last key are
+  // not read, rows past the end read the last row (like Q).
+  constexpr int kBiasCPR = BN / 8, kBiasRPI = 64 / kBiasCPR, kBiasNLD = 32 / kBiasRPI;
+  const T* const bias_bh =
+      kTensorBias ? reinterpret_cast<const T*>(p.bias) + (int64_t)b * p.bias_bs + (int64_t)h * p.bias_hs : nullptr;
+  unsigned char* const bias_lds = lds_raw + Cfg::kLdsBytes + wave * kBiasWaveBytes;
+  u32x4 braw[kTensorBias ? kBiasNLD : 1];
+  auto load_bias = [&](int tile) {
+#pragma unroll
+    for (int i = 0; i < kBiasNLD; i++) {
+      const int row = mw + i * kBiasRPI + lane / kBiasCPR, k0 = tile * BN + (lane % kBiasCPR) * 8;
+      braw[i] = u32x4{0, 0, 0, 0};
+      if (k0 < Lk) braw[i] = ld_global16(bias_bh + (uint32_t)(row < Lq ? row : Lq - 1) * (uint32_t)p.bias_rs + (uint32_t)k0);
+    }
+  };
+  auto bias_to_lds = [&]() {
+#pragma unroll
+    for (int i = 0; i < kBiasNLD; i++)
+      *reinterpret_cast<u32x4*>(bias_lds + (i * kBiasRPI + lane / kBiasCPR) * kBiasRowBytes + (lane % kBiasCPR) * 16) = braw[i];
+  };
   int voff[DV / 32];  // element offsets of this lane's transposed V reads and K row fragments inside a tile
 #pragma unroll
   for (int db = 0; db < DV / 32; db++) voff[db] = tr_off<D, kSwzTr>(0, db * 4, lane);
@@ -181,7 +202,10 @@ __global__ void __launch_bounds__(256, (!kDropout && kBias == 0 && D <= 64) ? 4 
 
   int it = next_active(tile0);
   bool row_on_cur = row_on_next;
-  if (it < ntiles) stage(it, 0);
+  if (it < ntiles) {
+    stage(it, 0);
+    if (kTensorBias) load_bias(it);
+  }
   while (it < ntiles) {
     const int n0 = it * BN;
     // Opaque redefinition of the accumulators at the top of every iteration: without it the register allocator
@@ -193,6 +217,10 @@ __global__ void __launch_bounds__(256, (!kDropout && kBias == 0 && D <= 64) ? 4 
     __syncthreads();                     // so is everyone else's, and nobody still reads the other buffer
     const int it_next = next_active(it + 1);
     if (it_next < ntiles) stage(it_next, buf ^ 1);
+    if (kTensorBias) {  // (the wave's own reads of the last tile's values are behind it: LDS operations of a wave stay in order)
+      bias_to_lds();
+      if (it_next < ntiles) load_bias(it_next);
+    }
     const T* Ks = reinterpret_cast<const T*>(lds_raw + buf * kBufBytes);
     const T* Vs = Ks + BN * D;
     buf ^= 1;
@@ -214,17 +242,14 @@ __global__ void __launch_bounds__(256, (!kDropout && kBias == 0 && D <= 64) ? 4 
       // ---- S^T = K Q^T, dead scores set to -inf, bias added
       auto scores = [&]() {
         // kTensorBias: the lane's 4 x 4 consecutive bias values per 32-key block (registers 4 j .. 4 j + 3 <-> keys
-        // 8 j + 4 hf ..), asked for before the MFMAs; groups that begin past the last key are not read
+        // 8 j + 4 hf ..) of its row
         typename E::vec4 bv[kTensorBias ? KBW : 1][4];
         if (kTensorBias) {
 #pragma unroll
           for (int kb = 0; kb < KBW; kb++)
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-              const int k0 = n0 + (kb0 + kb) * 32 + 8 * j + 4 * hf;
-              bv[kb][j] = typename E::vec4{0, 0, 0, 0};
-              if (k0 < Lk) bv[kb][j] = *reinterpret_cast<const typename E::vec4*>(bias_row + k0);
-            }
+            for (int j = 0; j < 4; j++)
+              bv[kb][j] = *reinterpret_cast<const typename E::vec4*>(bias_lds + c * kBiasRowBytes + ((kb0 + kb) * 32 + 8 * j + 4 * hf) * 2);
         }
 #pragma unroll
         for (int kb = 0; kb < KBW; kb++) {
@@ -250,13 +275,16 @@ __global__ void __launch_bounds__(256, (!kDropout && kBias == 0 && D <= 64) ? 4 
               if (dead) s[kb][r] = -INFINITY;
             }
         }
-        if (kTensorBias) {  // s <- s * scale * log2(e) + bias * log2(e); dead scores stay -inf whatever lies behind them
+        if (kTensorBias) {  // s <- s * scale * log2(e) + bias * log2(e)
+          // Dead scores must stay -inf whatever lies behind them: past the last key a row of the caller's tensor may hold
+          // anything, so on a tile that needs a mask +inf and NaN are cut off (fminf returns the number)
 #pragma unroll
           for (int kb = 0; kb < KBW; kb++)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-              const float bf = (s[kb][r] == -INFINITY) ? 0.f : (float)bv[kb][r >> 2][r & 3] * kLog2e;
-              s[kb][r] = __builtin_fmaf(s[kb][r], cs, bf);
+              float bf = (float)bv[kb][r >> 2][r & 3];
+              if (need_mask) bf = fminf(bf, 3.0e38f);
+              s[kb][r] = __builtin_fmaf(bf, kLog2e, s[kb][r] * cs);
             }
         }
         if (kAlibi) {  // s <- s * scale * log2(e) - slope2 * |key - query|; dead scores stay -inf
