@@ -79,7 +79,9 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasT
   static_assert(BM == 64 || BM == 32, "a tile is one or two 32-row slabs");
   constexpr int RBT = BM / 16;  // 16-row blocks per tile (sparse activity bits per tile)
 
-  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
+  // kTensorBias: behind everything else, per wave BM rows x its 32 keys of bias (see load_bias below)
+  constexpr int kBiasTileBytes = BM * 32 * 2;
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes + (kBias == kBiasTensor ? 4 * kBiasTileBytes : 0)];
 
   // XCD-aware id map (see map_tile): the key tiles of one (batch, head) share one XCD's L2 copy of Q and dO.
   int bh, kt;  // under a causal mask the first key tiles see the most query rows: rank order is already heavy-first
@@ -237,13 +239,34 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasT
   const float cs = p.scale_log2;
   const float sl2 = kAlibi ? p.alibi[h] * kLog2e : 0.f;  // ALiBi slope in base-2 exponent units (see fa_fwd_kernel)
   // kTensorBias: this lane's column (key) of the bias and of its gradient; row q is q * stride further
+  // kTensorBias: the bias of a tile's BM query rows and the wave's 32 keys comes in as whole rows (4 lanes fetch the 64 bytes of a
+  // row, 16 bytes each, one tile ahead), is written to a wave-private piece of LDS laid out like a Q tile of 32 columns, and is
+  // read back with the transposed reads that give the MFMA's B operand order: register r <-> row 8 (r / 4) + 4 hf + r % 4 of the
+  // lane's key, the accumulators' order.  (Read straight from global memory in that order - 16 two-byte loads per slab in front
+  // of the MFMAs whose results need them - the kernel took 274 us at the headline shape where it takes 198 us without a bias.)
   // (wave-uniform bases and 32-bit element offsets: a (batch, head) slice holds fewer than 2^31 elements, the front end checks)
   const T* const bias_bh =
       kTensorBias ? reinterpret_cast<const T*>(p.bias) + (int64_t)b * p.bias_bs + (int64_t)h * p.bias_hs : nullptr;
   T* const dbias_bh =
       (kTensorBias && p.dbias) ? reinterpret_cast<T*>(p.dbias) + (int64_t)b * p.dbias_bs + (int64_t)h * p.dbias_hs : nullptr;
-  const uint32_t bias_key = (uint32_t)(key < Lk ? key : Lk - 1);
   const uint32_t bias_rs = (uint32_t)p.bias_rs, dbias_rs = (uint32_t)p.dbias_rs;
+  T* const bias_lds = reinterpret_cast<T*>(lds_raw + Cfg::kLdsBytes + wave * kBiasTileBytes);
+  constexpr int kBiasNLD = BM * 4 / 64;  // 16-byte loads per lane and tile
+  u32x4 bpre[kTensorBias ? kBiasNLD : 1];
+  auto load_bias = [&](int q_first) {
+#pragma unroll
+    for (int i = 0; i < kBiasNLD; i++) {
+      const int qr = q_first + i * 16 + (lane >> 2), k0 = n0 + wave * 32 + (lane & 3) * 8;
+      bpre[i] = u32x4{0, 0, 0, 0};  // chunks that begin past the last key are not read; rows past the end read the last row
+      if (k0 < Lk) bpre[i] = ld_global16(bias_bh + (uint32_t)(qr < Lq ? qr : Lq - 1) * bias_rs + (uint32_t)k0);
+    }
+  };
+  auto bias_to_lds = [&]() {
+#pragma unroll
+    for (int i = 0; i < kBiasNLD; i++)
+      *reinterpret_cast<u32x4*>(bias_lds + frag_off<32, kSwzDual>(i * 16 + (lane >> 2), lane & 3)) = bpre[i];
+  };
+  const int bt_lo = tr_off<32, kSwzDual>(0, 0, lane), bt_hi = tr_off<32, kSwzDual>(8, 0, lane);
   // element offsets inside a tile of this lane's row fragments and of its transposed reads (rows +0 and +8)
   int foff[D / 16], tlo[DV / 32], thi[DV / 32];
 #pragma unroll
@@ -263,6 +286,7 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasT
     else stage(mt, 0);
   }
   finish_kv();
+  if (kTensorBias && more) load_bias(mt * BM);
   while (more) {
     const int m0 = mt * BM;
     wait_vmem();  // this thread's share of the tile has arrived (LDS) / is in statpre
@@ -277,6 +301,10 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasT
     } else {
       more = mt + 1 < mt_end;
       if (more) stage(mt + 1, buf ^ 1);
+    }
+    if (kTensorBias) {  // (the wave's own reads of the last tile's values are behind it: LDS operations of a wave stay in order)
+      bias_to_lds();
+      if (more) load_bias((mt + 1) * BM);
     }
     const T* const Ql = reinterpret_cast<const T*>(lds_raw + buf * kBufBytes);
     const T* const dOl = Ql + BM * D;
@@ -324,11 +352,13 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasT
       // 8 (r / 4) + 4 hf + r % 4), asked for before the MFMAs; rows past the end read the last row (their P is 0)
       T braw[kTensorBias ? 16 : 1];
       if (kTensorBias) {
-        const uint32_t q0 = (uint32_t)(q_lo + 4 * hf), qlast = (uint32_t)(Lq - 1);
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const uint32_t qr = q0 + 8 * (r >> 2) + (r & 3);
-          braw[r] = bias_bh[(qr < qlast ? qr : qlast) * bias_rs + bias_key];
+        for (int t = 0; t < 2; t++) {
+          const T* bp = bias_lds + (qb * 32 + 16 * t) * 32;
+          const u32x2 lo = lds_read_tr16(bp + bt_lo), hi = lds_read_tr16(bp + bt_hi);
+          const vec8 bv = bitcast<vec8>(u32x4{lo[0], lo[1], hi[0], hi[1]});
+#pragma unroll
+          for (int i = 0; i < 8; i++) braw[8 * t + i] = bv[i];
         }
       }
       vec8 aq[D / 16], ad[D / 16];
