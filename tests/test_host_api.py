@@ -366,3 +366,28 @@ def test_header_is_plain_c(tmp_path):
                         "-I", os.path.join(ROOT, "include"), str(src)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     assert r.returncode == 0, r.stdout
 
+
+
+def test_prepare_attn_bias_layout_rules():
+    """prepare_attn_bias hands the caller's tensor through when the kernels can read it as it is (keys contiguous, rows a
+    multiple of 8 elements, 16-byte aligned) and pads a copy otherwise; shape, dtype and device are checked."""
+    from flash_attn import flash_attn_gfx950 as be
+    q = torch.zeros(10, 3, 64, dtype=torch.float16)
+    good = torch.randn(1, 3, 40, 48).half()
+    assert be.prepare_attn_bias(good, q, 2, 3, 40, 48) is good
+    assert be.prepare_attn_bias(good, q, 2, 3, 33, 41) is good                       # larger than needed is fine
+    odd = torch.randn(2, 1, 40, 45).half()
+    p = be.prepare_attn_bias(odd, q, 2, 3, 40, 45)
+    assert p is not odd and tuple(p.shape) == (2, 1, 40, 48) and p.stride(2) % 8 == 0 and p.stride(3) == 1
+    assert torch.equal(p[..., :45], odd) and torch.equal(p[..., 45:], torch.zeros(2, 1, 40, 3).half())
+    view = torch.randn(1, 3, 40, 96).half()[..., ::2]                                  # keys not contiguous
+    p = be.prepare_attn_bias(view, q, 2, 3, 40, 48)
+    assert p.stride(3) == 1 and torch.equal(p, view)
+    for bad, msg in ((torch.zeros(3, 3, 40, 48).half(), "attn_bias must be"),           # batch neither 1 nor 2
+                     (torch.zeros(1, 2, 40, 48).half(), "attn_bias must be"),           # heads neither 1 nor 3
+                     (torch.zeros(1, 3, 39, 48).half(), "attn_bias must be"),           # too few rows
+                     (torch.zeros(1, 3, 40, 47).half(), "attn_bias must be"),           # too few keys
+                     (torch.zeros(3, 40, 48).half(), "attn_bias must be"),              # not 4-D
+                     (torch.zeros(1, 3, 40, 48), "dtype and device")):                  # fp32 for fp16 inputs
+        with pytest.raises(RuntimeError, match=msg):
+            be.prepare_attn_bias(bad, q, 2, 3, 40, 48)
