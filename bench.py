@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused attention path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all] [--no-cpu] [--no-configs]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all] [--no-cpu] [--no-configs] [--backward PLAN]
 
 One step = one forward + one backward pass of the headline workload (fp16, B=8, H=12, d=64, N=2048, packed qkv,
 non-causal, dropout 0, synthetic N(0,1) data resident in HBM), called through the C ABI.  Prints ONE JSON line:
@@ -371,6 +371,9 @@ def main():
     ap.add_argument("--only", default=None, metavar="TEXT",
                     help="time only the BASELINE configurations whose name contains TEXT and print their table rows "
                          "(no JSON line): for collecting rocprofv3 counters of one configuration")
+    ap.add_argument("--backward", choices=("auto", "two-kernel", "one-kernel"), default="auto",
+                    help="backward plan (fa_set_launch_policy 0x10 / 0x20): the dQ + dK/dV kernel pair, or the one-kernel "
+                         "backward where it exists (head dim 64, dense, no mask, dropout or bias)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     a = ap.parse_args()
@@ -382,6 +385,7 @@ def main():
     be.load_library()  # fails loudly if the HIP library is not built
     if a.redraw_dropout:
         be.KEEP_WORDS_MAX_BYTES = 0
+    be.set_launch_policy({"auto": 0, "two-kernel": 0x10, "one-kernel": 0x20}[a.backward])
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
 

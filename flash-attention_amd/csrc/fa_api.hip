@@ -274,6 +274,18 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
   return FA_OK;
 }
 
+// Scratch of the one-kernel backward (fa_bwd_fused_kernel.h) where it applies, else 0: an fp32 dQ and its hand-over counters.
+// It applies to head_dim 64 without mask, dropout, bias or block layout, when the launch policy asks for it, and only when
+// all key tiles of a (batch, head) fit one XCD at once with room to spare (they wait for each other).
+size_t fused_bwd_bytes(const fa_bwd_args* a) {
+  if ((fa::launch_policy() & 0x30) != 0x20) return 0;
+  if (a->head_dim != 64 || a->blockmask || a->p_dropout > 0.f || a->alibi_slopes || a->attn_bias || a->is_causal) return 0;
+  if (a->batch <= 0 || a->nheads <= 0 || a->max_seqlen_q <= 0 || a->max_seqlen_k <= 0) return 0;
+  if ((a->max_seqlen_k + fa::kBwdBN - 1) / fa::kBwdBN > 32) return 0;
+  const size_t nqt = ((size_t)a->max_seqlen_q + fa::kFusedBM - 1) / fa::kFusedBM;
+  return (size_t)a->batch * a->nheads * nqt * (fa::kFusedBM * 64 * 4 + 4 * 4);
+}
+
 int bwd_impl(const fa_bwd_args* a, bool want_block, void* ev_main_start = nullptr, void* ev_main_stop = nullptr) {
   if (!a) return fail(FA_ERR_INVALID_ARGUMENT, "args is NULL");
   int rc = check_common(a->struct_bytes, sizeof(fa_bwd_args), a->dtype, a->batch, a->nheads, a->head_dim, a->total_q,
@@ -377,6 +389,16 @@ int bwd_impl(const fa_bwd_args* a, bool want_block, void* ev_main_start = nullpt
     p.kw_kb = (int)fa::keep_words_key_blocks(a->max_seqlen_k);
   }
 
+  // the whole backward in one kernel, if the caller brought the scratch for it
+  const size_t fused_need = fused_bwd_bytes(a);
+  if (fused_need > 0 && !a->dbias && a->workspace && a->workspace_bytes >= fused_need && aligned16(a->workspace)) {
+    p.nqt_ring = (a->max_seqlen_q + fa::kFusedBM - 1) / fa::kFusedBM;
+    p.dq_acc = reinterpret_cast<float*>(a->workspace);
+    p.dq_flags = reinterpret_cast<int*>(ws + (size_t)a->batch * a->nheads * p.nqt_ring * fa::kFusedBM * a->head_dim * 4);
+    FA_LAUNCH(fa::launch_bwd_fused(p, a->dtype, stream, reinterpret_cast<hipEvent_t>(ev_main_start),
+                                   reinterpret_cast<hipEvent_t>(ev_main_stop)));
+    return FA_OK;
+  }
   // short query side, long key side: the dQ kernel would walk all keys with one workgroup per (batch, head)
   const SplitPlan sp = split_plan(a->batch, a->nheads, a->head_dim, a->total_q, a->max_seqlen_q, a->max_seqlen_k, r.sq_r,
                                   a->is_causal != 0, sparse);
@@ -456,7 +478,10 @@ size_t fa_fwd_workspace_bytes(const fa_fwd_args* a) {
 size_t fa_bwd_workspace_bytes(const fa_bwd_args* a) {
   if (!a) return 0;
   if (a->blockmask) return sparse_layout(round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, true)).bytes;
-  // optional: partial dQ of the key-split dQ kernel (same plan as the forward's; o_bytes is n_splits fp32 copies of dq)
+  // optional: the fp32 dQ and counters of the one-kernel backward, or the partial dQ of the key-split dQ kernel (same plan as
+  // the forward's; o_bytes is n_splits fp32 copies of dq)
+  const size_t fused = fused_bwd_bytes(a);
+  if (fused > 0) return fused;
   const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, false);
   return split_plan(a->batch, a->nheads, a->head_dim, a->total_q, a->max_seqlen_q, a->max_seqlen_k, r.sq_r,
                     a->is_causal != 0, false).o_bytes;
@@ -547,7 +572,9 @@ int fa_rotary(const fa_rotary_args* a) {
 }
 
 int fa_set_launch_policy(int policy) {
-  FA_REQUIRE(policy >= 0 && policy <= 2, "launch policy must be 0 (automatic), 1 (full-size tiles) or 2 (half-size tiles)");
+  FA_REQUIRE((policy & ~0x33) == 0 && (policy & 3) != 3 && (policy & 0x30) != 0x30,
+             "launch policy: tile shape 0 (automatic), 1 (full-size) or 2 (half-size), plus 0x10 (two-kernel backward) or 0x20 "
+             "(one-kernel backward where it exists)");
   g_launch_policy.store(policy, std::memory_order_relaxed);
   return FA_OK;
 }

@@ -128,6 +128,12 @@ struct BwdParams {
   const uint32_t* keep_words;
   int kw_q;   // query extent of the buffer (max_seqlen_q rounded up to 128)
   int kw_kb;  // 32-key blocks (max_seqlen_k rounded up to 128, / 32)
+  // One-kernel backward (fa_bwd_fused_kernel.h): fp32 running sums of dQ [B * H, nqt_ring tiles, 2048] and their hand-over
+  // counters [B * H, nqt_ring, 4]
+  float* dq_acc;
+  int* dq_flags;
+  int nqt_ring;     // query tiles of max_seqlen_q
+  int ring_stride;  // tiles between the starting points of consecutive key tiles (0: the kernel's default)
 };
 
 // Sequence extent of batch entry b, clamped so that a cu_seqlens array that disagrees with the declared
@@ -188,7 +194,7 @@ inline int tile_grid(bool tile_major, int tiles_per_bh, int BH) {
 // (fa_set_launch_policy; the parity tests run both shapes on the same inputs).
 int launch_policy();
 inline bool small_launch(int BH, int max_s, bool causal) {
-  const int policy = launch_policy();
+  const int policy = launch_policy() & 3;
   if (policy != 0) return policy == 2;
   const int64_t wgs = (int64_t)BH * ((max_s + 127) / 128);
   (void)causal;
@@ -201,6 +207,9 @@ hipError_t launch_fwd(const FwdParams& p, int dtype, int head_dim, bool causal, 
                       hipStream_t stream);
 hipError_t launch_fwd_combine(const FwdParams& p, int dtype, int head_dim, hipStream_t stream);
 hipError_t launch_dq_combine(const BwdParams& p, int dtype, int head_dim, hipStream_t stream);
+// The whole backward in one kernel (fa_bwd_fused_kernel.h; head_dim 64, dense, no mask, no dropout, no bias): softmax_d pass, then
+// the kernel.  ev_start / ev_stop: null, or events recorded around the main kernel.
+hipError_t launch_bwd_fused(const BwdParams& p, int dtype, hipStream_t stream, hipEvent_t ev_start, hipEvent_t ev_stop);
 // fa_rotary: rotate the first n_rotated of n_parts (row, part, head, head_dim) slices, copy the others
 struct RotaryParams {
   const void* src;
@@ -235,5 +244,6 @@ hipError_t launch_zero_rows(void* base, int64_t row_stride, int64_t head_stride,
 // Tile shapes, needed by the front end for grid sizes and workspace layout.
 constexpr int kFwdBM = 128;   // query rows per forward workgroup
 constexpr int kBwdBN = 128;   // keys per dK/dV workgroup
+constexpr int kFusedBM = 32;  // query rows per step of the one-kernel backward
 
 }  // namespace fa

@@ -171,8 +171,9 @@ def load_library():
 
 
 def set_launch_policy(policy):
-    """0: tile shapes chosen per launch (default); 1: always the full-size tiles; 2: the half-size tiles wherever they
-    exist (fa_set_launch_policy)."""
+    """Tile shape: 0 chosen per launch (default), 1 always the full-size tiles, 2 the half-size tiles wherever they exist;
+    plus the backward plan: 0x10 the dQ + dK/dV kernel pair (also the default), 0x20 the one-kernel backward where it
+    exists (fa_set_launch_policy)."""
     lib = load_library()
     rc = lib.fa_set_launch_policy(int(policy))
     if rc != 0:

@@ -181,8 +181,9 @@ int fa_fwd_block_noalloc(const fa_fwd_args* args);
  * batch * nheads < 128, max_seqlen_k >= 512: decoding and cross-attention shapes) fa_fwd_workspace_bytes() returns the size of the
  * partial results of a key-split pass: if `workspace` holds that much, fa_fwd shares the keys of each query tile
  * among several workgroups and merges their results; if not, it runs the single pass.  fa_bwd_workspace_bytes() does the
- * same for the dQ kernel of such shapes (fp32 partial dQ per key split).  Only shapes, is_causal and blockmask != NULL
- * are read. */
+ * same for the dQ kernel of such shapes (fp32 partial dQ per key split), and, under launch policy 0x20, returns the
+ * scratch of the one-kernel backward (fp32 running sums of dQ and their hand-over counters: about twice the bytes of dq).
+ * Only shapes, is_causal, p_dropout, the bias pointers and blockmask != NULL are read. */
 size_t fa_fwd_workspace_bytes(const fa_fwd_args* args);
 size_t fa_bwd_workspace_bytes(const fa_bwd_args* args);
 /* Size of fa_fwd_args.keep_words / fa_bwd_args.keep_words: one bit per (batch, head, query, key) with both sequence
@@ -244,11 +245,16 @@ typedef struct fa_rotary_args {
 } fa_rotary_args;
 int fa_rotary(const fa_rotary_args* args);
 
-/* Tile shape selection (process-wide; no counterpart in the reference, whose launchers pick their tile by head size
- * and sequence length alone, fmha_api.cpp:232-241).  0 (default): short-sequence launches that would leave compute units
- * idle with the full-size tiles (128 query rows / 128 keys per workgroup) use the half-size variants where they exist
- * (head_dim <= 64, no blockmask, no alibi_slopes); 1: always full-size; 2: always half-size where they exist.  Results
- * agree within rounding between the shapes (the order of fp32 summation differs), not bit for bit. */
+/* Launch policy (process-wide state; no counterpart in the reference, whose launchers pick their tile by head size
+ * and sequence length alone, fmha_api.cpp:232-241).  policy = tile shape | backward plan.
+ * Tile shape (bits 0-1): 0 (default): short-sequence launches that would leave compute units idle with the full-size
+ * tiles (128 query rows / 128 keys per workgroup) use the half-size variants where they exist (head_dim <= 64, no
+ * blockmask, no alibi_slopes); 1: always full-size; 2: always half-size where they exist.
+ * Backward plan (bits 4-5): 0 (default) and 0x10: two kernels (dQ with softmax_d, then dK/dV), no scratch; 0x20: one kernel
+ * that also passes dQ from key tile to key tile through fp32 scratch, where it exists (head_dim 64, no blockmask, mask,
+ * dropout or bias, max_seqlen_k <= 4096) and only if the caller brings the scratch fa_bwd_workspace_bytes() then asks for.
+ * Results agree within rounding between the choices (the order of fp32 summation differs), not bit for bit; each choice is
+ * reproducible bit for bit from run to run. */
 int fa_set_launch_policy(int policy);
 
 /* Message for the last non-zero status returned on the calling thread. */

@@ -294,6 +294,32 @@ def test_blocksparse_module_layout_handling_on_host():
             FlashBlocksparseAttention({"_target_": "some.module.Config"})
 
 
+def test_launch_policy_values_and_one_kernel_backward_scratch(lib):
+    """fa_set_launch_policy: tile shape in the low bits, backward plan in 0x30; the one-kernel backward asks for scratch only
+    where it exists (head dim 64, dense, no mask, dropout or bias, at most 32 key tiles)"""
+    from flash_attn import flash_attn_gfx950 as be
+    for ok in (0, 1, 2, 0x10, 0x11, 0x12, 0x20, 0x21, 0x22):
+        assert lib.fa_set_launch_policy(ok) == 0
+    for bad in (3, 0x30, 0x40, -1, 0x100):
+        assert lib.fa_set_launch_policy(bad) == -1 and b"launch policy" in lib.fa_last_error()
+    a = be.BwdArgs()
+    a.struct_bytes = ctypes.sizeof(a)
+    a.batch, a.nheads, a.head_dim = 8, 12, 64
+    a.max_seqlen_q = a.max_seqlen_k = 2048
+    try:
+        lib.fa_set_launch_policy(0)
+        assert lib.fa_bwd_workspace_bytes(ctypes.byref(a)) == 0      # the two-kernel backward needs no scratch
+        lib.fa_set_launch_policy(0x20)
+        want = 8 * 12 * 64 * (32 * 64 * 4 + 16)                      # fp32 running sums and four counters per 32-row tile
+        assert lib.fa_bwd_workspace_bytes(ctypes.byref(a)) == want
+        for field, value in (("head_dim", 128), ("is_causal", 1), ("p_dropout", 0.1), ("max_seqlen_k", 4097)):
+            b = be.BwdArgs.from_buffer_copy(a)
+            setattr(b, field, value)
+            assert lib.fa_bwd_workspace_bytes(ctypes.byref(b)) == 0, field
+    finally:
+        lib.fa_set_launch_policy(0)
+
+
 def test_key_split_workspace_plan(lib):
     """fa_fwd_workspace_bytes asks for scratch only for dense, non-causal forwards with one query tile, few
     (batch, head) pairs and many keys; the size is n_splits * (fp32 partial outputs + partial lse)."""

@@ -1178,6 +1178,70 @@ def test_flash_mha_matches_torch_multihead_attention():
 # ------------------------------------------------------------------------------------------------
 # BASELINE configurations at full size: fp32 PyTorch on the GPU as the reference, plus size-independent properties
 # ------------------------------------------------------------------------------------------------
+# ------------------------------------------------------------------------------------------------
+# the one-kernel backward (launch policy 0x20: head dim 64, dense, no mask / dropout / bias)
+# ------------------------------------------------------------------------------------------------
+@pytest.fixture
+def one_kernel_backward():
+    from flash_attn import flash_attn_gfx950 as be
+    be.set_launch_policy(0x20)
+    yield
+    be.set_launch_policy(0)
+
+
+@pytest.mark.parametrize("lens_q,lens_k,dtype,packing", [
+    ([256, 256], [256, 256], torch.float16, "qkv"),
+    ([300, 77], [300, 77], torch.float16, "qkv"),
+    ([1024, 130, 640], [1024, 130, 640], torch.bfloat16, "qkv"),
+    ([200, 31, 512], [640, 129, 96], torch.float16, "kv"),     # more key tiles than query tiles and the reverse
+    ([33], [1500], torch.bfloat16, "sep"),                     # two query tiles, twelve key tiles
+    ([700, 5], [1, 260], torch.float16, "sep"),
+])
+def test_one_kernel_backward_parity(lens_q, lens_k, dtype, packing, one_kernel_backward):
+    """the same parity bar as the two-kernel backward, on shapes that wrap the ring of query tiles in every way"""
+    from flash_attn import flash_attn_gfx950 as be
+    a = be.BwdArgs()
+    a.struct_bytes = ctypes.sizeof(a)
+    a.batch, a.nheads, a.head_dim = len(lens_q), 3, 64
+    a.max_seqlen_q, a.max_seqlen_k = max(lens_q), max(lens_k)
+    assert be.load_library().fa_bwd_workspace_bytes(ctypes.byref(a)) > 0  # the path under test is the one that runs
+    _parity_case(lens_q, lens_k, 3, 64, dtype, False, packing, seed=11)
+
+
+def test_one_kernel_backward_headline_and_determinism(one_kernel_backward):
+    """the headline shape: parity, bitwise equal results from run to run (one owner at a time, fixed order), and agreement
+    with the two-kernel backward within the rounding of the 16-bit results"""
+    from flash_attn import flash_attn_gfx950 as be
+    q, k, v, do, cu, ours = _full_size_check([2048] * 8, 12, 64, torch.float16, False, seed=1)
+    again = run_ours(q, k, v, do, cu, cu, 2048, 2048, 0.0, None, False, "qkv")
+    for n in ("dq", "dk", "dv"):
+        assert torch.equal(ours[n], again[n]), n
+    be.set_launch_policy(0x10)
+    two = run_ours(q, k, v, do, cu, cu, 2048, 2048, 0.0, None, False, "qkv")
+    for n in ("dq", "dk", "dv"):
+        assert _maxerr(ours[n], two[n]) <= 4 * HALF_ULP[torch.float16] * two[n].float().abs().max().item(), n
+
+
+def test_one_kernel_backward_batch_entries_without_keys_or_queries(one_kernel_backward):
+    """a batch entry without keys has no key tile: its dq rows are zero; one without queries leaves dk = dv = 0"""
+    from flash_attn import flash_attn_gfx950 as be
+    lens_q, lens_k, H, D = [100, 64, 0], [90, 0, 70], 2, 64
+    q, k, v, do = (x.cuda() for x in _inputs(lens_q, lens_k, H, D, torch.float16, 5))
+    cu_q, cu_k = _cu(lens_q), _cu(lens_k)
+    o, lse = be.fwd(q, k, v, cu_q, cu_k, 100, 90, 0.0, 0.125, False, False, False, None)
+    dq, dk, dv = (torch.full_like(x, float("nan")) for x in (q, k, v))
+    be.bwd(do, q, k, v, o, lse, dq, dk, dv, cu_q, cu_k, 100, 90, 0.0, 0.125, False, False, None)
+    torch.cuda.synchronize()
+    be.set_launch_policy(0x10)
+    dq2, dk2, dv2 = (torch.full_like(x, float("nan")) for x in (q, k, v))
+    be.bwd(do, q, k, v, o, lse, dq2, dk2, dv2, cu_q, cu_k, 100, 90, 0.0, 0.125, False, False, None)
+    torch.cuda.synchronize()
+    assert not torch.isnan(dq).any() and not torch.isnan(dk).any() and not torch.isnan(dv).any()
+    assert torch.equal(dq[100:164], torch.zeros_like(dq[100:164])) and torch.equal(dk[90:], torch.zeros_like(dk[90:]))
+    for a_, b_ in ((dq, dq2), (dk, dk2), (dv, dv2)):
+        assert _maxerr(a_, b_) <= 4 * HALF_ULP[torch.float16] * max(1.0, b_.float().abs().max().item())
+
+
 def _full_size_check(lens, H, D, dtype, causal, p=0.0, seed=0):
     q, k, v, do = (x.cuda() for x in _inputs(lens, lens, H, D, dtype, seed))
     cu = _cu(lens, "cpu")
