@@ -9,7 +9,7 @@
 #include <atomic>
 #include <mutex>
 
-#include "../../include/flash_attn_gfx950.h"
+#include "../../include/flash_attn_gfx950_bench.h"
 #include "fa_params.h"
 
 // ---- fa_fwd_block_noalloc: the block activity maps live in this file-scope device array instead of caller scratch.
@@ -372,8 +372,12 @@ int bwd_impl(const fa_bwd_args* a, bool want_block, void* ev_main_start = nullpt
   }
   if (a->dbias) {
     FA_REQUIRE(a->attn_bias, "dbias without attn_bias");
-    FA_REQUIRE(a->dbias_row_stride >= a->max_seqlen_k && a->dbias_head_stride > 0 && (a->dbias_batch_stride > 0 || a->batch == 1),
-               "dbias needs its own slice for every (batch, head) and rows of at least max_seqlen_k elements");
+    FA_REQUIRE(a->dbias_row_stride >= a->max_seqlen_k &&
+                   a->dbias_head_stride >= (int64_t)a->max_seqlen_q * a->dbias_row_stride &&
+                   (a->batch == 1 || a->dbias_batch_stride >= (int64_t)a->nheads * a->dbias_head_stride) &&
+                   (reinterpret_cast<uintptr_t>(a->dbias) & 1) == 0,
+               "dbias needs its own slice for every (batch, head) - rows of at least max_seqlen_k elements, head stride of at least "
+               "max_seqlen_q rows, batch stride of at least nheads head strides - and 2-byte alignment");
     if ((int64_t)a->max_seqlen_q * a->dbias_row_stride >= ((int64_t)1 << 31))
       return fail(FA_ERR_UNSUPPORTED, "dbias: a (batch, head) slice is limited to 2^31 elements");
     p.dbias = a->dbias;

@@ -48,7 +48,8 @@ __global__ void __launch_bounds__(512) gather_rows_kernel(const unsigned char* _
     if (i < nrows) *reinterpret_cast<C*>(dst + (row0 + i) * dst_stride + (int64_t)ch * V) = v[i];
 }
 
-// inv[idx[i]] = i (inv pre-filled with -1): the inverse of the index list, for the single-pass scatter below
+// inv[idx[i]] = i for the entries that have a source (the others keep whatever the scratch held: see scatter_rows_kernel):
+// the inverse of the index list, for the single-pass scatter below
 __global__ void __launch_bounds__(256) invert_index_kernel(const int64_t* __restrict__ idx, int64_t n_idx, int64_t n_dst,
                                                            int32_t* __restrict__ inv) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;

@@ -26,8 +26,10 @@ _c_i32p = ctypes.c_void_p
 
 # Dropout keep words: the forward can leave its keep decisions (one bit per score) in a buffer from which the backward's two
 # kernels read them instead of drawing them again with Philox; results are the same bit for bit.  new_keep_words() makes
-# that buffer unless it would be larger than this many bytes (0: never), in which case every kernel draws its own decisions,
-# as the reference's do, and no memory beyond O(seqlen) is held between forward and backward.
+# that buffer unless it would be larger than this many bytes (0: never) or larger than q, k and v together (one bit per score
+# grows with the square of the sequence length: from about 3 * 16 * head_dim tokens on it would outweigh the inputs), in which
+# case every kernel draws its own decisions, as the reference's do, and no memory beyond O(seqlen) is held between forward
+# and backward.
 KEEP_WORDS_MAX_BYTES = 1 << 30
 
 
@@ -106,11 +108,13 @@ class RotaryArgs(ctypes.Structure):
 
 
 EXPORTED_SYMBOLS = (
-    "fa_fwd", "fa_bwd", "fa_bwd_profiled", "fa_fwd_block", "fa_bwd_block", "fa_fwd_block_noalloc", "fa_fwd_workspace_bytes", "fa_bwd_workspace_bytes",
+    "fa_fwd", "fa_bwd", "fa_fwd_block", "fa_bwd_block", "fa_fwd_block_noalloc", "fa_fwd_workspace_bytes", "fa_bwd_workspace_bytes",
     "fa_round_seqlens", "fa_philox_offset_increment", "fa_last_error", "fa_abi_version",
     "fa_gather_rows", "fa_scatter_rows", "fa_scatter_rows_workspace_bytes", "fa_rotary", "fa_set_launch_policy",
     "fa_keep_words_bytes",
 )
+# declared in include/flash_attn_gfx950_bench.h: instrumentation for bench.py, not part of the drop-in boundary
+BENCH_SYMBOLS = ("fa_bwd_profiled",)
 
 _lib = None
 _lib_lock = threading.Lock()
@@ -303,13 +307,15 @@ def _bias_arg(a, attn_bias, q, batch, nheads, max_seqlen_q, max_seqlen_k, sparse
     return t
 
 
-def new_keep_words(q, cu_seqlens_q, max_seqlen_q, max_seqlen_k, p_dropout):
+def new_keep_words(q, cu_seqlens_q, max_seqlen_q, max_seqlen_k, p_dropout, total_k=None):
     """Buffer for the dropout keep words of one forward call (argument keep_words of fwd and bwd), or None if there is no
-    dropout or the buffer would exceed KEEP_WORDS_MAX_BYTES."""
+    dropout or the buffer would exceed KEEP_WORDS_MAX_BYTES or the bytes of q, k and v (total_k: rows of k and v; default:
+    those of q)."""
     if not p_dropout > 0:
         return None
     n = load_library().fa_keep_words_bytes(cu_seqlens_q.numel() - 1, q.shape[1], int(max_seqlen_q), int(max_seqlen_k))
-    if n == 0 or n > KEEP_WORDS_MAX_BYTES:
+    inputs = (q.shape[0] + 2 * (q.shape[0] if total_k is None else int(total_k))) * q.shape[1] * q.shape[2] * q.element_size()
+    if n == 0 or n > KEEP_WORDS_MAX_BYTES or n > inputs:
         return None
     return torch.empty((n,), dtype=torch.uint8, device=q.device)
 

@@ -50,10 +50,11 @@ def _forward(ctx, packing, tensors, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, ma
     if softmax_scale is None:
         softmax_scale = q.shape[-1] ** (-0.5)
     # with a backward to come, the forward leaves its dropout decisions (one bit per score) for it to read instead of
-    # drawing them twice more; None (no dropout, no gradient wanted, or too large: _backend.KEEP_WORDS_MAX_BYTES) = redraw
+    # drawing them twice more; None (no dropout, no gradient wanted, or larger than _backend.KEEP_WORDS_MAX_BYTES or than the
+    # inputs themselves) = redraw
     keep_words = None
     if dropout_p > 0 and any(ctx.needs_input_grad):
-        keep_words = _backend.new_keep_words(q, cu_seqlens_q, max_seqlen_q, max_seqlen_k, dropout_p)
+        keep_words = _backend.new_keep_words(q, cu_seqlens_q, max_seqlen_q, max_seqlen_k, dropout_p, total_k=k.shape[0])
     # the bias in the form the kernels read (the caller's tensor itself if its layout allows, else a padded copy)
     bias_t = None
     if attn_bias is not None:

@@ -85,7 +85,8 @@ typedef struct fa_fwd_args {
    * encoding").  NULL, or a device tensor of `dtype` indexed [batch, head, query, key] with the strides below in elements
    * (keys contiguous; batch and head stride may be 0: one bias for all of them): softmax_scale * q.k + bias[b, h, i, j] is
    * what the softmax sees, i < max_seqlen_q and j < max_seqlen_k being positions inside the sequences.  -inf entries mask.
-   * 16-byte aligned, bias_row_stride a multiple of 8 and >= max_seqlen_k.  Not with a blockmask, not with alibi_slopes. */
+   * 16-byte aligned, bias_row_stride a multiple of 8 and >= max_seqlen_k; every row is read in 16-byte pieces, i.e. up to the
+   * next multiple of 8 keys past max_seqlen_k (inside the row stride).  Not with a blockmask, not with alibi_slopes. */
   const void* attn_bias;
   int64_t bias_batch_stride, bias_head_stride, bias_row_stride;
 } fa_fwd_args;
@@ -141,8 +142,8 @@ typedef struct fa_bwd_args {
   const void* attn_bias;
   int64_t bias_batch_stride, bias_head_stride, bias_row_stride;
   /* NULL, or where to leave d(loss)/d(attn_bias): a tensor of `dtype` indexed [batch, head, query, key] with the strides
-   * below (nonzero batch and head strides: every (batch, head) has its own slice; sum over them for a shared bias), 2-byte
-   * aligned.  Only the (query, key) tiles the backward visits are written (under a causal mask none above the diagonal,
+   * below (every (batch, head) has its own slice: row stride >= max_seqlen_k, head stride >= max_seqlen_q rows, batch
+   * stride >= nheads head strides; sum over the slices for a shared bias), 2-byte aligned.  Only the (query, key) tiles the backward visits are written (under a causal mask none above the diagonal,
    * none past a sequence's end): the caller clears the tensor first. */
   void* dbias;
   int64_t dbias_batch_stride, dbias_head_stride, dbias_row_stride;
@@ -152,10 +153,6 @@ typedef struct fa_bwd_args {
 int fa_fwd(const fa_fwd_args* args);
 /* replaces flash_attn_cuda.bwd -> mha_bwd, csrc/flash_attn/fmha_api.cpp:302-449 */
 int fa_bwd(const fa_bwd_args* args);
-/* fa_bwd with two timing events (hipEvent_t, either may be NULL) recorded on args->stream immediately before and after the
- * dK/dV kernel, the longer of the backward's two kernels (dQ + softmax_d kernel first, then dK/dV).  No counterpart in
- * the reference; for benchmarks that price that kernel against its roofline.  Results are those of fa_bwd. */
-int fa_bwd_profiled(const fa_bwd_args* args, void* ev_main_start, void* ev_main_stop);
 /* replaces flash_attn_cuda.fwd_block -> mha_fwd_block, csrc/flash_attn/fmha_api.cpp:451-573
  * (args->blockmask must be non-NULL).  is_causal may be set together with a blockmask, here and in fa_bwd_block: a score
  * counts iff its block is listed AND key <= query; blocks that lie wholly above the diagonal may be listed or not.  The
@@ -171,7 +168,9 @@ int fa_bwd_block(const fa_bwd_args* args);
  * outputs are the caller's as usual.  Layouts whose maps need more (fa_fwd_workspace_bytes() > FA_NOALLOC_SCRATCH_BYTES;
  * the limit is reached between 16384 and 32768 tokens) are refused with FA_ERR_WORKSPACE.  The call allocates nothing
  * and the maps are rebuilt by every call, but all calls on one GPU share the one array: calls that overlap on a GPU
- * (different streams or host threads) race; serialise them.  Results are those of fa_fwd_block. */
+ * (different streams or host threads) race; serialise them.  The first call on a device looks up the array's device
+ * address, which is not meant to happen under stream capture: make one eager call per device before capturing.  The
+ * current device must be the device of args->stream.  Results are those of fa_fwd_block. */
 #define FA_NOALLOC_SCRATCH_BYTES (64u * 1024u)
 int fa_fwd_block_noalloc(const fa_fwd_args* args);
 
