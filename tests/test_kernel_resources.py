@@ -79,6 +79,30 @@ def test_d64_kernels_keep_their_waves_per_simd():
 
 
 @pytest.mark.timeout(600)
+def test_d64_bias_tensor_and_one_kernel_backward_variants():
+    """The variants that read a bias tensor run at three (forward without dropout) and two waves per SIMD; the dK/dV variant
+    that also draws dropout decisions is at the register limit and may spill a few registers, the others must not.  The
+    one-kernel backward runs two workgroups per compute unit: two waves per SIMD, nothing spilled, at most 80 KB of LDS."""
+    fwd = _resources("fa_fwd_d64.hip")
+    bwd = _resources("fa_bwd_d64.hip")
+    for causal in ("Lb0E", "Lb1E"):
+        k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", causal + "Lb0ELb0ELi2ELi1ELb0EEEv")
+        assert k["Occupancy"] >= 3 and k["VGPRs Spill"] <= 3, ("forward, bias tensor", causal, k)
+        for drop, words in (("Lb1E", "Lb0E"), ("Lb1E", "Lb1E")):
+            k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", causal + drop + "Lb0ELi2ELi1E" + words + "EEv")
+            assert k["Occupancy"] >= 2 and k["VGPRs Spill"] == 0, ("forward, bias tensor, dropout", causal, words, k)
+        for drop, spill in (("Li0E", 0), ("Li2E", 4), ("Li1E", 12)):
+            k = _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", causal + drop + "Lb0ELi2ELi1EEEv")
+            assert k["Occupancy"] >= 2 and k["VGPRs Spill"] == 0, ("dq, bias tensor", causal, drop, k)
+            k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", causal + drop + "Lb0ELi2E")
+            assert k["Occupancy"] >= 2 and k["VGPRs Spill"] <= spill, ("dkdv, bias tensor", causal, drop, k)
+    fused = _resources("fa_bwd_fused.hip")
+    for dt in ("IDF16_", "IDF16b"):
+        k = _pick(fused, "fa_bwd_fused_kernel%sLi64ELi0E" % dt)
+        assert k["Occupancy"] >= 2 and k["VGPRs Spill"] == 0 and k["LDS Size"] <= 80 * 1024, ("one-kernel backward", dt, k)
+
+
+@pytest.mark.timeout(600)
 def test_d128_backward_keeps_two_waves_per_simd():
     """d = 128: the dK/dV kernel holds its V tile in LDS so that K, the two accumulators and the scores fit 256 registers
     (two waves per SIMD, nothing spilled: a spill's scratch load would wait behind the tile prefetch on every step)."""
