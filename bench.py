@@ -354,6 +354,46 @@ def config_list(torch):
     ]
 
 
+def tile_sweep(torch, be, steps, warmup):
+    """Full-size (128 query rows / keys per workgroup) against half-size tiles (64 rows, wave pairs split the keys) of the
+    forward and the dQ kernel on launches of growing size: the table small_launch() (csrc/fa_params.h) takes its threshold
+    from.  The dK/dV kernel has one shape, so the backward column moves with the dQ kernel alone."""
+    g = torch.Generator().manual_seed(0)
+    bert = torch.randint(256, 513, (8,), generator=g).tolist()
+    bert16 = torch.randint(256, 513, (16,), generator=g).tolist()
+    shapes = [("BERT varlen p=0.1", dict(B=8, H=12, D=64, N=512, dtype=torch.float16, p=0.1, lens=bert)),
+              ("BERT varlen p=0.1, B=4", dict(B=4, H=12, D=64, N=512, dtype=torch.float16, p=0.1, lens=bert[:4])),
+              ("BERT varlen p=0.1, B=16", dict(B=16, H=12, D=64, N=512, dtype=torch.float16, p=0.1, lens=bert16)),
+              ("BERT varlen p=0, B=8", dict(B=8, H=12, D=64, N=512, dtype=torch.float16, lens=bert))]
+    for B, N in ((8, 512), (12, 512), (16, 512), (4, 1024), (8, 1024), (4, 2048)):
+        shapes.append(("fp16 p=0.1 B=%d N=%d" % (B, N), dict(B=B, H=12, D=64, N=N, dtype=torch.float16, p=0.1)))
+    for B, N in ((16, 128), (32, 128), (64, 128), (8, 256), (16, 256), (24, 256), (32, 256), (64, 256), (4, 512), (8, 512), (12, 512),
+                 (16, 512), (32, 512), (2, 1024), (4, 1024), (6, 1024), (8, 1024), (16, 1024), (1, 2048), (2, 2048), (3, 2048),
+                 (4, 2048), (6, 2048), (8, 2048), (12, 2048), (1, 4096), (2, 4096), (4, 4096)):
+        shapes.append(("fp16 B=%d N=%d" % (B, N), dict(B=B, H=12, D=64, N=N, dtype=torch.float16)))
+    for B, N in ((8, 256), (16, 256), (8, 512), (12, 512), (16, 512), (4, 1024), (6, 1024), (8, 1024), (16, 1024), (2, 2048), (3, 2048),
+                 (4, 2048), (8, 2048), (2, 4096), (4, 4096)):
+        shapes.append(("bf16 causal B=%d N=%d" % (B, N), dict(B=B, H=12, D=64, N=N, dtype=torch.bfloat16, causal=True)))
+    for B, N in ((8, 512), (16, 512), (8, 1024)):
+        shapes.append(("fp16 d=32 B=%d N=%d" % (B, N), dict(B=B, H=12, D=32, N=N, dtype=torch.float16)))
+    print("| launch | workgroups of 128 rows per compute unit | fwd full / half (us) | bwd full / half (us) | half wins fwd / bwd |",
+          file=sys.stderr)
+    print("|---|---|---|---|---|", file=sys.stderr)
+    for name, kw in shapes:
+        wl = Workload(torch, **kw)
+        wgs = wl.B * wl.H * ((wl.max_s + 127) // 128) / 256.0
+        t = {}
+        for pol in (1, 2):
+            be.set_launch_policy(pol)
+            t[pol] = time_steps(torch, be, wl, steps, warmup, 0.1)
+        be.set_launch_policy(0)
+        print("| %s | %.2f | %.1f / %.1f | %.1f / %.1f | %s / %s |" % (
+            name, wgs, t[1]["fwd_ms"] * 1e3, t[2]["fwd_ms"] * 1e3, t[1]["bwd_ms"] * 1e3, t[2]["bwd_ms"] * 1e3,
+            "yes" if t[2]["fwd_ms"] < t[1]["fwd_ms"] else "no", "yes" if t[2]["bwd_ms"] < t[1]["bwd_ms"] else "no"), file=sys.stderr)
+        del wl
+        torch.cuda.empty_cache()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -374,6 +414,8 @@ def main():
     ap.add_argument("--backward", choices=("auto", "two-kernel", "one-kernel"), default="auto",
                     help="backward plan (fa_set_launch_policy 0x10 / 0x20): the dQ + dK/dV kernel pair, or the one-kernel "
                          "backward where it exists (head dim 64, dense, no mask, dropout or bias)")
+    ap.add_argument("--tile-sweep", action="store_true",
+                    help="time full-size against half-size tiles on launches of growing size (markdown table on stderr, no JSON line)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     a = ap.parse_args()
@@ -395,6 +437,10 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+
+    if a.tile_sweep:
+        tile_sweep(torch, be, max(20, a.steps // 5), 5)
+        return
 
     if a.only is not None:
         for name, kw in config_list(torch):

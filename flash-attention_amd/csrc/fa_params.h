@@ -188,17 +188,24 @@ inline int tile_grid(bool tile_major, int tiles_per_bh, int BH) {
   return ((BH + 7) & ~7) * tiles_per_bh;
 }
 
-// Launch shape: with 128-row (128-key) tiles a short-sequence batch gives fewer workgroups than three per compute unit;
-// the kernels then run their half-size tile variants (twice the workgroups, half the serial work of each).
-// launch_policy(): 0 = by this rule, 1 = always the full-size tiles, 2 = the half-size tiles wherever they exist
+// Launch shape: with 128-row tiles a short-sequence batch gives the compute units one or two workgroups each, and one
+// workgroup's walk over its keys is the launch's critical path; the forward and the dQ kernel then run their half-size
+// tile variants (64 query rows, wave pairs split the keys: twice the workgroups, half the serial work of each).  The rule is
+// read off a sweep over batch size, sequence length, mask and dropout (bench.py --tile-sweep): with x = full-size
+// workgroups per compute unit,
+//   forward: half-size for x < 2 (more than one key tile pair to split: sequences beyond 128), and up to x < 3 with dropout
+//            (whose Philox work makes the serial walk longer);
+//   dQ:      half-size for 1 <= x < 2 under a causal mask or with dropout; the plain kernel gains nothing from it.
+// launch_policy() & 3: 0 = by this rule, 1 = always the full-size tiles, 2 = the half-size tiles wherever they exist
 // (fa_set_launch_policy; the parity tests run both shapes on the same inputs).
 int launch_policy();
-inline bool small_launch(int BH, int max_s, bool causal) {
+constexpr int kSmallLaunchFwd = 0, kSmallLaunchDq = 1;
+inline bool small_launch(int kernel, int BH, int max_s, bool causal, bool dropout) {
   const int policy = launch_policy() & 3;
   if (policy != 0) return policy == 2;
-  const int64_t wgs = (int64_t)BH * ((max_s + 127) / 128);
-  (void)causal;
-  return wgs < 3 * 256;
+  const int64_t wgs = (int64_t)BH * ((max_s + 127) / 128);  // x = wgs / 256 compute units
+  if (kernel == kSmallLaunchFwd) return max_s > 128 && (wgs < 2 * 256 || (dropout && wgs < 3 * 256));
+  return wgs >= 256 && wgs < 2 * 256 && (causal || dropout);
 }
 
 // Launchers (defined in fa_fwd.hip / fa_bwd.hip / fa_aux.hip).  Return hipError_t of the launch.
