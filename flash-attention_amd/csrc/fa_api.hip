@@ -137,6 +137,18 @@ int build_maps(const int32_t* blockmask, unsigned char* ws, const SparseLayout& 
   return FA_OK;
 }
 
+// Causal launches (fa_params.h, map_tile): how many (batch, head) pairs of an XCD are in flight together.  All of them while
+// their K and V stay within about twice an XCD's 4 MB of L2 (dearest-first over everything balances best, and what the L2
+// misses then costs nothing measurable); beyond that as many as hold 6 MB of K and V, and at least four (fewer cost more in
+// balance than their traffic saves).  Measured: profiles/causal_tile_order_hbm_traffic.md.
+int causal_tile_group(int batch, int nheads, int head_dim, int max_seqlen_k) {
+  const int64_t pairs = ((int64_t)batch * nheads + 7) / 8;
+  const int64_t kv_bytes = (int64_t)max_seqlen_k * head_dim * 2 * 2;
+  if (pairs * kv_bytes <= ((int64_t)8 << 20)) return 0;
+  const int64_t g = ((int64_t)6 << 20) / kv_bytes;
+  return (int)(g < 4 ? 4 : g);
+}
+
 fa::PhiloxKey make_key(uint64_t seed, uint64_t offset) {
   fa::PhiloxKey k;
   k.k0 = (uint32_t)seed;
@@ -219,6 +231,7 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
   p.max_sq = a->max_seqlen_q; p.max_sk = a->max_seqlen_k;
   p.sq_r = r.sq_r;
   p.nq_tiles = (a->max_seqlen_q + fa::kFwdBM - 1) / fa::kFwdBM;
+  p.tile_group = a->is_causal ? causal_tile_group(a->batch, a->nheads, a->head_dim, a->max_seqlen_k) : 0;
   p.scale = a->softmax_scale;
   p.scale_log2 = a->softmax_scale * fa::kLog2e;
   p.rp_keep = 1.f / p_keep;
@@ -354,6 +367,7 @@ int bwd_impl(const fa_bwd_args* a, bool want_block, void* ev_main_start = nullpt
   p.sq_r = r.sq_r; p.lse_stride = a->lse_seq_stride;
   p.nk_tiles = (a->max_seqlen_k + fa::kBwdBN - 1) / fa::kBwdBN;
   p.nq_tiles = (a->max_seqlen_q + fa::kFwdBM - 1) / fa::kFwdBM;
+  p.tile_group = a->is_causal ? causal_tile_group(a->batch, a->nheads, a->head_dim, a->max_seqlen_k) : 0;
   p.scale = a->softmax_scale;
   p.scale_log2 = a->softmax_scale * fa::kLog2e;
   p.p_keep = p_keep;

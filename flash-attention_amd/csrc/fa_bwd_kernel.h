@@ -85,7 +85,7 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasT
 
   // XCD-aware id map (see map_tile): the key tiles of one (batch, head) share one XCD's L2 copy of Q and dO.
   int bh, kt;  // under a causal mask the first key tiles see the most query rows: rank order is already heavy-first
-  if (!map_tile<kCausal>(blockIdx.x, p.nk_tiles, p.B * p.H, &bh, &kt)) return;
+  if (!map_tile<kCausal>(blockIdx.x, p.nk_tiles, p.B * p.H, &bh, &kt, p.tile_group)) return;
   const int b = bh / p.H, h = bh % p.H;
 
   int q_begin = 0, Lq = 0, k_begin, Lk;
@@ -529,7 +529,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
 
   int bh, rank;
   const int n_splits = p.n_splits > 1 ? p.n_splits : 1;  // key splits per query tile (see BwdParams)
-  if (!map_tile<kCausal>(blockIdx.x, p.nq_tiles * n_splits, p.B * p.H, &bh, &rank)) return;
+  if (!map_tile<kCausal>(blockIdx.x, p.nq_tiles * n_splits, p.B * p.H, &bh, &rank, p.tile_group)) return;
   const int split = rank % n_splits;
   rank /= n_splits;
   const int qt = kCausal ? p.nq_tiles - 1 - rank : rank;

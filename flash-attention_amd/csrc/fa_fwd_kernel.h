@@ -69,7 +69,7 @@ __global__ void __launch_bounds__(256, (!kDropout && kBias == 0 && D <= 64) ? 4 
   // one XCD's L2 copy of K and V.
   int bh, rank;
   const int n_splits = p.n_splits > 1 ? p.n_splits : 1;   // key splits per query tile (see FwdParams)
-  if (!map_tile<kCausal>(blockIdx.x, p.nq_tiles * n_splits, p.B * p.H, &bh, &rank)) return;
+  if (!map_tile<kCausal>(blockIdx.x, p.nq_tiles * n_splits, p.B * p.H, &bh, &rank, p.tile_group)) return;
   const int split = rank % n_splits;
   rank /= n_splits;
   const int qt = kCausal ? p.nq_tiles - 1 - rank : rank;  // under a causal mask the last query tiles cost most

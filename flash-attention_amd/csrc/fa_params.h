@@ -43,6 +43,7 @@ struct FwdParams {
   int max_sq, max_sk;  // caller's bounds on the sequence lengths; longer sequences are truncated to them
   int sq_r;  // rounded max_seqlen_q = innermost extent of lse
   int nq_tiles;
+  int tile_group;    // causal launches: (batch, head) pairs of an XCD in flight together (map_tile); 0 = all
   float scale;       // softmax_scale
   float scale_log2;  // softmax_scale * log2(e)
   float rp_keep;     // 1 / keep probability
@@ -108,6 +109,7 @@ struct BwdParams {
   int lse_stride;  // innermost extent of lse
   int nk_tiles;      // key tiles of the dK/dV kernel
   int nq_tiles;      // query tiles of the dQ kernel
+  int tile_group;    // causal launches: (batch, head) pairs of an XCD in flight together (map_tile); 0 = all
   float scale;
   float scale_log2;
   float p_keep;
@@ -155,9 +157,22 @@ FA_DEVICE bool seq_extent(const int32_t* cu, int b, int total, int max_len, int*
 //     most expensive tiles of all (batch, head) pairs start first; batch*head is padded to a multiple of 8 so that a
 //     given (batch, head) still always lands on the same XCD.
 template <bool kTileMajor>
-FA_DEVICE bool map_tile(int block, int tiles_per_bh, int BH, int* bh, int* rank) {
+FA_DEVICE bool map_tile(int block, int tiles_per_bh, int BH, int* bh, int* rank, int group = 0) {
   if (kTileMajor) {
     const int bhp = (BH + 7) & ~7;
+    const int P = bhp >> 3;  // (batch, head) pairs per XCD
+    if (group > 0 && group < P) {
+      // Long sequences: an XCD that streams the K and V of all its pairs at once reads them from memory again for every
+      // query tile (they exceed its L2 many times over).  The pairs of an XCD are therefore taken `group` at a time -
+      // ranks outermost inside a group, the groups one after the other - so that what is in flight shares a few pairs' keys.
+      const int x = block & 7, j = block >> 3;
+      const int g = j / (group * tiles_per_bh);
+      const int r = j - g * group * tiles_per_bh;
+      const int members = P - g * group < group ? P - g * group : group;
+      *rank = r / members;
+      *bh = x + 8 * (g * group + (r - *rank * members));
+      return *bh < BH && *rank < tiles_per_bh;
+    }
     // A grid small enough to be resident all at once (up to 4 workgroups on each of the 256 compute units) is dealt
     // out in one go, compute unit c getting ids c, c + 256, ...: then every odd group of 256 ids is walked backwards
     // (in steps of 8, so that id % 8 is kept), and a compute unit that got one of the dearest tiles of a group gets
