@@ -73,6 +73,9 @@ class Workload:
             self.fwd_flops = 4.0 * B * H * D * 16 * 256 * float(blockmask.sum())
             from flash_attn.flash_blocksparse_attn_interface import convert_blockmask
             self.blockmask = convert_blockmask(blockmask.cuda(), causal=False)  # the entry points' own column-major form
+            # the order the workgroups take the 16-row blocks in, worked out once per layout (as the autograd functions do)
+            from flash_attn import flash_attn_gfx950 as be
+            self.row_order = be.blockmask_row_order(blockmask.cuda()) if os.environ.get("FA_BENCH_ROW_ORDER", "1") != "0" else None
         self.bytes_fwd = 4 * total * H * D * 2 + 4 * B * H * self.max_s          # q,k,v read + o written, lse
         self.bytes_bwd = 8 * total * H * D * 2 + 2 * 4 * B * H * self.max_s      # q,k,v,o,do read + dq,dk,dv written
         # dropout (dense): the forward leaves its keep decisions, one bit per score, for the backward's two kernels, as
@@ -90,7 +93,7 @@ class Workload:
         q, k, v = self.q, self.k, self.v
         if self.blockmask is not None:
             self.out, self.lse = be.fwd_block(q, k, v, self.cu, self.cu, self.blockmask, self.max_s, self.max_s, self.p,
-                                              self.scale, self.causal, False, None)
+                                              self.scale, self.causal, False, None, row_order=self.row_order)
             return
         self.out, self.lse = be.fwd(q, k, v, self.cu, self.cu, self.max_s, self.max_s, self.p, self.scale, False,
                                     self.causal, False, None, self.alibi, self.keep_words)
@@ -102,7 +105,7 @@ class Workload:
             if events is not None:
                 events[0].record()
             be.bwd_block(self.dout, q, k, v, self.out, self.lse, dq, dk, dv, self.cu, self.cu, self.blockmask, self.max_s,
-                         self.max_s, self.p, self.scale, self.causal, None)
+                         self.max_s, self.p, self.scale, self.causal, None, row_order=self.row_order)
             if events is not None:
                 events[1].record()  # whole backward: the sparse entry point has no per-kernel hook
             return

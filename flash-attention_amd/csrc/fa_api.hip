@@ -79,7 +79,7 @@ Rounded round_seqlens(int head_dim, int max_sq, int max_sk, bool blocksparse) {
 
 struct SparseLayout {
   int nrb, ncb, nqt, ncw, nrw;
-  size_t offr, offq, offc, bytes;
+  size_t offr, offq, offc, offi, bytes;
 };
 
 SparseLayout sparse_layout(const Rounded& r) {
@@ -92,7 +92,8 @@ SparseLayout sparse_layout(const Rounded& r) {
   s.offr = 0;
   s.offq = s.offr + align16((size_t)s.nrb * s.ncw * 8);
   s.offc = s.offq + align16((size_t)s.nqt * s.ncw * 8);
-  s.bytes = s.offc + align16((size_t)s.ncb * s.nrw * 8);
+  s.offi = s.offc + align16((size_t)s.ncb * s.nrw * 8);  // inverse of the row order
+  s.bytes = s.offi + align16((size_t)s.nrb * 4);
   return s;
 }
 
@@ -119,13 +120,14 @@ SplitPlan split_plan(int batch, int nheads, int head_dim, int total_q, int max_s
   return sp;
 }
 
-int build_maps(const int32_t* blockmask, unsigned char* ws, const SparseLayout& sl, fa::SparseMaps* out,
-               hipStream_t stream) {
+int build_maps(const int32_t* blockmask, const int32_t* row_order, unsigned char* ws, const SparseLayout& sl,
+               fa::SparseMaps* out, hipStream_t stream) {
   FA_LAUNCH(fa::launch_fill_f32(reinterpret_cast<float*>(ws), sl.bytes / 4, 0.f, stream));
   FA_LAUNCH(fa::launch_build_sparse_maps(blockmask, reinterpret_cast<uint64_t*>(ws + sl.offr),
                                          reinterpret_cast<uint64_t*>(ws + sl.offq),
                                          reinterpret_cast<uint64_t*>(ws + sl.offc), sl.nrb, sl.ncb, fa::kFwdBM, sl.nqt,
-                                         sl.ncw, sl.nrw, stream));
+                                         sl.ncw, sl.nrw, row_order, reinterpret_cast<int32_t*>(ws + sl.offi), stream));
+  out->order = row_order;
   out->rbits = reinterpret_cast<const uint64_t*>(ws + sl.offr);
   out->qbits = reinterpret_cast<const uint64_t*>(ws + sl.offq);
   out->cbits = reinterpret_cast<const uint64_t*>(ws + sl.offc);
@@ -209,7 +211,9 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
     if (!a->workspace || a->workspace_bytes < sl.bytes)
       return fail(FA_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", sl.bytes, a->workspace_bytes);
     FA_REQUIRE(aligned16(a->workspace), "workspace must be 16-byte aligned");
-    rc = build_maps(a->blockmask, reinterpret_cast<unsigned char*>(a->workspace), sl, &p.sp, stream);
+    FA_REQUIRE(!a->row_order || (reinterpret_cast<uintptr_t>(a->row_order) & 3) == 0, "row_order must be 4-byte aligned");
+    rc = build_maps(a->blockmask, a->is_causal ? nullptr : a->row_order, reinterpret_cast<unsigned char*>(a->workspace), sl,
+                    &p.sp, stream);
     if (rc) return rc;
   }
   if (a->zero_tensors) {  // fmha_api.cpp:256-260
@@ -340,7 +344,8 @@ int bwd_impl(const fa_bwd_args* a, bool want_block, void* ev_main_start = nullpt
   fa::BwdParams p;
   memset(&p, 0, sizeof(p));
   if (sparse) {
-    rc = build_maps(a->blockmask, ws, sl, &p.sp, stream);
+    FA_REQUIRE(!a->row_order || (reinterpret_cast<uintptr_t>(a->row_order) & 3) == 0, "row_order must be 4-byte aligned");
+    rc = build_maps(a->blockmask, a->is_causal ? nullptr : a->row_order, ws, sl, &p.sp, stream);
     if (rc) return rc;
   }
   if (a->zero_tensors) {  // fmha_api.cpp:406-411

@@ -27,8 +27,19 @@ __global__ void zero_rows_kernel(uint16_t* base, int64_t rs, int64_t hs, int tot
 
 // blockmask: [ncb][nrb] int32, entries 4*rowblock + flags for the active 16-row blocks of each 256-key
 // column block, -1 padded (flash_blocksparse_attn_interface.py:8-40; read as fmha_blockmask.h:41-53 does).
+// inv[order[i]] = i + 1: where each row block stands in the row order (entries that are no row block are skipped; inv was
+// cleared: 0 = the order does not list the row block, it belongs to no tile)
+__global__ void invert_order_kernel(const int32_t* order, int32_t* inv, int nrb) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= nrb) return;
+  const int rb = order[i];
+  if (rb >= 0 && rb < nrb) inv[rb] = i + 1;
+}
+
+// inv: null, or the position of every row block in the row order (then query tile t owns the row blocks at positions
+// rpq t .. rpq t + rpq - 1, not the row blocks with those numbers)
 __global__ void sparse_maps_kernel(const int32_t* blockmask, uint32_t* rbits, uint32_t* qbits, uint32_t* cbits, int nrb,
-                                   int ncb, int rpq, int nqt, int ncw, int nrw) {
+                                   int ncb, int rpq, int nqt, int ncw, int nrw, const int32_t* inv) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= nrb * ncb) return;
   const int cb = i / nrb;
@@ -38,7 +49,8 @@ __global__ void sparse_maps_kernel(const int32_t* blockmask, uint32_t* rbits, ui
   if (rb >= nrb) return;
   // the 64-bit words are addressed as pairs of 32-bit words (bit b of a word: half b / 32, bit b % 32)
   atomicOr(rbits + ((int64_t)rb * ncw * 2 + (cb >> 5)), 1u << (cb & 31));
-  if (rb / rpq < nqt) atomicOr(qbits + ((int64_t)(rb / rpq) * ncw * 2 + (cb >> 5)), 1u << (cb & 31));
+  const int pos = inv ? inv[rb] - 1 : rb;
+  if (pos >= 0 && pos / rpq < nqt) atomicOr(qbits + ((int64_t)(pos / rpq) * ncw * 2 + (cb >> 5)), 1u << (cb & 31));
   atomicOr(cbits + ((int64_t)cb * nrw * 2 + (rb >> 5)), 1u << (rb & 31));
 }
 
@@ -106,11 +118,19 @@ hipError_t launch_zero_rows(void* base, int64_t row_stride, int64_t head_stride,
 }
 
 hipError_t launch_build_sparse_maps(const int32_t* blockmask, uint64_t* rbits, uint64_t* qbits, uint64_t* cbits, int nrb,
-                                    int ncb, int rows_per_qt, int nqt, int ncw, int nrw, hipStream_t stream) {
+                                    int ncb, int rows_per_qt, int nqt, int ncw, int nrw, const int32_t* order, int32_t* inv,
+                                    hipStream_t stream) {
   const int n = nrb * ncb;
+  if (order && inv) {  // (inv was cleared by the caller)
+    hipLaunchKernelGGL(invert_order_kernel, dim3((nrb + 255) / 256), dim3(256), 0, stream, order, inv, nrb);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+  } else {
+    inv = nullptr;
+  }
   hipLaunchKernelGGL(sparse_maps_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, blockmask,
                      reinterpret_cast<uint32_t*>(rbits), reinterpret_cast<uint32_t*>(qbits),
-                     reinterpret_cast<uint32_t*>(cbits), nrb, ncb, rows_per_qt / 16, nqt, ncw, nrw);
+                     reinterpret_cast<uint32_t*>(cbits), nrb, ncb, rows_per_qt / 16, nqt, ncw, nrw, inv);
   return hipGetLastError();
 }
 

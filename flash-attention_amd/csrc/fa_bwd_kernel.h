@@ -539,7 +539,6 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
   if (!seq_extent(p.cu_q, b, p.total_q, p.max_sq, &q_begin, &Lq)) return;
   if (!seq_extent(p.cu_k, b, p.total_k, p.max_sk, &k_begin, &Lk)) Lk = 0;  // no keys: dQ = 0
   const int m0 = qt * BM;
-  if (m0 >= Lq) return;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -547,7 +546,25 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
   const int rs = KS > 1 ? wave % Cfg::RW : wave;  // this wave's 32-row slab of the tile
   const int kh = KS > 1 ? wave / Cfg::RW : 0;     // ... and its share of every key tile's 32-key blocks
   const int mw = m0 + rs * 32;
-  const int qrow = mw + c;
+  int qrow = mw + c;
+  // Sparse: the wave's 32 rows are two 16-row blocks, consecutive ones or two that the row order puts next to each other
+  // (as in fa_fwd_kernel); rows of no block count as lying past the end
+  int rb_a = -1, rb_b = -1;
+  bool wave_live = mw < Lq;
+  if (kSparse) {
+    const bool ordered = !kCausal && p.sp.order != nullptr;
+    slab_row_blocks(p.sp, ordered, qt, rs, &rb_a, &rb_b);
+    const int rbl = c < 16 ? rb_a : rb_b;
+    qrow = rbl >= 0 ? rbl * 16 + (c & 15) : 0x3fffffff;
+    wave_live = (rb_a >= 0 && rb_a * 16 < Lq) || (rb_b >= 0 && rb_b * 16 < Lq);
+    if (ordered) {
+      if (!__syncthreads_or(wave_live)) return;  // no row of the workgroup exists
+    } else if (m0 >= Lq) {
+      return;
+    }
+  } else if (m0 >= Lq) {
+    return;
+  }
 
   // ---- Q and dO fragments (B operands), lse and Dk of this lane's query row.  Dk = keep * rowsum(dO o O) is computed
   // here (fmha_dgrad_kernel_1xN_loop.h:15-30 does it on the first column block) and stored to softmax_d, which the
@@ -613,8 +630,8 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
       if ((cb >> 6) != bits_word) {
         bits_word = cb >> 6;
         tile_bits = uniform64(p.sp.qbits[(int64_t)qt_u * p.sp.ncw + bits_word]);
-        const int rb = (qrow >> 4) < p.sp.nrb ? (qrow >> 4) : p.sp.nrb - 1;
-        row_bits = p.sp.rbits[(int64_t)rb * p.sp.ncw + bits_word];
+        const int rbl = c < 16 ? rb_a : rb_b;
+        row_bits = rbl >= 0 ? p.sp.rbits[(int64_t)rbl * p.sp.ncw + bits_word] : 0;
       }
       const uint64_t rest = tile_bits >> (cb & 63);  // bit 0: this tile's block
       if (rest & 1) break;
@@ -714,7 +731,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
     const T* const Vs = Ks + BN * D;
     buf ^= 1;
 
-    bool wave_work = mw < Lq;  // a wave whose 32 rows all lie past the sequence's end only helps with the staging
+    bool wave_work = wave_live;  // a wave whose 32 rows all lie past the sequence's end only helps with the staging
     const int kb0 = kh * KBW;  // this wave's 32-key blocks of the tile: kb0, kb0 + 1, ... (all of them without a key split)
     if (kCausal && n0 + kb0 * 32 > mw + 31) wave_work = false;  // every key of the wave's share is above its diagonal
     if (KS > 1 && n0 + kb0 * 32 >= Lk) wave_work = false;       // ... or past the last key
@@ -863,9 +880,11 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
   for (int i = 0; i < (32 * CH + 63) / 64; i++) {
     const int ch = lane + i * 64;
     const int row = ch / CH, col = (ch % CH) * 8;
-    if ((32 * CH % 64 == 0 || ch < 32 * CH) && mw + row < Lq) {
+    int orow = mw + row;  // (sparse: the wave's rows are those of its two row blocks)
+    if (kSparse) orow = (row < 16 ? rb_a : rb_b) < 0 ? 0x3fffffff : (row < 16 ? rb_a : rb_b) * 16 + (row & 15);
+    if ((32 * CH % 64 == 0 || ch < 32 * CH) && orow < Lq) {
       u32x4 val = *reinterpret_cast<const u32x4*>(Os + row * OS + col);
-      st_global16(gbase + (int64_t)(mw + row) * p.dq_rs + col, val);
+      st_global16(gbase + (int64_t)orow * p.dq_rs + col, val);
     }
   }
 }

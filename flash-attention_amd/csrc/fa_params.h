@@ -22,7 +22,27 @@ struct SparseMaps {
   int nqt;   // forward query tiles
   int ncw;   // 64-bit words per row of rbits / qbits
   int nrw;   // 64-bit words per row of cbits
+  // Row order (or null = 0, 1, 2, ...): a permutation of the 16-row blocks.  The forward and the dQ kernel give query tile t
+  // the row blocks order[8 t .. 8 t + 7] (qbits is built for those), so that a caller who lists row blocks with similar key
+  // blocks next to each other makes a workgroup stage few tiles that only one of its row blocks needs.  Not used under a
+  // causal mask (the tile ranges there follow the rows' positions).
+  const int32_t* order;
 };
+
+// The two 16-row blocks of the 32-row slab `slab` (0 .. 3) of query tile qt: positions 8 qt + 2 slab and + 1 of the row
+// order; -1 = none (past the last row block, or an entry that is not a row block).
+FA_DEVICE void slab_row_blocks(const SparseMaps& sp, bool ordered, int qt, int slab, int* a, int* b) {
+  const int pos = 8 * qt + 2 * slab;
+  int ra = pos < sp.nrb ? pos : -1, rb = pos + 1 < sp.nrb ? pos + 1 : -1;
+  if (ordered) {
+    if (ra >= 0) ra = sp.order[pos];
+    if (rb >= 0) rb = sp.order[pos + 1];
+    if (ra >= sp.nrb) ra = -1;
+    if (rb >= sp.nrb) rb = -1;
+  }
+  *a = __builtin_amdgcn_readfirstlane(ra);
+  *b = __builtin_amdgcn_readfirstlane(rb);
+}
 
 // What is added to the scaled scores before the softmax (template parameter kBias of the kernels)
 constexpr int kBiasNone = 0;    // nothing
@@ -255,8 +275,10 @@ hipError_t launch_dump_probs(const DumpParams& p, int dtype, hipStream_t stream)
 // which: 0 = dQ kernel, 1 = dK/dV kernel
 hipError_t launch_bwd(const BwdParams& p, int which, int dtype, int head_dim, bool causal, bool dropout, bool sparse,
                       hipStream_t stream);
+// order / inv: null, or the row order (SparseMaps::order) and nrb ints of scratch for its inverse
 hipError_t launch_build_sparse_maps(const int32_t* blockmask, uint64_t* rbits, uint64_t* qbits, uint64_t* cbits, int nrb,
-                                    int ncb, int rows_per_qt, int nqt, int ncw, int nrw, hipStream_t stream);
+                                    int ncb, int rows_per_qt, int nqt, int ncw, int nrw, const int32_t* order, int32_t* inv,
+                                    hipStream_t stream);
 hipError_t launch_fill_f32(float* p, size_t n, float value, hipStream_t stream);
 // Zero a strided [total, H, D] tensor of 16-bit elements.
 hipError_t launch_zero_rows(void* base, int64_t row_stride, int64_t head_stride, int total, int H, int D,

@@ -20,7 +20,7 @@ LIB_NAME = "libflash_attn_gfx950.so"
 LIB_PATH = os.path.join(_HERE, LIB_NAME)
 
 FA_FP16, FA_BF16 = 0, 1
-FA_ABI_VERSION = 4
+FA_ABI_VERSION = 5
 
 _c_i32p = ctypes.c_void_p
 
@@ -56,6 +56,7 @@ class FwdArgs(ctypes.Structure):
         ("keep_words", ctypes.c_void_p), ("keep_words_bytes", ctypes.c_size_t),
         ("attn_bias", ctypes.c_void_p), ("bias_batch_stride", ctypes.c_int64), ("bias_head_stride", ctypes.c_int64),
         ("bias_row_stride", ctypes.c_int64),
+        ("row_order", ctypes.c_void_p),
     ]
 
 
@@ -90,6 +91,7 @@ class BwdArgs(ctypes.Structure):
         ("bias_row_stride", ctypes.c_int64),
         ("dbias", ctypes.c_void_p), ("dbias_batch_stride", ctypes.c_int64), ("dbias_head_stride", ctypes.c_int64),
         ("dbias_row_stride", ctypes.c_int64),
+        ("row_order", ctypes.c_void_p),
     ]
 
 
@@ -328,8 +330,64 @@ def _keep_words_arg(a, keep_words, dev, sparse):
     a.keep_words, a.keep_words_bytes = keep_words.data_ptr(), keep_words.numel()
 
 
+def _row_order_arg(a, row_order, sq_r, dev):
+    if row_order is None:
+        return
+    _check(row_order.device == dev and row_order.dtype == torch.int32 and row_order.is_contiguous() and
+           row_order.numel() == sq_r // 16, "row_order must be a contiguous int32 tensor of max_seqlen_q_rounded / 16 row blocks "
+                                            "on the tensors' device (see blockmask_row_order)")
+    a.row_order = row_order.data_ptr()
+
+
+def blockmask_row_order(layout):
+    """An order of the 16-row blocks of a block-sparse layout ((rows / 16, keys / 256) of 0 / 1) for the `row_order` argument
+    of fwd_block / bwd_block.  A workgroup of the forward and of the dQ kernel owns eight consecutive entries and stages every
+    key tile that any of the eight lists; each of its waves owns two consecutive entries and computes on every tile that
+    either of the two lists.  Greedy: a group starts with the fullest row block left and takes, seven times, the row block
+    that adds the fewest key blocks to the group's set (most shared ones on a tie); inside a group the two row blocks with
+    the smallest union are paired, then the next two.  If that saves less than 5 % of the staged tiles against the plain
+    order 0, 1, 2, ... (layouts made of whole 128-row tiles), the plain order is returned.  int32 tensor on the layout's
+    device; computed on the host."""
+    import numpy as np
+    m = (layout != 0).cpu().numpy()
+    nr, nc = m.shape
+    left = np.ones(nr, dtype=bool)
+    counts = m.sum(1)
+    order, staged = [], 0
+    while left.any():
+        seed = int(np.argmax(np.where(left, counts, -1)))
+        left[seed] = False
+        group, union = [seed], m[seed].copy()
+        while len(group) < 8 and left.any():
+            added = (m & ~union).sum(1)
+            shared = (m & union).sum(1)
+            score = np.where(left, added * (nc + 1) - shared, np.iinfo(np.int64).max)
+            best = int(np.argmin(score))
+            left[best] = False
+            group.append(best)
+            union |= m[best]
+        staged += int(union.sum())
+        rest = sorted(group)
+        while len(rest) >= 2:  # pair the two with the smallest union (the wave's work), ties: the lowest row blocks
+            best = None
+            for i in range(len(rest)):
+                for j in range(i + 1, len(rest)):
+                    u = int((m[rest[i]] | m[rest[j]]).sum())
+                    if best is None or u < best[0]:
+                        best = (u, i, j)
+            _, i, j = best
+            order += [rest[i], rest[j]]
+            rest = [r for n, r in enumerate(rest) if n not in (i, j)]
+        order += rest
+    plain = sum(int(m[i:i + 8].any(0).sum()) for i in range(0, nr, 8))
+    if staged > 0.95 * plain:
+        order = list(range(nr))
+    return torch.tensor(order, dtype=torch.int32, device=layout.device)
+
+
 def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
-              zero_tensors, is_causal, return_softmax, gen, alibi_slopes=None, keep_words=None, attn_bias=None):
+              zero_tensors, is_causal, return_softmax, gen, alibi_slopes=None, keep_words=None, attn_bias=None,
+              row_order=None):
     lib = load_library()
     code = _dtype_code(q)
     _check(q.dim() == 3, "q must be (total_q, nheads, head_size)")
@@ -383,6 +441,8 @@ def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_
         a.alibi_slopes = _check_alibi(alibi_slopes, nheads, dev, sparse)
         _keep_words_arg(a, keep_words, dev, sparse)
         bias_t = _bias_arg(a, attn_bias, q, batch, nheads, max_seqlen_q, max_seqlen_k, sparse)  # noqa: F841 (kept alive)
+        if sparse:
+            _row_order_arg(a, row_order, sq_r, dev)
         rc = (lib.fa_fwd_block if sparse else lib.fa_fwd)(ctypes.byref(a))
         if rc != 0:
             _raise(rc, lib)
@@ -391,7 +451,7 @@ def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_
 
 def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q,
               max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen, main_kernel_events=None,
-              alibi_slopes=None, keep_words=None, attn_bias=None, dbias=None):
+              alibi_slopes=None, keep_words=None, attn_bias=None, dbias=None, row_order=None):
     lib = load_library()
     code = _dtype_code(q)
     _check(q.dim() == 3, "q must be (total_q, nheads, head_size)")
@@ -460,6 +520,8 @@ def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seql
                    "dbias must be (batch, nheads, >= max_seqlen_q, >= max_seqlen_k) in q's dtype, keys contiguous")
             a.dbias = dbias.data_ptr()
             a.dbias_batch_stride, a.dbias_head_stride, a.dbias_row_stride = dbias.stride(0), dbias.stride(1), dbias.stride(2)
+        if sparse:
+            _row_order_arg(a, row_order, sq_r, dev)
         if main_kernel_events is not None and not sparse:  # (start, stop) torch.cuda.Event created with enable_timing=True
             for ev in main_kernel_events:
                 if not ev.cuda_event:  # torch creates the HIP event lazily, on first record
@@ -498,19 +560,20 @@ def bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
 
 
 def fwd_block(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
-              is_causal, return_softmax, gen=None):
-    """mha_fwd_block (fmha_api.cpp:451-573)."""
+              is_causal, return_softmax, gen=None, row_order=None):
+    """mha_fwd_block (fmha_api.cpp:451-573).  row_order (extension): None, or the int32 order of the 16-row blocks from
+    blockmask_row_order() of the layout: the kernels' workgroups then own row blocks with similar key-block lists."""
     _check(blockmask is not None, "blockmask is required")
     return _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout,
-                     softmax_scale, False, is_causal, return_softmax, gen)
+                     softmax_scale, False, is_causal, return_softmax, gen, row_order=row_order)
 
 
 def bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q,
-              max_seqlen_k, p_dropout, softmax_scale, is_causal, gen=None):
-    """mha_bwd_block (fmha_api.cpp:575-718)."""
+              max_seqlen_k, p_dropout, softmax_scale, is_causal, gen=None, row_order=None):
+    """mha_bwd_block (fmha_api.cpp:575-718).  row_order: as in fwd_block."""
     _check(blockmask is not None, "blockmask is required")
     return _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q,
-                     max_seqlen_k, p_dropout, softmax_scale, False, is_causal, gen)
+                     max_seqlen_k, p_dropout, softmax_scale, False, is_causal, gen, row_order=row_order)
 
 
 def _check_rows(name, t):

@@ -36,10 +36,35 @@ def convert_blockmask(blockmask, causal):
     return torch.gather(code, 0, order).T.contiguous().to(torch.int32)
 
 
+_ROW_ORDERS = {}  # converted blockmask (address, shape, version) -> row order
+
+
+def _row_order(blockmask, causal):
+    """The order of the 16-row blocks the kernels' workgroups take them in (flash_attn_gfx950.blockmask_row_order), worked
+    out once per converted blockmask (the first call reads the blockmask back to the host).  Any order gives the same
+    results; a cache entry that outlived its tensor costs speed at worst."""
+    if causal:
+        return None
+    key = (blockmask.data_ptr(), tuple(blockmask.shape), blockmask._version, str(blockmask.device))
+    order = _ROW_ORDERS.get(key)
+    if order is None:
+        conv = blockmask.cpu()
+        ncol, nrow = conv.shape
+        layout = torch.zeros(nrow, ncol, dtype=torch.bool)
+        cols = torch.arange(ncol)[:, None].expand(ncol, nrow)
+        live = (conv >= 0) & ((conv >> 2) < nrow)
+        layout[(conv >> 2)[live].long(), cols[live]] = True
+        order = _backend.blockmask_row_order(layout).to(blockmask.device)
+        if len(_ROW_ORDERS) >= 64:
+            _ROW_ORDERS.clear()
+        _ROW_ORDERS[key] = order
+    return order
+
+
 def _flash_blocksparse_attn_forward(qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal,
                                     return_softmax):
     res = _backend.fwd_block(qkv[:, 0], qkv[:, 1], qkv[:, 2], cu_seqlens, cu_seqlens, blockmask, max_s, max_s,
-                             dropout_p, softmax_scale, causal, return_softmax, None)
+                             dropout_p, softmax_scale, causal, return_softmax, None, row_order=_row_order(blockmask, causal))
     return res[0], res[1], (res[2] if return_softmax else None)
 
 
@@ -48,7 +73,7 @@ def _flash_blocksparse_attn_backward(dout, qkv, out, S_dmask, softmax_lse, cu_se
     dqkv = torch.empty_like(qkv)
     _backend.bwd_block(dout.contiguous(), qkv[:, 0], qkv[:, 1], qkv[:, 2], out, softmax_lse, dqkv[:, 0], dqkv[:, 1],
                        dqkv[:, 2], cu_seqlens, cu_seqlens, blockmask, max_s, max_s, dropout_p, softmax_scale, causal,
-                       None)
+                       None, row_order=_row_order(blockmask, causal))
     return dqkv
 
 

@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define FA_ABI_VERSION 4
+#define FA_ABI_VERSION 5
 
 enum fa_dtype { FA_FP16 = 0, FA_BF16 = 1 };
 
@@ -89,6 +89,14 @@ typedef struct fa_fwd_args {
    * next multiple of 8 keys past max_seqlen_k (inside the row stride).  Not with a blockmask, not with alibi_slopes. */
   const void* attn_bias;
   int64_t bias_batch_stride, bias_head_stride, bias_row_stride;
+  /* Block-sparse only (no counterpart in the reference).  NULL, or a device array of max_seqlen_q_rounded / 16 int32: a
+   * permutation of the 16-row blocks.  A workgroup of the forward and of the backward's dQ kernel owns eight consecutive
+   * entries of it (without it: eight consecutive row blocks) and has to stage every key tile that any of the eight lists;
+   * an order that puts row blocks with similar key-block lists next to each other saves that staging (at 25 % of
+   * independently drawn blocks about a third of it).  Results do not depend on the order beyond rounding.  The entries
+   * must be distinct row blocks (a row block that is not listed is not computed: its rows of o / dq are left unwritten);
+   * ignored with is_causal. */
+  const int32_t* row_order;
 } fa_fwd_args;
 
 /* Arguments of the backward pass.  Mirrors mha_bwd (fmha_api.cpp:302-321) and, when `blockmask`
@@ -147,6 +155,8 @@ typedef struct fa_bwd_args {
    * none past a sequence's end): the caller clears the tensor first. */
   void* dbias;
   int64_t dbias_batch_stride, dbias_head_stride, dbias_row_stride;
+  /* as in fa_fwd_args (the backward need not be given the order the forward had) */
+  const int32_t* row_order;
 } fa_bwd_args;
 
 /* replaces flash_attn_cuda.fwd -> mha_fwd, csrc/flash_attn/fmha_api.cpp:173-299 */

@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol(lib):
     assert declared_bench == set(be.BENCH_SYMBOLS) and not (declared & declared_bench)
     for name in declared | declared_bench:
         assert hasattr(lib, name), name
-    assert lib.fa_abi_version() == be.FA_ABI_VERSION == 4
+    assert lib.fa_abi_version() == be.FA_ABI_VERSION == 5
 
 
 def test_struct_layout_matches_library(lib):

@@ -1045,6 +1045,45 @@ def test_blocksparse_random_layouts_sweep():
         check_against_oracle(ours, ref, half, dtype, what=what)
 
 
+@pytest.mark.parametrize("D,N,dtype", [(64, 1280, torch.float16), (32, 300, torch.bfloat16), (128, 700, torch.float16)])
+def test_blocksparse_row_order(D, N, dtype):
+    """the 16-row blocks a workgroup owns may be any eight of a caller's order: no order, the greedy grouping the autograd
+    functions use, and a random permutation give the same results within rounding, each within the parity bar"""
+    from flash_attn import flash_attn_gfx950 as be
+    from flash_attn.flash_blocksparse_attn_interface import convert_blockmask
+    H, lens = 2, [N, N - 150, 20]
+    sq_r, sk_r = be.round_seqlens(D, N, N, True)
+    layout = _layout(sq_r // 16, sk_r // 256, 0.25, N + D)
+    layout[5] = False
+    q, k, v, do = _inputs(lens, lens, H, D, dtype, N)
+    cu = _cu(lens, "cpu")
+    conv = convert_blockmask(layout.cuda(), causal=False)
+    nrb = sq_r // 16
+    greedy = be.blockmask_row_order(layout.cuda())
+    assert sorted(greedy.tolist()) == list(range(nrb))
+    rand = torch.randperm(nrb, generator=torch.Generator().manual_seed(3)).to(torch.int32).cuda()
+    ref = orc.varlen_attention(q, k, v, cu, cu, None, False, layout=layout.numpy(), dout=do)
+    half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu.tolist(), cu.tolist(), D ** -0.5, False, layout=layout.numpy(),
+                          dout=do.cuda())
+    qg, kg, vg, dog, cug = q.cuda(), k.cuda(), v.cuda(), do.cuda(), cu.cuda()
+    res = []
+    for order in (None, greedy, rand):
+        o, lse = be.fwd_block(qg, kg, vg, cug, cug, conv, N, N, 0.0, D ** -0.5, False, False, None, row_order=order)
+        dq, dk, dv = (torch.full_like(x, float("nan")) for x in (qg, kg, vg))
+        be.bwd_block(dog, qg, kg, vg, o, lse, dq, dk, dv, cug, cug, conv, N, N, 0.0, D ** -0.5, False, None, row_order=order)
+        torch.cuda.synchronize()
+        ours = {"out": o, "dq": dq, "dk": dk, "dv": dv}
+        check_against_oracle(ours, ref, half, dtype, what="blocksparse row order D%d N%d" % (D, N))
+        assert o[80:96].abs().max() == 0 and dq[80:96].abs().max() == 0  # the row block without an active tile
+        res.append(ours)
+    for other in res[1:]:
+        for n in ("out", "dq", "dk", "dv"):
+            assert _maxerr(res[0][n], other[n]) <= 4 * HALF_ULP[dtype] * max(1.0, res[0][n].float().abs().max().item()), n
+    bad = torch.zeros(nrb - 1, dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="row_order"):
+        be.fwd_block(qg, kg, vg, cug, cug, conv, N, N, 0.0, D ** -0.5, False, False, None, row_order=bad)
+
+
 def test_blocksparse_full_layout_equals_dense(full_size_tiles):
     from flash_attn.flash_blocksparse_attn_interface import flash_blocksparse_attn_func
     from flash_attn.flash_attn_interface import flash_attn_unpadded_qkvpacked_func
