@@ -559,6 +559,32 @@ def main():
         print("%-28s %9.4f ms  %8.1f GB/s of %d (%.1f %% of HBM peak)  [B=%d S=%d H=%d d=%d fp16 packed qkv, in place]"
               % ("rotary q,k (fa_rotary)", ms, nbytes / ms / 1e6, HBM_PEAK_GBS, 100 * nbytes / ms / 1e6 / HBM_PEAK_GBS,
                  Br, Sr, Hr, Dr), file=sys.stderr)
+        # the same embedding around one attention step (fwd + bwd), as FlashMHA(use_rotary_emb="1d") runs it: q and k rotated
+        # by a pass before the forward and dq, dk by a pass after the backward, against the rotation inside the attention
+        # kernels (only k takes a pass)
+        packed = qkv_r.view(Br * Sr, 3, Hr, Dr)
+        do_r = torch.randn(Br * Sr, Hr, Dr, device="cuda", dtype=torch.float16)
+        cu_r = torch.arange(0, (Br + 1) * Sr, Sr, dtype=torch.int32, device="cuda")
+        dqkv_r, rot_r = torch.empty_like(packed), torch.empty(Br * Sr, 2, Hr, Dr, device="cuda", dtype=torch.float16)
+        scale_r = Dr ** -0.5
+
+        def step_separate():
+            be.rotary(qkv_r, qkv_r, cos_h, sin_h, n_rotated=2)
+            o, lse = be.fwd(packed[:, 0], packed[:, 1], packed[:, 2], cu_r, cu_r, Sr, Sr, 0.0, scale_r, False, False, False)
+            be.bwd(do_r, packed[:, 0], packed[:, 1], packed[:, 2], o, lse, dqkv_r[:, 0], dqkv_r[:, 1], dqkv_r[:, 2], cu_r, cu_r,
+                   Sr, Sr, 0.0, scale_r, False, False)
+            g5 = dqkv_r.view(Br, Sr, 3, Hr, Dr)
+            be.rotary(g5, torch.empty_like(g5), cos_h, sin_h, n_rotated=2, conjugate=True)
+
+        def step_in_kernel():
+            be.rotary(qkv_r[:, :, 1:2], rot_r.view(Br, Sr, 2, Hr, Dr)[:, :, 1:2], cos_h, sin_h, n_rotated=1)
+            o, lse = be.fwd(packed[:, 0], rot_r[:, 1], packed[:, 2], cu_r, cu_r, Sr, Sr, 0.0, scale_r, False, False, False,
+                            rotary=(cos_h, sin_h), q_rot=rot_r[:, 0])
+            be.bwd(do_r, rot_r[:, 0], rot_r[:, 1], packed[:, 2], o, lse, dqkv_r[:, 0], dqkv_r[:, 1], dqkv_r[:, 2], cu_r, cu_r,
+                   Sr, Sr, 0.0, scale_r, False, False, rotary=(cos_h, sin_h))
+        ms_sep, ms_in = graph_replay_ms(torch, step_separate), graph_replay_ms(torch, step_in_kernel)
+        print("%-28s %9.4f ms with separate passes, %.4f ms inside the kernels (%.1f %% less)  [same shape, fwd + bwd, no "
+              "dropout]" % ("rotary + attention step", ms_sep, ms_in, 100 * (1 - ms_in / ms_sep)), file=sys.stderr)
     print(json.dumps(res))
 
 

@@ -251,6 +251,21 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
     p.bias = a->attn_bias;
     p.bias_bs = a->bias_batch_stride; p.bias_hs = a->bias_head_stride; p.bias_rs = a->bias_row_stride;
   }
+  if (a->rotary_cos || a->rotary_sin) {
+    FA_REQUIRE(a->rotary_cos && a->rotary_sin && aligned16(a->rotary_cos) && aligned16(a->rotary_sin),
+               "rotary_cos and rotary_sin come together, 16-byte aligned");
+    FA_REQUIRE(a->rotary_table_rows >= a->max_seqlen_q, "the rotary tables must have a row for every query position");
+    if (sparse || a->alibi_slopes || a->attn_bias)
+      return fail(FA_ERR_UNSUPPORTED, "rotary_cos with a blockmask, alibi_slopes or attn_bias: rotate with fa_rotary first");
+    if (a->s_dmask) return fail(FA_ERR_UNSUPPORTED, "rotary_cos with s_dmask: rotate with fa_rotary first");
+    p.rot_cos = a->rotary_cos; p.rot_sin = a->rotary_sin; p.rot_rows = a->rotary_table_rows;
+    if (a->q_rot) {
+      FA_REQUIRE(aligned16(a->q_rot) && a->q_rot_row_stride % 8 == 0 && a->q_rot_head_stride % 8 == 0 &&
+                     a->q_rot_head_stride >= a->head_dim && a->q_rot_row_stride >= a->head_dim,
+                 "q_rot must be 16-byte aligned with strides that are multiples of 8 and at least head_dim");
+      p.q_rot = a->q_rot; p.qr_rs = a->q_rot_row_stride; p.qr_hs = a->q_rot_head_stride;
+    }
+  }
   if (a->keep_words && dropout && !sparse) {
     FA_REQUIRE(aligned16(a->keep_words), "keep_words must be 16-byte aligned");
     const size_t kw_need = fa_keep_words_bytes(a->batch, a->nheads, a->max_seqlen_q, a->max_seqlen_k);
@@ -296,7 +311,9 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
 // all key tiles of a (batch, head) fit one XCD at once with room to spare (they wait for each other).
 size_t fused_bwd_bytes(const fa_bwd_args* a) {
   if ((fa::launch_policy() & 0x30) != 0x20) return 0;
-  if (a->head_dim != 64 || a->blockmask || a->p_dropout > 0.f || a->alibi_slopes || a->attn_bias || a->is_causal) return 0;
+  if (a->head_dim != 64 || a->blockmask || a->p_dropout > 0.f || a->alibi_slopes || a->attn_bias || a->is_causal ||
+      a->rotary_cos)
+    return 0;
   if (a->batch <= 0 || a->nheads <= 0 || a->max_seqlen_q <= 0 || a->max_seqlen_k <= 0) return 0;
   if ((a->max_seqlen_k + fa::kBwdBN - 1) / fa::kBwdBN > 32) return 0;
   const size_t nqt = ((size_t)a->max_seqlen_q + fa::kFusedBM - 1) / fa::kFusedBM;
@@ -401,6 +418,16 @@ int bwd_impl(const fa_bwd_args* a, bool want_block, void* ev_main_start = nullpt
       return fail(FA_ERR_UNSUPPORTED, "dbias: a (batch, head) slice is limited to 2^31 elements");
     p.dbias = a->dbias;
     p.dbias_bs = a->dbias_batch_stride; p.dbias_hs = a->dbias_head_stride; p.dbias_rs = a->dbias_row_stride;
+  }
+  if (a->rotary_cos || a->rotary_sin) {
+    FA_REQUIRE(a->rotary_cos && a->rotary_sin && (reinterpret_cast<uintptr_t>(a->rotary_cos) & 3) == 0 &&
+                   (reinterpret_cast<uintptr_t>(a->rotary_sin) & 3) == 0,
+               "rotary_cos and rotary_sin come together, 4-byte aligned");
+    FA_REQUIRE(a->rotary_table_rows >= a->max_seqlen_q && a->rotary_table_rows >= a->max_seqlen_k,
+               "the rotary tables must have a row for every query and key position");
+    if (sparse || a->alibi_slopes || a->attn_bias)
+      return fail(FA_ERR_UNSUPPORTED, "rotary_cos with a blockmask, alibi_slopes or attn_bias: rotate with fa_rotary first");
+    p.rot_cos = a->rotary_cos; p.rot_sin = a->rotary_sin; p.rot_rows = a->rotary_table_rows;
   }
   if (a->keep_words && dropout && !sparse) {
     FA_REQUIRE(aligned16(a->keep_words), "keep_words must be 16-byte aligned");

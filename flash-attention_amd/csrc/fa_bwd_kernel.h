@@ -65,8 +65,11 @@ struct BwdCfg {
 // kDrop: 0 = no dropout; 1 = the keep decisions are drawn here (Philox); 2 = they are read from the keep words the
 // forward left (fa_common.h; dense only): the kernel then has the tile shape of the one without dropout.
 // kBias: as in fa_fwd_kernel; with a bias tensor the kernel also leaves d(loss)/d(bias) in p.dbias if that is not null
-template <typename T, int D, bool kCausal, int kDrop, bool kSparse, int kBias = 0>
+// kRot: the keys came in rotated (rotary position embedding) and dK goes out turned back (dense variants without score bias
+// only; a variant of its own because the plain kernels sit at their register limit)
+template <typename T, int D, bool kCausal, int kDrop, bool kSparse, int kBias = 0, bool kRot = false>
 __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasTensor) ? 3 : ((D == 128 && kBias == kBiasTensor) ? 1 : BwdCfg<T, D, kDrop == 1>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
+  static_assert(!kRot || (!kSparse && kBias == 0), "rotary: dense variants without score bias");
   constexpr bool kDropout = kDrop == 1, kStored = kDrop == 2;
   constexpr bool kAlibi = kBias == kBiasAlibi, kTensorBias = kBias == kBiasTensor;
   static_assert(!(kStored && kSparse), "keep words: dense only");
@@ -445,6 +448,27 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasT
     else mt++;
   }
 
+  // ---- rotary: k came in rotated; dk goes out turned back by the angles of this lane's key (linear, so it can precede the
+  // scaling), in fp32 before its one rounding
+  if constexpr (kRot) {
+    const int krow = n0 + wave * 32 + (int)(threadIdx.x & 31);
+    const int t = krow < p.rot_rows ? krow : p.rot_rows - 1;
+#pragma unroll
+    for (int db = 0; db < DV / 32; db++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        const int d0 = db * 32 + g4 * 8 + (int)(threadIdx.x >> 5 & 1) * 4;
+        if (d0 < D) {
+          f32x4 x;
+#pragma unroll
+          for (int i = 0; i < 4; i++) x[i] = acc_dk[db][g4 * 4 + i];
+          x = unrotate4<T>(x, p.rot_cos, p.rot_sin, t, D / 2, d0);
+#pragma unroll
+          for (int i = 0; i < 4; i++) acc_dk[db][g4 * 4 + i] = x[i];
+        }
+      }
+  }
+
   // ---- epilogue: scale, transpose dK^T / dV^T through LDS, coalesced stores
   __syncthreads();
   constexpr int ES = D + 8;
@@ -517,6 +541,7 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
   constexpr bool kAlibi = kBias == kBiasAlibi, kTensorBias = kBias == kBiasTensor;
   static_assert(kBias == 0 || !kSparse, "score bias: dense variants only");
   static_assert(!(kStored && kSparse), "keep words: dense only");
+  constexpr bool kRotCapable = !kSparse && kBias == 0;  // rotary (p.rot_cos): dense variants without score bias
   using Cfg = DqCfg<T, D, BN, KS>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
@@ -853,6 +878,8 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
             f32x4 x;
 #pragma unroll
             for (int i = 0; i < 4; i++) x[i] = acc[db][g4 * 4 + i] * f;
+            if (kRotCapable && p.rot_cos != nullptr)  // rotary: the turn back is linear, so every partial sum takes it
+              x = unrotate4<T>(x, p.rot_cos, p.rot_sin, qrow < p.rot_rows ? qrow : p.rot_rows - 1, D / 2, d0);
             *reinterpret_cast<f32x4*>(op + d0) = x;
           }
         }
@@ -871,6 +898,11 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
         f32x4 x;
 #pragma unroll
         for (int i = 0; i < 4; i++) x[i] = acc[db][g4 * 4 + i] * f;
+        // rotary: q came in rotated; dq goes out turned back (this lane's query row sits at table row `qrow`)
+        if (kRotCapable && p.rot_cos != nullptr) {
+          int t = qrow < Lq ? qrow : Lq - 1;
+          x = unrotate4<T>(x, p.rot_cos, p.rot_sin, t < p.rot_rows ? t : p.rot_rows - 1, D / 2, d0);
+        }
         *reinterpret_cast<typename E::vec4*>(Os + c * OS + d0) = cvt4<T>(x);
       }
     }

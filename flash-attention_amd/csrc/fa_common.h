@@ -125,6 +125,42 @@ FA_DEVICE float half_sum(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// Rotary position embedding of one 16-byte chunk: pairs (x[2e], x[2e+1]) turned by the angles whose cosines / sines are
+// c4[e] / s4[e] (rounded to the tensor dtype, as the reference's cached tables are: flash_attn/rotary.py:66-87), products
+// and sums in fp32, one rounding.  The one definition serves the stand-alone pass (fa_rotary.hip) and the attention
+// kernels, so both give the same bits.
+template <typename T>
+FA_DEVICE typename Elem<T>::vec8 rotate8(typename Elem<T>::vec8 x, typename Elem<T>::vec4 c4, typename Elem<T>::vec4 s4,
+                                         bool conjugate) {
+  typename Elem<T>::vec8 y;
+#pragma unroll
+  for (int e = 0; e < 4; e++) {
+    const float a = (float)x[2 * e], b = (float)x[2 * e + 1];
+    const float c = (float)c4[e], s = conjugate ? -(float)s4[e] : (float)s4[e];
+    y[2 * e] = (T)(a * c - b * s);
+    y[2 * e + 1] = (T)(b * c + a * s);
+  }
+  return y;
+}
+// The opposite rotation of four consecutive fp32 values (two pairs; d0 = index of the first inside the head dimension) of
+// the row at table position t: what turns a gradient with respect to rotated queries or keys into the gradient with respect
+// to the unrotated ones, before it is rounded.
+template <typename T>
+FA_DEVICE f32x4 unrotate4(f32x4 x, const void* cos_table, const void* sin_table, int t, int half_dim, int d0) {
+  typedef T t2 __attribute__((ext_vector_type(2)));
+  const int64_t off = (int64_t)t * half_dim + (d0 >> 1);
+  const t2 c2 = *reinterpret_cast<const t2*>(reinterpret_cast<const T*>(cos_table) + off);
+  const t2 s2 = *reinterpret_cast<const t2*>(reinterpret_cast<const T*>(sin_table) + off);
+  f32x4 y;
+#pragma unroll
+  for (int e = 0; e < 2; e++) {
+    const float c = (float)c2[e], s = (float)s2[e];
+    y[2 * e] = x[2 * e] * c + x[2 * e + 1] * s;
+    y[2 * e + 1] = x[2 * e + 1] * c - x[2 * e] * s;
+  }
+  return y;
+}
+
 // 16-byte global load/store helpers.
 FA_DEVICE u32x4 ld_global16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
 FA_DEVICE void st_global16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }

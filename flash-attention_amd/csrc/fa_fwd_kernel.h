@@ -223,6 +223,24 @@ __global__ void __launch_bounds__(256, (!kDropout && kBias == 0 && D <= 64) ? 4 
     stage(it, 0);
     if (kTensorBias) load_bias(it);
   }
+  // Rotary embedding of the queries (what the reference's FlashMHA does to q before attention, flash_attention.py:109-113,
+  // with elementwise ops): the fragments are turned where they sit, after the first tile has been asked for; the rotated
+  // rows are left in q_rot for the backward, whose kernels stream Q through LDS and cannot do the same
+  if (p.rot_cos != nullptr) {
+    int t = qrow < Lq ? qrow : Lq - 1;
+    t = t < p.rot_rows ? t : p.rot_rows - 1;
+    const T* const ct = reinterpret_cast<const T*>(p.rot_cos) + (int64_t)t * (D / 2) + hf * 4;
+    const T* const st = reinterpret_cast<const T*>(p.rot_sin) + (int64_t)t * (D / 2) + hf * 4;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ks++)
+      qreg[ks] = rotate8<T>(qreg[ks], *reinterpret_cast<const typename E::vec4*>(ct + ks * 8),
+                            *reinterpret_cast<const typename E::vec4*>(st + ks * 8), false);
+    if (p.q_rot != nullptr && kh == 0 && split == 0 && qrow < Lq) {
+      T* const qo = reinterpret_cast<T*>(p.q_rot) + (int64_t)(q_begin + qrow) * p.qr_rs + (int64_t)h * p.qr_hs + hf * 8;
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ks++) st_global16(qo + ks * 16, bitcast<u32x4>(qreg[ks]));
+    }
+  }
   while (it < ntiles) {
     const int n0 = it * BN;
     // Opaque redefinition of the accumulators at the top of every iteration: without it the register allocator

@@ -79,6 +79,15 @@ struct FwdParams {
   const float* alibi;  // null, or one slope per head: the score of (query i, key j) gets -slope * |i - j| added
   const void* bias;    // null, or a tensor of the element type added to the scaled scores: [b, h, query, key]
   int64_t bias_bs, bias_hs, bias_rs;  // its batch, head (0: shared) and row strides in elements; keys are contiguous
+  // Rotary position embedding of the queries inside the kernel (null: none): cos / sin tables [rot_rows, head_dim / 2] of
+  // the element type; the row at position i of its sequence is turned by table row i when its Q fragment is loaded (the
+  // keys come in rotated: their tiles go to LDS without passing through registers).  q_rot: null, or where the rotated
+  // queries are left for the backward ([total_q, H, d], strides in elements).
+  const void* rot_cos;
+  const void* rot_sin;
+  int rot_rows;
+  void* q_rot;
+  int64_t qr_rs, qr_hs;
   // Dropout keep words (fa_common.h), or null: the keep decisions of every score, left for the backward
   uint32_t* keep_words;
   int kw_q;   // query extent of the buffer (max_seqlen_q rounded up to 128)
@@ -146,6 +155,11 @@ struct BwdParams {
   int64_t bias_bs, bias_hs, bias_rs;
   void* dbias;         // null, or where the dK/dV kernel leaves d(loss)/d(bias) = dS / keep: [b, h, query, key], written for the
   int64_t dbias_bs, dbias_hs, dbias_rs;  // (query, key) tiles it visits (the caller clears the tensor)
+  // Rotary position embedding (as in FwdParams; null: none): q and k are the rotated tensors, and dq and dk are turned back
+  // by the opposite angles in the kernels' epilogues, before they are rounded
+  const void* rot_cos;
+  const void* rot_sin;
+  int rot_rows;
   // Dropout keep words (fa_common.h) as the forward left them, or null: read by both kernels in place of Philox
   const uint32_t* keep_words;
   int kw_q;   // query extent of the buffer (max_seqlen_q rounded up to 128)

@@ -62,15 +62,7 @@ __global__ void __launch_bounds__(512) rotary_kernel(const RotaryParams p, int w
   for (int i = 0; i < kRotaryRows; i++) {
     if (i < nrows) {
       vec8 y = x[i];
-      if (rot) {
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          const float a = (float)x[i][2 * e], b = (float)x[i][2 * e + 1];
-          const float c = (float)c4[i][e], s = p.conjugate ? -(float)s4[i][e] : (float)s4[i][e];
-          y[2 * e] = (T)(a * c - b * s);
-          y[2 * e + 1] = (T)(b * c + a * s);
-        }
-      }
+      if (rot) y = rotate8<T>(x[i], c4[i], s4[i], p.conjugate != 0);
       st_global16(dst + (int64_t)i * p.dst_row_stride, bitcast<u32x4>(y));
     }
   }

@@ -4,7 +4,7 @@ import torch
 import torch.nn as nn
 
 from .bert_padding import pad_input, unpad_input
-from .flash_attn_interface import flash_attn_unpadded_qkvpacked_func
+from .flash_attn_interface import flash_attn_unpadded_qkvpacked_func, flash_attn_unpadded_qkvpacked_rotary_func
 
 
 class FlashAttention(nn.Module):
@@ -22,18 +22,34 @@ class FlashAttention(nn.Module):
         self.dropout_p = attention_dropout
 
     def forward(self, qkv, attn_mask=None, key_padding_mask=None, causal=False, cu_seqlens=None, max_s=None,
-                need_weights=False, alibi_slopes=None, attn_bias=None):
+                need_weights=False, alibi_slopes=None, attn_bias=None, rotary=None):
         """qkv is (B, S, 3, H, D) when cu_seqlens is None, else already packed (nnz, 3, H, D) with cu_seqlens / max_s.
         key_padding_mask, if given, is an object whose `.bool_matrix` is a (B, S) bool tensor, True = keep.
         alibi_slopes (not in the reference): (H,) fp32 slopes of the in-kernel attention bias -slope * |i - j|.
         attn_bias (not in the reference): (1 or B, 1 or H, S, S) in qkv's dtype, added to the scaled scores; positions are
         counted inside each sequence (so with a key_padding_mask, among the tokens that are kept); differentiable.
+        rotary (not in the reference): (cos_half, sin_half) tables of RotaryEmbedding.half_tables: q and k are turned by
+        their position inside their sequence within the attention kernels (not with key_padding_mask, alibi_slopes or
+        attn_bias).
         Returns (output, None); output has the layout of the input's token dimensions."""
         assert not need_weights
         assert attn_mask is None
         assert qkv.dtype == torch.float16  # the reference's module restriction (:41); the functional API takes bf16 too
         assert qkv.is_cuda
         p = self.dropout_p if self.training else 0.0
+
+        if rotary is not None:
+            assert key_padding_mask is None and alibi_slopes is None and attn_bias is None
+            if cu_seqlens is not None:
+                assert max_s is not None
+                return flash_attn_unpadded_qkvpacked_rotary_func(qkv, *rotary, cu_seqlens, max_s, p,
+                                                                 softmax_scale=self.softmax_scale, causal=causal), None
+            batch, seqlen = qkv.shape[0], qkv.shape[1]
+            packed = qkv.reshape(batch * seqlen, *qkv.shape[2:])
+            cu = torch.arange(0, (batch + 1) * seqlen, step=seqlen, dtype=torch.int32, device=qkv.device)
+            out = flash_attn_unpadded_qkvpacked_rotary_func(packed, *rotary, cu, seqlen, p,
+                                                            softmax_scale=self.softmax_scale, causal=causal)
+            return out.reshape(batch, seqlen, *out.shape[1:]), None
 
         if cu_seqlens is not None:
             assert max_s is not None
@@ -85,6 +101,11 @@ class FlashMHA(nn.Module):
     def forward(self, x, x_ignored_, x_ignored_1_, attn_mask=None, key_padding_mask=None, need_weights=False):
         b, s = x.shape[0], x.shape[1]
         qkv = self.Wqkv(x).reshape(b, s, 3, self.num_heads, self.head_dim)
+        if (self.use_rotary_emb == "1d" and key_padding_mask is None and qkv.is_cuda and qkv.dtype == torch.float16):
+            # the rotation happens inside the attention kernels (q as it is loaded, dq and dk as they are stored)
+            context, attn_weights = self.inner_attn(qkv, need_weights=need_weights, causal=self.causal,
+                                                    rotary=self.rotary_emb.half_tables(qkv))
+            return self.out_proj(context.reshape(b, s, self.embed_dim)), attn_weights
         if self.use_rotary_emb and qkv.is_cuda and qkv.dtype in (torch.float16, torch.bfloat16) and (
                 self.use_rotary_emb == "1d" or self.head_dim % 16 == 0):
             qkv = self.rotary_emb.rotate_qkv_(qkv)  # q and k rotated in place by the HIP kernel (one pass; "2d": two)

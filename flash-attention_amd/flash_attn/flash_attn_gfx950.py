@@ -57,6 +57,9 @@ class FwdArgs(ctypes.Structure):
         ("attn_bias", ctypes.c_void_p), ("bias_batch_stride", ctypes.c_int64), ("bias_head_stride", ctypes.c_int64),
         ("bias_row_stride", ctypes.c_int64),
         ("row_order", ctypes.c_void_p),
+        ("rotary_cos", ctypes.c_void_p), ("rotary_sin", ctypes.c_void_p),
+        ("rotary_table_rows", ctypes.c_int32), ("reserved0", ctypes.c_int32),
+        ("q_rot", ctypes.c_void_p), ("q_rot_row_stride", ctypes.c_int64), ("q_rot_head_stride", ctypes.c_int64),
     ]
 
 
@@ -92,6 +95,8 @@ class BwdArgs(ctypes.Structure):
         ("dbias", ctypes.c_void_p), ("dbias_batch_stride", ctypes.c_int64), ("dbias_head_stride", ctypes.c_int64),
         ("dbias_row_stride", ctypes.c_int64),
         ("row_order", ctypes.c_void_p),
+        ("rotary_cos", ctypes.c_void_p), ("rotary_sin", ctypes.c_void_p),
+        ("rotary_table_rows", ctypes.c_int32), ("reserved0", ctypes.c_int32),
     ]
 
 
@@ -385,9 +390,21 @@ def blockmask_row_order(layout):
     return torch.tensor(order, dtype=torch.int32, device=layout.device)
 
 
+def _rotary_arg(a, rotary, q, rows_needed):
+    """(cos, sin) tables of the in-kernel rotary embedding into an argument struct."""
+    if rotary is None:
+        return
+    cos, sin = rotary
+    _check(cos.shape == sin.shape and cos.ndim == 2 and cos.shape[1] == q.shape[-1] // 2 and cos.dtype == q.dtype
+           and sin.dtype == q.dtype and cos.is_contiguous() and sin.is_contiguous() and cos.device == q.device
+           and sin.device == q.device, "rotary: cos / sin must be contiguous (rows, headdim / 2) tables in q's dtype")
+    _check(cos.shape[0] >= rows_needed, "rotary: the tables have fewer rows than the sequences have positions")
+    a.rotary_cos, a.rotary_sin, a.rotary_table_rows = cos.data_ptr(), sin.data_ptr(), cos.shape[0]
+
+
 def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
               zero_tensors, is_causal, return_softmax, gen, alibi_slopes=None, keep_words=None, attn_bias=None,
-              row_order=None):
+              row_order=None, rotary=None, q_rot=None):
     lib = load_library()
     code = _dtype_code(q)
     _check(q.dim() == 3, "q must be (total_q, nheads, head_size)")
@@ -443,6 +460,11 @@ def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_
         bias_t = _bias_arg(a, attn_bias, q, batch, nheads, max_seqlen_q, max_seqlen_k, sparse)  # noqa: F841 (kept alive)
         if sparse:
             _row_order_arg(a, row_order, sq_r, dev)
+        _rotary_arg(a, rotary, q, int(max_seqlen_q))
+        if q_rot is not None:
+            _check(rotary is not None, "q_rot without rotary tables")
+            _check_qkv("q_rot", q_rot, q.dtype, total_q, nheads, head_dim)
+            a.q_rot, a.q_rot_row_stride, a.q_rot_head_stride = q_rot.data_ptr(), q_rot.stride(0), q_rot.stride(1)
         rc = (lib.fa_fwd_block if sparse else lib.fa_fwd)(ctypes.byref(a))
         if rc != 0:
             _raise(rc, lib)
@@ -451,7 +473,7 @@ def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_
 
 def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q,
               max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen, main_kernel_events=None,
-              alibi_slopes=None, keep_words=None, attn_bias=None, dbias=None, row_order=None):
+              alibi_slopes=None, keep_words=None, attn_bias=None, dbias=None, row_order=None, rotary=None):
     lib = load_library()
     code = _dtype_code(q)
     _check(q.dim() == 3, "q must be (total_q, nheads, head_size)")
@@ -522,6 +544,7 @@ def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seql
             a.dbias_batch_stride, a.dbias_head_stride, a.dbias_row_stride = dbias.stride(0), dbias.stride(1), dbias.stride(2)
         if sparse:
             _row_order_arg(a, row_order, sq_r, dev)
+        _rotary_arg(a, rotary, q, max(int(max_seqlen_q), int(max_seqlen_k)))
         if main_kernel_events is not None and not sparse:  # (start, stop) torch.cuda.Event created with enable_timing=True
             for ev in main_kernel_events:
                 if not ev.cuda_event:  # torch creates the HIP event lazily, on first record
@@ -535,28 +558,34 @@ def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seql
 
 
 def fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale, zero_tensors,
-        is_causal, return_softmax, gen=None, alibi_slopes=None, keep_words=None, attn_bias=None):
+        is_causal, return_softmax, gen=None, alibi_slopes=None, keep_words=None, attn_bias=None, rotary=None, q_rot=None):
     """mha_fwd (fmha_api.cpp:173-299): returns [o, softmax_lse] or [o, softmax_lse, s].
     alibi_slopes (extension, not in the reference): nheads fp32 slopes; scores get -slope * |i - j| added.
     keep_words (extension): a buffer from new_keep_words() in which the dropout keep decisions are left for bwd.
     attn_bias (extension): (1 or batch, 1 or nheads, max_seqlen_q, max_seqlen_k) in q's dtype, added to the scaled scores
-    (positions counted inside the sequences; -inf masks); see prepare_attn_bias."""
+    (positions counted inside the sequences; -inf masks); see prepare_attn_bias.
+    rotary (extension): None, or (cos, sin) tables as for rotary(): q is turned by its position inside its sequence as the
+    kernel loads it (k must come in rotated; not with return_softmax); q_rot: a (total_q, nheads, head_size) tensor that
+    receives the rotated q, which bwd wants."""
     return _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, None, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
-                     zero_tensors, is_causal, return_softmax, gen, alibi_slopes, keep_words, attn_bias)
+                     zero_tensors, is_causal, return_softmax, gen, alibi_slopes, keep_words, attn_bias, rotary=rotary,
+                     q_rot=q_rot)
 
 
 def bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
         p_dropout, softmax_scale, zero_tensors, is_causal, gen=None, main_kernel_events=None, alibi_slopes=None,
-        keep_words=None, attn_bias=None, dbias=None):
+        keep_words=None, attn_bias=None, dbias=None, rotary=None):
     """mha_bwd (fmha_api.cpp:302-449): fills dq, dk, dv in place, returns [dq, dk, dv, softmax_d].
     attn_bias: the bias the forward was given; dbias: None, or a zero-filled (batch, nheads, max_seqlen_q, max_seqlen_k)
     tensor of q's dtype in which the gradient of the bias is left (per batch entry and head: sum for a shared bias).
     main_kernel_events: optional (start, stop) timing events recorded around the dq/dk/dv kernel alone.
     alibi_slopes: the slopes the forward was given (extension, not in the reference).
-    keep_words (extension): the buffer the forward of this call filled; the kernels then read the dropout decisions."""
+    keep_words (extension): the buffer the forward of this call filled; the kernels then read the dropout decisions.
+    rotary (extension): the tables the forward was given; q and k are then the rotated tensors and dq, dk come out as
+    gradients with respect to the unrotated ones."""
     return _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, None, max_seqlen_q,
                      max_seqlen_k, p_dropout, softmax_scale, zero_tensors, is_causal, gen, main_kernel_events, alibi_slopes,
-                     keep_words, attn_bias, dbias)
+                     keep_words, attn_bias, dbias, rotary=rotary)
 
 
 def fwd_block(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,

@@ -16,19 +16,40 @@ def _get_block_size(device, head_dim, is_dropout):
 
 
 def _flash_attn_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-                        softmax_scale, causal, return_softmax, alibi_slopes=None, keep_words=None, attn_bias=None):
+                        softmax_scale, causal, return_softmax, alibi_slopes=None, keep_words=None, attn_bias=None,
+                        rotary=None, q_rot=None):
     res = _backend.fwd(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale,
-                       False, causal, return_softmax, None, alibi_slopes, keep_words, attn_bias)
+                       False, causal, return_softmax, None, alibi_slopes, keep_words, attn_bias, rotary=rotary, q_rot=q_rot)
     return res[0], res[1], (res[2] if return_softmax else None)
 
 
 def _flash_attn_backward(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
                          max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, causal, alibi_slopes=None,
-                         keep_words=None, attn_bias=None, dbias=None):
+                         keep_words=None, attn_bias=None, dbias=None, rotary=None):
     _, _, _, softmax_d = _backend.bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
                                       max_seqlen_q, max_seqlen_k, dropout_p, softmax_scale, False, causal, None,
-                                      alibi_slopes=alibi_slopes, keep_words=keep_words, attn_bias=attn_bias, dbias=dbias)
+                                      alibi_slopes=alibi_slopes, keep_words=keep_words, attn_bias=attn_bias, dbias=dbias,
+                                      rotary=rotary)
     return dq, dk, dv, softmax_d
+
+
+def _rotated_keys(qkv, cu_seqlens, max_seqlen, cos_half, sin_half):
+    """(total, 2, nheads, headdim) buffer whose part 1 holds the rotated keys of a packed qkv (part 0 is left for the
+    rotated queries, which the attention kernel writes): one pass of the rotary kernel over the k third only."""
+    total, _, nheads, headdim = qkv.shape
+    batch = cu_seqlens.numel() - 1
+    rot = torch.empty((total, 2, nheads, headdim), dtype=qkv.dtype, device=qkv.device)
+    positions = None
+    if total != batch * max_seqlen:  # ragged: every row's position inside its sequence
+        lens = (cu_seqlens[1:] - cu_seqlens[:-1]).long()
+        positions = (torch.arange(total, device=qkv.device, dtype=torch.int32)
+                     - torch.repeat_interleave(cu_seqlens[:-1], lens, output_size=total))
+        src, dst = qkv[None, :, 1:2], rot[None, :, 1:2]
+    else:
+        src = qkv.reshape(batch, max_seqlen, 3, nheads, headdim)[:, :, 1:2]
+        dst = rot.view(batch, max_seqlen, 2, nheads, headdim)[:, :, 1:2]
+    _backend.rotary(src, dst, cos_half, sin_half, n_rotated=1, positions=positions)
+    return rot
 
 
 def _split(packing, tensors):
@@ -43,8 +64,14 @@ def _split(packing, tensors):
 
 
 def _forward(ctx, packing, tensors, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p,
-             softmax_scale, causal, return_softmax, alibi_slopes=None, attn_bias=None):
+             softmax_scale, causal, return_softmax, alibi_slopes=None, attn_bias=None, rotary=None):
     q, k, v = _split(packing, tensors)
+    # rotary embedding inside the kernels (packed qkv only): the keys are rotated into a side buffer by the rotary kernel,
+    # the queries by the attention kernel as it loads them, which also leaves them in the side buffer for the backward
+    rot = q_rot = None
+    if rotary is not None:
+        rot = _rotated_keys(tensors[0], cu_seqlens_q, int(max_seqlen_q), *rotary)
+        q_rot, k = rot[:, 0], rot[:, 1]
     # the dropout mask is a function of the generator state at this point; the backward rewinds to it
     rng_state = torch.cuda.get_rng_state(q.device) if dropout_p > 0 else None
     if softmax_scale is None:
@@ -62,8 +89,9 @@ def _forward(ctx, packing, tensors, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, ma
                                             int(max_seqlen_k))
     out, softmax_lse, S_dmask = _flash_attn_forward(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
                                                     dropout_p, softmax_scale, causal, return_softmax, alibi_slopes,
-                                                    keep_words, bias_t)
-    ctx.save_for_backward(*tensors, out, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state, bias_t)
+                                                    keep_words, bias_t, rotary, q_rot)
+    ctx.save_for_backward(*tensors, out, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state, bias_t, rot)
+    ctx.rotary = rotary  # constant tables, not differentiated
     ctx.bias_shape = tuple(attn_bias.shape) if attn_bias is not None else None
     ctx.bias_needs_grad = attn_bias is not None and attn_bias.requires_grad
     ctx.keep_words = keep_words
@@ -80,8 +108,10 @@ def _forward(ctx, packing, tensors, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, ma
 def _backward(ctx, dout):
     saved = ctx.saved_tensors
     tensors = saved[:ctx.n_in]
-    out, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state, bias_t = saved[ctx.n_in:]
+    out, softmax_lse, cu_seqlens_q, cu_seqlens_k, rng_state, bias_t, rot = saved[ctx.n_in:]
     q, k, v = _split(ctx.packing, tensors)
+    if rot is not None:  # the kernels take the rotated q and k and turn dq and dk back themselves
+        q, k = rot[:, 0], rot[:, 1]
     grads = tuple(torch.empty_like(t) for t in tensors)
     dq, dk, dv = _split(ctx.packing, grads)
     dev = q.device
@@ -94,7 +124,7 @@ def _backward(ctx, dout):
         torch.cuda.set_rng_state(rng_state, dev)
     _flash_attn_backward(dout.contiguous(), q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
                          ctx.max_seqlen_q, ctx.max_seqlen_k, ctx.dropout_p, ctx.softmax_scale, ctx.causal,
-                         ctx.alibi_slopes, ctx.keep_words, bias_t, dbias)
+                         ctx.alibi_slopes, ctx.keep_words, bias_t, dbias, ctx.rotary)
     if rng_state is not None:
         torch.cuda.set_rng_state(cur_rng_state, dev)
     ctx.dbias = None
@@ -127,6 +157,22 @@ class FlashAttnQKVPackedFunc(torch.autograd.Function):
         ctx.n_extra = 6 + len(bias)  # the reference's six non-tensor arguments (:72), plus the optional alibi_slopes, attn_bias
         return _forward(ctx, "qkv", (qkv,), cu_seqlens, cu_seqlens, max_seqlen, max_seqlen, dropout_p, softmax_scale,
                         causal, return_softmax, *bias)
+
+    @staticmethod
+    def backward(ctx, dout, *args):
+        return _extra_grads(ctx, _backward(ctx, dout))
+
+
+class FlashAttnRotaryQKVPackedFunc(torch.autograd.Function):
+    """apply(qkv, cos_half, sin_half, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal): self-attention on a
+    packed qkv whose q and k get the rotary embedding inside the kernels (no counterpart in the reference, whose FlashMHA
+    rotates them with elementwise ops first, flash_attention.py:109-113).  qkv itself is left as it is."""
+
+    @staticmethod
+    def forward(ctx, qkv, cos_half, sin_half, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal):
+        ctx.n_extra = 7
+        return _forward(ctx, "qkv", (qkv,), cu_seqlens, cu_seqlens, max_seqlen, max_seqlen, dropout_p, softmax_scale,
+                        causal, False, rotary=(cos_half, sin_half))
 
     @staticmethod
     def backward(ctx, dout, *args):
@@ -197,6 +243,19 @@ def flash_attn_unpadded_qkvpacked_func(qkv, cu_seqlens, max_seqlen, dropout_p, s
     """Self-attention on a packed (total, 3, nheads, headdim) tensor of variable-length sequences."""
     return FlashAttnQKVPackedFunc.apply(qkv, cu_seqlens, max_seqlen, dropout_p, softmax_scale, causal,
                                         return_attn_probs, alibi_slopes, attn_bias)
+
+
+def flash_attn_unpadded_qkvpacked_rotary_func(qkv, cos_half, sin_half, cu_seqlens, max_seqlen, dropout_p,
+                                              softmax_scale=None, causal=False):
+    """flash_attn_unpadded_qkvpacked_func on a qkv whose q and k are first turned by the rotary position embedding
+    (not in the reference's functional API; its FlashMHA does apply_rotary_pos_emb to q and k and then calls the function
+    above).  cos_half, sin_half: (>= max_seqlen, headdim / 2) tables in qkv's dtype, one entry per rotated pair
+    (RotaryEmbedding.half_tables); the token at position i of its sequence is turned by row i.  Same result as
+    apply_rotary_emb_qkv_ followed by flash_attn_unpadded_qkvpacked_func, bit for bit in the forward; the gradient is
+    rounded once instead of twice.  The rotation of q and of the gradients happens inside the attention kernels; only k
+    takes a pass of its own.  Differentiable with respect to qkv."""
+    return FlashAttnRotaryQKVPackedFunc.apply(qkv, cos_half, sin_half, cu_seqlens, max_seqlen, dropout_p, softmax_scale,
+                                              causal)
 
 
 def flash_attn_unpadded_kvpacked_func(q, kv, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,

@@ -79,11 +79,19 @@ class RotaryEmbedding(torch.nn.Module):
             self._sin_cached = torch.sin(angles).to(x.dtype).repeat_interleave(2, dim=-1)
         return self._cos_cached, self._sin_cached
 
+    def half_tables(self, qkv):
+        """(cos, sin) of shape (seqlen, headdim / 2) for a (batch, seqlen, 3, nheads, headdim) tensor: one entry per rotated
+        pair, the form the HIP kernels read.  Same values as forward()'s tables; kept until those change."""
+        cos, sin = self._update_cos_sin_tables(qkv[:, :, 0], seq_dimension=-3)
+        if getattr(self, "_half_of", None) is not cos:
+            self._half = (cos[:, ::2].contiguous(), sin[:, ::2].contiguous())
+            self._half_of = cos
+        return self._half
+
     def rotate_qkv_(self, qkv):
         """q and k of a packed (batch, seqlen, 3, nheads, headdim) GPU tensor rotated in place (one HIP kernel); returns
         qkv.  Same tables as forward()."""
-        cos, sin = self._update_cos_sin_tables(qkv[:, :, 0], seq_dimension=-3)
-        return apply_rotary_emb_qkv_(qkv, cos[:, ::2].contiguous(), sin[:, ::2].contiguous())
+        return apply_rotary_emb_qkv_(qkv, *self.half_tables(qkv))
 
     def forward(self, q: torch.Tensor, k: torch.Tensor, seq_dimension=-2) -> Tuple[torch.Tensor, torch.Tensor]:
         assert seq_dimension in [-2, -3]  # (bs, h, s, d) or (bs, s, h, d)

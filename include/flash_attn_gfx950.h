@@ -97,6 +97,21 @@ typedef struct fa_fwd_args {
    * must be distinct row blocks (a row block that is not listed is not computed: its rows of o / dq are left unwritten);
    * ignored with is_causal. */
   const int32_t* row_order;
+  /* Rotary position embedding inside the kernels (replaces the elementwise passes of the reference's FlashMHA,
+   * flash_attention.py:109-113 with rotary.py:90-99, which read and write q and k once more in each direction).  NULL, or
+   * the interleaved-pair cos / sin tables of fa_rotary ([rotary_table_rows, head_dim / 2] of `dtype`, contiguous, 16-byte
+   * aligned, rotary_table_rows >= max_seqlen_q): the query at position i of its sequence is turned by table row i as
+   * it is loaded, with fa_rotary's arithmetic, so o and softmax_lse are bit for bit those of fa_rotary followed by
+   * fa_fwd.  k is NOT turned here - key tiles never pass through registers - the caller gives the rotated keys (fa_rotary
+   * over the k part only: a third of the bytes of rotating q and k).  q_rot: NULL, or a [total_q, nheads, head_dim] tensor
+   * (strides below, 16-byte aligned like q) that receives the rotated queries, which fa_bwd wants.  Not with
+   * return-softmax (s_dmask), whose pass reads q itself; not with a blockmask, alibi_slopes or attn_bias. */
+  const void* rotary_cos;
+  const void* rotary_sin;
+  int32_t rotary_table_rows;
+  int32_t reserved0; /* 0 */
+  void* q_rot;
+  int64_t q_rot_row_stride, q_rot_head_stride;
 } fa_fwd_args;
 
 /* Arguments of the backward pass.  Mirrors mha_bwd (fmha_api.cpp:302-321) and, when `blockmask`
@@ -157,6 +172,14 @@ typedef struct fa_bwd_args {
   int64_t dbias_batch_stride, dbias_head_stride, dbias_row_stride;
   /* as in fa_fwd_args (the backward need not be given the order the forward had) */
   const int32_t* row_order;
+  /* Rotary position embedding inside the kernels.  NULL, or the tables the forward was given (rotary_table_rows >=
+   * max(max_seqlen_q, max_seqlen_k)): q and k are then the ROTATED tensors (fa_fwd_args.q_rot and the k the forward
+   * read), and dq and dk come out as gradients with respect to the unrotated ones - turned back by the opposite angles in
+   * fp32 before their one rounding - so no elementwise pass over them follows. */
+  const void* rotary_cos;
+  const void* rotary_sin;
+  int32_t rotary_table_rows;
+  int32_t reserved0; /* 0 */
 } fa_bwd_args;
 
 /* replaces flash_attn_cuda.fwd -> mha_fwd, csrc/flash_attn/fmha_api.cpp:173-299 */

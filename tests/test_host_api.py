@@ -190,7 +190,11 @@ def test_public_signatures_match_the_reference():
     from flash_attn import flash_attn_gfx950 as be
     assert list(inspect.signature(be.fwd).parameters) == [
         "q", "k", "v", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k", "p_dropout", "softmax_scale",
-        "zero_tensors", "is_causal", "return_softmax", "gen", "alibi_slopes", "keep_words", "attn_bias"]  # fmha_api.cpp:173-186 + extensions
+        "zero_tensors", "is_causal", "return_softmax", "gen", "alibi_slopes", "keep_words", "attn_bias", "rotary",
+        "q_rot"]  # fmha_api.cpp:173-186 + extensions
+    assert sig(fi.flash_attn_unpadded_qkvpacked_rotary_func) == [
+        ("qkv", "<req>"), ("cos_half", "<req>"), ("sin_half", "<req>"), ("cu_seqlens", "<req>"), ("max_seqlen", "<req>"),
+        ("dropout_p", "<req>"), ("softmax_scale", None), ("causal", False)]  # extension: rotary embedding inside the kernels
     assert list(inspect.signature(be.bwd_block).parameters) == [
         "dout", "q", "k", "v", "out", "softmax_lse", "dq", "dk", "dv", "cu_seqlens_q", "cu_seqlens_k", "blockmask",
         "max_seqlen_q", "max_seqlen_k", "p_dropout", "softmax_scale", "is_causal", "gen", "row_order"]  # fmha_api.cpp:575-594 + extension
@@ -350,6 +354,52 @@ def test_dbias_layout_is_validated_before_anything_is_launched(lib):
     assert lib.fa_bwd(ctypes.byref(a)) == -1 and b"2-byte alignment" in lib.fa_last_error()
     a.dbias, a.attn_bias = fake, None
     assert lib.fa_bwd(ctypes.byref(a)) == -1 and b"dbias without attn_bias" in lib.fa_last_error()
+
+
+def test_in_kernel_rotary_arguments_are_validated_before_anything_is_launched(lib):
+    """tables come in pairs, aligned, with a row for every position; not together with the probability dump"""
+    from flash_attn import flash_attn_gfx950 as be
+    fake = 0x10000  # never dereferenced: the checks below fail before any launch
+    f = be.FwdArgs()
+    f.struct_bytes = ctypes.sizeof(f)
+    f.dtype = be.FA_FP16
+    f.batch, f.nheads, f.head_dim = 2, 3, 64
+    f.total_q = f.total_k = 64
+    f.max_seqlen_q = f.max_seqlen_k = 32
+    f.p_dropout, f.softmax_scale = 0.0, 0.125
+    for name in ("q", "k", "v", "o", "softmax_lse", "cu_seqlens_q", "cu_seqlens_k"):
+        setattr(f, name, fake)
+    for t in ("q", "k", "v", "o"):
+        setattr(f, t + "_row_stride", 192)
+        setattr(f, t + "_head_stride", 64)
+    f.rotary_cos, f.rotary_table_rows = fake, 32
+    assert lib.fa_fwd(ctypes.byref(f)) == -1 and b"come together" in lib.fa_last_error()
+    f.rotary_sin = fake + 8
+    assert lib.fa_fwd(ctypes.byref(f)) == -1 and b"16-byte aligned" in lib.fa_last_error()
+    f.rotary_sin, f.rotary_table_rows = fake, 31
+    assert lib.fa_fwd(ctypes.byref(f)) == -1 and b"a row for every query position" in lib.fa_last_error()
+    f.rotary_table_rows, f.s_dmask = 32, fake
+    assert lib.fa_fwd(ctypes.byref(f)) == -4 and b"rotate with fa_rotary first" in lib.fa_last_error()
+    f.s_dmask, f.q_rot, f.q_rot_row_stride, f.q_rot_head_stride = None, fake, 100, 64
+    assert lib.fa_fwd(ctypes.byref(f)) == -1 and b"q_rot must be" in lib.fa_last_error()
+
+    a = be.BwdArgs()
+    a.struct_bytes = ctypes.sizeof(a)
+    a.dtype = be.FA_FP16
+    a.batch, a.nheads, a.head_dim = 2, 3, 64
+    a.total_q = a.total_k = 64
+    a.max_seqlen_q, a.max_seqlen_k = 32, 40
+    a.lse_seq_stride = 32
+    a.p_dropout, a.softmax_scale = 0.0, 0.125
+    for name in ("dout", "q", "k", "v", "out", "softmax_lse", "dq", "dk", "dv", "softmax_d", "cu_seqlens_q", "cu_seqlens_k"):
+        setattr(a, name, fake)
+    for t in ("do", "q", "k", "v", "o", "dq", "dk", "dv"):
+        setattr(a, t + "_row_stride", 192)
+        setattr(a, t + "_head_stride", 64)
+    a.rotary_sin, a.rotary_table_rows = fake, 40
+    assert lib.fa_bwd(ctypes.byref(a)) == -1 and b"come together" in lib.fa_last_error()
+    a.rotary_cos, a.rotary_table_rows = fake, 39
+    assert lib.fa_bwd(ctypes.byref(a)) == -1 and b"a row for every query and key position" in lib.fa_last_error()
 
 
 def test_launch_policy_values_and_one_kernel_backward_scratch(lib):

@@ -68,13 +68,13 @@ def test_d64_kernels_keep_their_waves_per_simd():
         k = _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", flags + "Li2EEEv")
         assert k["Occupancy"] >= 3 and k["VGPRs Spill"] == 0, ("dq, key split", flags, k)
     for flags, want, spill in ((bplain, 3, 2), (bcausal, 3, 2), (bdrawn, 2, 0), (bread, 2, 0)):
-        k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", flags)
+        k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", flags + "Lb0EEEv")  # (last flag: the variant that turns dK back, rotary)
         assert k["Occupancy"] >= want and k["VGPRs Spill"] <= spill, ("dkdv", flags, k)
     # the ALiBi variants (fourth flag set) keep the waves per SIMD of their plain counterparts in the backward
     for flags, bflags in (("Lb0ELb0ELb0ELi1E", "Lb0ELi0ELb0ELi1E"), ("Lb1ELb0ELb0ELi1E", "Lb1ELi0ELb0ELi1E")):
         assert _pick(fwd, "fa_fwd_kernelIDF16_Li64E", flags + "Li1ELb0EEEv")["Occupancy"] >= 3, flags  # (the bias costs the fourth)
         assert _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", bflags + full)["Occupancy"] >= 3, bflags
-        k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", bflags)
+        k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", bflags + "Lb0EEEv")
         assert k["Occupancy"] >= 3 and k["VGPRs Spill"] <= 4, (bflags, k)
 
 
@@ -94,7 +94,7 @@ def test_d64_bias_tensor_and_one_kernel_backward_variants():
         for drop, spill in (("Li0E", 0), ("Li2E", 4), ("Li1E", 12)):
             k = _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", causal + drop + "Lb0ELi2ELi1EEEv")
             assert k["Occupancy"] >= 2 and k["VGPRs Spill"] == 0, ("dq, bias tensor", causal, drop, k)
-            k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", causal + drop + "Lb0ELi2E")
+            k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", causal + drop + "Lb0ELi2ELb0EEEv")
             assert k["Occupancy"] >= 2 and k["VGPRs Spill"] <= spill, ("dkdv, bias tensor", causal, drop, k)
     fused = _resources("fa_bwd_fused.hip")
     for dt in ("IDF16_", "IDF16b"):
@@ -111,7 +111,7 @@ def test_d128_backward_keeps_two_waves_per_simd():
         # plain, causal, both with a block layout, and the two without that read the dropout decisions from keep words
         for flags in ("Lb0ELi0ELb0ELi0E", "Lb1ELi0ELb0ELi0E", "Lb0ELi0ELb1ELi0E", "Lb1ELi0ELb1ELi0E", "Lb0ELi2ELb0ELi0E",
                       "Lb1ELi2ELb0ELi0E"):
-            k = _pick(bwd, "fa_bwd_dkdv_kernel%sLi128E" % dt, flags)
+            k = _pick(bwd, "fa_bwd_dkdv_kernel%sLi128E" % dt, flags + "Lb0EEEv")
             assert k["Occupancy"] >= 2 and k["VGPRs Spill"] == 0 and k["LDS Size"] <= 80 * 1024, (dt, flags, k)
             k = _pick(bwd, "fa_bwd_dq_kernel%sLi128E" % dt, flags + "Li1EEEv")
             assert k["Occupancy"] >= 2 and k["VGPRs Spill"] <= (1 if "Lb1ELi0E" in flags[8:] else 0), ("dq", dt, flags, k)

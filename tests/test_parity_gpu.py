@@ -1594,6 +1594,160 @@ def test_rotary_kernel_matches_oracle(dtype, D):
     assert torch.equal(x.grad[:, :, 2].cpu(), go[:, :, 2])
 
 
+# ------------------------------------------------------------------------------------------------
+# rotary embedding inside the attention kernels (fa_fwd_args.rotary_cos / fa_bwd_args.rotary_cos): the forward must give
+# the bits of fa_rotary followed by fa_fwd; the gradients, rounded once instead of twice, must be at least as close to an
+# fp32 PyTorch evaluation of rotation + attention as those of the separate passes are
+# ------------------------------------------------------------------------------------------------
+def _rotary_attention_fp32(qkv, cos_h, sin_h, lens, scale, causal, dout):
+    """d(out . dout)/d(qkv) of attention over rotated q, k, in fp32 PyTorch (tables as rounded to the tensors' dtype)"""
+    x = qkv.float().detach().requires_grad_(True)
+    outs, start = [], 0
+    for L in lens:
+        c = cos_h[:L].float()[:, None, :].repeat_interleave(2, -1)
+        s_ = sin_h[:L].float()[:, None, :].repeat_interleave(2, -1)
+
+        def rot(t):
+            pairs = t.reshape(*t.shape[:-1], -1, 2)
+            half_turn = torch.stack((-pairs[..., 1], pairs[..., 0]), -1).reshape(t.shape)
+            return t * c + half_turn * s_
+        q, k, v = rot(x[start:start + L, 0]), rot(x[start:start + L, 1]), x[start:start + L, 2]
+        sc = torch.einsum("ihd,jhd->hij", q, k) * scale
+        if causal:
+            sc = sc.masked_fill(torch.ones(L, L, dtype=torch.bool, device=x.device).triu(1), float("-inf"))
+        outs.append(torch.einsum("hij,jhd->ihd", torch.softmax(sc, -1), v))
+        start += L
+    out = torch.cat(outs)
+    out.backward(dout.float())
+    return out.detach(), x.grad
+
+
+@pytest.mark.parametrize("D,dtype,causal,lens", [
+    (64, torch.float16, False, [256, 256]),
+    (64, torch.float16, True, [200, 37, 129]),
+    (128, torch.bfloat16, False, [150, 300]),
+    (32, torch.bfloat16, True, [128, 128, 128]),
+    (16, torch.float16, False, [65, 500]),
+    (64, torch.bfloat16, False, [1024]),
+])
+def test_in_kernel_rotary_equals_the_separate_passes(D, dtype, causal, lens, tile_shape):
+    from flash_attn import flash_attn_gfx950 as be
+    from flash_attn import flash_attn_interface as fi
+    from flash_attn.rotary import RotaryEmbedding
+    torch.manual_seed(D + len(lens))
+    H, total, max_s = 3, sum(lens), max(lens)
+    cu = _cu(lens)
+    qkv = torch.randn(total, 3, H, D, device="cuda").to(dtype)
+    dout = torch.randn(total, H, D, device="cuda").to(dtype)
+    emb = RotaryEmbedding(D)
+    cos_h, sin_h = emb.half_tables(torch.empty(1, max_s + 3, 3, H, D, device="cuda", dtype=dtype))   # (max_s + 3, D / 2)
+    scale = D ** -0.5
+    positions = torch.cat([torch.arange(L, dtype=torch.int32) for L in lens]).cuda()
+
+    # separate passes: rotate q and k, attention, rotate the gradients back
+    a = qkv.clone()
+    be.rotary(a[None], a[None], cos_h, sin_h, n_rotated=2, positions=positions)
+    a.requires_grad_(True)
+    out_a = fi.flash_attn_unpadded_qkvpacked_func(a, cu, max_s, 0.0, causal=causal)
+    out_a.backward(dout)
+    g = a.grad.contiguous()
+    grad_a = be.rotary(g[None], torch.empty_like(g)[None], cos_h, sin_h, n_rotated=2, conjugate=True, positions=positions)[0]
+
+    b = qkv.clone().requires_grad_(True)
+    out_b = fi.flash_attn_unpadded_qkvpacked_rotary_func(b, cos_h, sin_h, cu, max_s, 0.0, causal=causal)
+    out_b.backward(dout)
+    assert torch.equal(b.detach(), qkv)                               # the caller's tensor is left as it is
+    assert torch.equal(out_b, out_a)                                  # same bits
+    assert torch.equal(b.grad[:, 2], grad_a[:, 2])                    # dv: same kernel on the same bits
+    out_ref, grad_ref = _rotary_attention_fp32(qkv, cos_h, sin_h, lens, scale, causal, dout)
+    # both paths round the same fp32 sums: the separate passes twice (rotating in between), the kernels once; the largest
+    # errors may sit on different elements, so one path's may exceed the other's by the three roundings (half a unit in the
+    # last place of the largest value each), and must not by more
+    ulp = 2.0 ** (-10 if dtype == torch.float16 else -7)
+    for part, name in ((0, "dq"), (1, "dk")):
+        top = float(grad_ref[:, part].abs().max())
+        err_a = _maxerr(grad_a[:, part], grad_ref[:, part])
+        err_b = _maxerr(b.grad[:, part], grad_ref[:, part])
+        assert err_b <= err_a + 2 * ulp * top, (name, err_b, err_a)
+        assert err_a < 0.05 * top, (name, err_a)   # the yardstick itself is sound
+        # and element by element they differ by those roundings only
+        assert _maxerr(b.grad[:, part], grad_a[:, part]) <= 2 * ulp * max(top, float(grad_a[:, part].abs().max()))
+
+
+def test_in_kernel_rotary_with_dropout_short_queries_and_the_module():
+    """dropout (the keep words ride along), a decode-like shape whose keys are split over workgroups, and FlashMHA, whose
+    "1d" rotary path goes through the kernels when no padding mask is given and through the separate pass otherwise"""
+    from flash_attn import flash_attn_gfx950 as be
+    from flash_attn import flash_attn_interface as fi
+    from flash_attn.flash_attention import FlashMHA
+    from flash_attn.rotary import RotaryEmbedding
+    D, H, dtype = 64, 4, torch.float16
+    for lens, p in (([300, 212], 0.17), ([2048] * 2, 0.0)):
+        torch.manual_seed(5)
+        total, max_s = sum(lens), max(lens)
+        cu = _cu(lens)
+        qkv = torch.randn(total, 3, H, D, device="cuda").to(dtype)
+        dout = torch.randn(total, H, D, device="cuda").to(dtype)
+        cos_h, sin_h = RotaryEmbedding(D).half_tables(torch.empty(1, max_s, 3, H, D, device="cuda", dtype=dtype))
+        positions = torch.cat([torch.arange(L, dtype=torch.int32) for L in lens]).cuda()
+        a = qkv.clone()
+        be.rotary(a[None], a[None], cos_h, sin_h, n_rotated=2, positions=positions)
+        a.requires_grad_(True)
+        torch.manual_seed(11)
+        out_a = fi.flash_attn_unpadded_qkvpacked_func(a, cu, max_s, p)
+        out_a.backward(dout)
+        g = a.grad.contiguous()
+        grad_a = be.rotary(g[None], torch.empty_like(g)[None], cos_h, sin_h, n_rotated=2, conjugate=True, positions=positions)[0]
+        b = qkv.clone().requires_grad_(True)
+        torch.manual_seed(11)
+        out_b = fi.flash_attn_unpadded_qkvpacked_rotary_func(b, cos_h, sin_h, cu, max_s, p)
+        out_b.backward(dout)
+        assert torch.equal(out_b, out_a) and torch.equal(b.grad[:, 2], grad_a[:, 2])
+        for part in range(2):  # two roundings against one: a few units in the last place of the larger of a pair
+            assert _maxerr(b.grad[:, part], grad_a[:, part]) <= 2.0 ** -8 * float(grad_a[:, part].abs().max())
+
+    # few queries, many keys: the forward and the dQ kernel split the keys (their partial sums take the rotation too)
+    torch.manual_seed(3)
+    Lq, Lk, Hs = 16, 8192, 2
+    q = torch.randn(Lq, Hs, D, device="cuda").to(dtype)
+    k = torch.randn(Lk, Hs, D, device="cuda").to(dtype)
+    v = torch.randn(Lk, Hs, D, device="cuda").to(dtype)
+    do = torch.randn(Lq, Hs, D, device="cuda").to(dtype)
+    cos_h, sin_h = RotaryEmbedding(D).half_tables(torch.empty(1, Lk, 3, Hs, D, device="cuda", dtype=dtype))
+    cu_q, cu_k = _cu([Lq]), _cu([Lk])
+    q_r = be.rotary(q[None, :, None], torch.empty_like(q)[None, :, None], cos_h, sin_h, n_rotated=1)[0, :, 0]
+    k_r = be.rotary(k[None, :, None], torch.empty_like(k)[None, :, None], cos_h, sin_h, n_rotated=1)[0, :, 0]
+    o_a, lse_a = be.fwd(q_r, k_r, v, cu_q, cu_k, Lq, Lk, 0.0, D ** -0.5, False, False, False)
+    q_rot = torch.empty_like(q)
+    o_b, lse_b = be.fwd(q, k_r, v, cu_q, cu_k, Lq, Lk, 0.0, D ** -0.5, False, False, False, rotary=(cos_h, sin_h), q_rot=q_rot)
+    assert torch.equal(o_a, o_b) and torch.equal(lse_a, lse_b) and torch.equal(q_rot, q_r)
+    ga = [torch.empty_like(t) for t in (q, k, v)]
+    gb = [torch.empty_like(t) for t in (q, k, v)]
+    be.bwd(do, q_r, k_r, v, o_a, lse_a, *ga, cu_q, cu_k, Lq, Lk, 0.0, D ** -0.5, False, False)
+    be.bwd(do, q_rot, k_r, v, o_b, lse_b, *gb, cu_q, cu_k, Lq, Lk, 0.0, D ** -0.5, False, False, rotary=(cos_h, sin_h))
+    dq_a = be.rotary(ga[0][None, :, None], torch.empty_like(q)[None, :, None], cos_h, sin_h, n_rotated=1, conjugate=True)[0, :, 0]
+    dk_a = be.rotary(ga[1][None, :, None], torch.empty_like(k)[None, :, None], cos_h, sin_h, n_rotated=1, conjugate=True)[0, :, 0]
+    assert torch.equal(ga[2], gb[2])
+    assert _maxerr(gb[0], dq_a) <= 2.0 ** -8 * float(dq_a.abs().max())
+    assert _maxerr(gb[1], dk_a) <= 2.0 ** -8 * float(dk_a.abs().max())
+
+    torch.manual_seed(0)
+    E, Hm, B, S = 256, 4, 2, 100
+    mha = FlashMHA(E, Hm, use_rotary_emb="1d", causal=True, device="cuda", dtype=torch.float16).eval()
+    x = torch.randn(B, S, E, device="cuda", dtype=torch.float16)
+
+    class AllKept:
+        bool_matrix = torch.ones(B, S, dtype=torch.bool, device="cuda")
+    y_fused, _ = mha(x, None, None)
+    y_fused.float().square().sum().backward()
+    g_fused = mha.Wqkv.weight.grad.clone()
+    mha.zero_grad()
+    y_sep, _ = mha(x, None, None, key_padding_mask=AllKept)
+    y_sep.float().square().sum().backward()
+    assert torch.equal(y_fused, y_sep)
+    assert _maxerr(g_fused, mha.Wqkv.weight.grad) <= 2.0 ** -7 * float(g_fused.abs().max())
+
+
 @pytest.mark.parametrize("dtype,D", [(torch.float16, 64), (torch.bfloat16, 32), (torch.float16, 16)])
 def test_rotary_2d_kernel_path_matches_oracle(dtype, D):
     """RotaryEmbedding2D.rotate_qkv_ (flash_attn/rotary.py:103-135 done by two passes of fa_rotary over the half-channel
