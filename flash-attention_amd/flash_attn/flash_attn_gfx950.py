@@ -31,6 +31,8 @@ _c_i32p = ctypes.c_void_p
 # case every kernel draws its own decisions, as the reference's do, and no memory beyond O(seqlen) is held between forward
 # and backward.
 KEEP_WORDS_MAX_BYTES = 1 << 30
+# ... and at most this multiple of the bytes of q, k and v (None: no such limit)
+KEEP_WORDS_MAX_INPUT_RATIO = 1.0
 
 
 class FwdArgs(ctypes.Structure):
@@ -316,13 +318,13 @@ def _bias_arg(a, attn_bias, q, batch, nheads, max_seqlen_q, max_seqlen_k, sparse
 
 def new_keep_words(q, cu_seqlens_q, max_seqlen_q, max_seqlen_k, p_dropout, total_k=None):
     """Buffer for the dropout keep words of one forward call (argument keep_words of fwd and bwd), or None if there is no
-    dropout or the buffer would exceed KEEP_WORDS_MAX_BYTES or the bytes of q, k and v (total_k: rows of k and v; default:
-    those of q)."""
+    dropout or the buffer would exceed KEEP_WORDS_MAX_BYTES or KEEP_WORDS_MAX_INPUT_RATIO times the bytes of q, k and v
+    (total_k: rows of k and v; default: those of q)."""
     if not p_dropout > 0:
         return None
     n = load_library().fa_keep_words_bytes(cu_seqlens_q.numel() - 1, q.shape[1], int(max_seqlen_q), int(max_seqlen_k))
     inputs = (q.shape[0] + 2 * (q.shape[0] if total_k is None else int(total_k))) * q.shape[1] * q.shape[2] * q.element_size()
-    if n == 0 or n > KEEP_WORDS_MAX_BYTES or n > inputs:
+    if n == 0 or n > KEEP_WORDS_MAX_BYTES or (KEEP_WORDS_MAX_INPUT_RATIO is not None and n > KEEP_WORDS_MAX_INPUT_RATIO * inputs):
         return None
     return torch.empty((n,), dtype=torch.uint8, device=q.device)
 

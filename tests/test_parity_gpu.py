@@ -63,10 +63,10 @@ def dropout_path(request):
     """Runs a dropout test both ways: the forward leaves its keep decisions for the backward to read (the default when
     the buffer is small enough), or every kernel draws them again (flash_attn_gfx950.KEEP_WORDS_MAX_BYTES = 0)."""
     from flash_attn import flash_attn_gfx950 as be
-    old = be.KEEP_WORDS_MAX_BYTES
-    be.KEEP_WORDS_MAX_BYTES = request.param
+    old = be.KEEP_WORDS_MAX_BYTES, be.KEEP_WORDS_MAX_INPUT_RATIO
+    be.KEEP_WORDS_MAX_BYTES, be.KEEP_WORDS_MAX_INPUT_RATIO = request.param, None  # (no cap relative to the inputs' size either)
     yield request.param
-    be.KEEP_WORDS_MAX_BYTES = old
+    be.KEEP_WORDS_MAX_BYTES, be.KEEP_WORDS_MAX_INPUT_RATIO = old
 
 
 def _cu(lens, device="cuda"):
@@ -492,12 +492,14 @@ def test_dropout_backward_reuses_the_forward_mask_without_probs(dropout_path):
     (64, torch.float16, False, [64, 100], [2048, 1500], False),   # short query side: the key-split dQ
     (64, torch.float16, True, [300, 129], None, True),
 ])
-def test_keep_words_hold_the_defined_mask_and_give_the_same_results(D, dtype, causal, lens_q, lens_k, alibi, tile_shape):
+def test_keep_words_hold_the_defined_mask_and_give_the_same_results(D, dtype, causal, lens_q, lens_k, alibi, tile_shape,
+                                                                   monkeypatch):
     """The forward's keep words (one bit per score) equal the oracle's mask bit for bit in their documented layout, the
     forward's outputs do not depend on whether it leaves them, and the backward that reads them gives the gradients of the
     backward that draws the decisions again: bit for bit (at head dim 128 dq within one rounding: there the two dQ variants
     subtract Dk from dP at different points)."""
     from flash_attn import flash_attn_gfx950 as be
+    monkeypatch.setattr(be, "KEEP_WORDS_MAX_INPUT_RATIO", None)  # small head dims: the words outweigh the inputs early
     lens_k = lens_k or lens_q
     p, H = 0.17, 3
     q, k, v, do = (x.cuda() for x in _inputs(lens_q, lens_k, H, D, dtype, 77))
@@ -569,6 +571,12 @@ def test_keep_words_argument_checks():
         be.KEEP_WORDS_MAX_BYTES = need
         assert be.new_keep_words(q, cu, 100, 100, p).numel() == need
         assert be.new_keep_words(q, cu, 100, 100, 0.0) is None
+        # ... and not when it would outweigh q, k and v (here 8192 bytes against 3 * 160 * 2 * 64 * 2)
+        ratio = be.KEEP_WORDS_MAX_INPUT_RATIO
+        be.KEEP_WORDS_MAX_INPUT_RATIO = 8191.0 / (3 * 160 * 2 * 64 * 2)
+        assert be.new_keep_words(q, cu, 100, 100, p) is None
+        be.KEEP_WORDS_MAX_INPUT_RATIO = ratio
+        assert ratio == 1.0 and be.new_keep_words(q, cu, 100, 100, p) is not None
     finally:
         be.KEEP_WORDS_MAX_BYTES = old
     torch.cuda.synchronize()
