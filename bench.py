@@ -417,6 +417,8 @@ def main():
     ap.add_argument("--backward", choices=("auto", "two-kernel", "one-kernel"), default="auto",
                     help="backward plan (fa_set_launch_policy 0x10 / 0x20): the dQ + dK/dV kernel pair, or the one-kernel "
                          "backward where it exists (head dim 64, dense, no mask, dropout or bias)")
+    ap.add_argument("--d128-wave-pairs", action="store_true",
+                    help="launch policy 0x40: the head-dim-128 dK/dV kernel as wave pairs (64 keys per workgroup)")
     ap.add_argument("--tile-sweep", action="store_true",
                     help="time full-size against half-size tiles on launches of growing size (markdown table on stderr, no JSON line)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -430,7 +432,7 @@ def main():
     be.load_library()  # fails loudly if the HIP library is not built
     if a.redraw_dropout:
         be.KEEP_WORDS_MAX_BYTES = 0
-    be.set_launch_policy({"auto": 0, "two-kernel": 0x10, "one-kernel": 0x20}[a.backward])
+    be.set_launch_policy({"auto": 0, "two-kernel": 0x10, "one-kernel": 0x20}[a.backward] | (0x40 if a.d128_wave_pairs else 0))
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
 

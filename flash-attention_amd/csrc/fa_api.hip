@@ -622,9 +622,9 @@ int fa_rotary(const fa_rotary_args* a) {
 }
 
 int fa_set_launch_policy(int policy) {
-  FA_REQUIRE((policy & ~0x33) == 0 && (policy & 3) != 3 && (policy & 0x30) != 0x30,
+  FA_REQUIRE((policy & ~0x73) == 0 && (policy & 3) != 3 && (policy & 0x30) != 0x30,
              "launch policy: tile shape 0 (automatic), 1 (full-size) or 2 (half-size), plus 0x10 (two-kernel backward) or 0x20 "
-             "(one-kernel backward where it exists)");
+             "(one-kernel backward where it exists), plus 0x40 (head dim 128: dK/dV kernel of wave pairs where it exists)");
   g_launch_policy.store(policy, std::memory_order_relaxed);
   return FA_OK;
 }

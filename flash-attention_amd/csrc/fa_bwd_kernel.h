@@ -509,6 +509,247 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasT
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// dK, dV at head dim 128 without dropout, mask layout or score bias: wave pairs
+// ---------------------------------------------------------------------------------------------------------------
+// At d = 128 one wave cannot hold K, V and both accumulators of 32 keys next to the scores at more than two waves per SIMD
+// (fa_bwd_dkdv_kernel keeps its V tile in LDS for that reason and reads every V fragment from there).  Here two waves share
+// 32 keys: the first holds the K fragments, forms S = Q K^T and P and owns dV^T += dO^T P; the second holds the V
+// fragments, forms dP - D = dO V^T - D, takes P from the first through LDS (rounded to the element type, as dV's MFMA
+// takes it; the accumulator layout on both sides: a straight copy), forms dS' = P o (dP - D) and owns dK^T += Q^T dS'.
+// Each wave then needs one operand's fragments and one accumulator: three waves per SIMD, and no V fragment is read from
+// LDS.  The second wave runs one 32-row slab behind the first, so that it never waits for its partner inside a step: in
+// step i it finishes slab i - 1 (P from LDS, Q^T of slab i - 1: the Q tile has three buffers, dO two) and then starts
+// slab i.  A workgroup is two pairs (64 keys); a step is one 32-row slab of Q and dO and has one barrier.
+struct PairCfg {
+  static constexpr int D = 128, BM = 32, BN = 64, CH = D / 8;
+  typedef TilePairStager<D, BM, kSwzDual, kSwzDual> Stager;
+  static constexpr int kTile = Stager::kTileBytes;        // one 32 x 128 tile
+  static constexpr int kOffQ = 0;                         // three Q tiles
+  static constexpr int kOffdO = 3 * kTile;                // two dO tiles
+  static constexpr int kOffStat = 5 * kTile;
+  static constexpr int kStatBytes = 2 * BM * 4;           // lse[BM], -Dk[BM]
+  static constexpr int kOffP = kOffStat + 2 * kStatBytes;
+  static constexpr int kPBytes = 2 * 64 * 16;             // one pair's P of one slab: 2 x 64 lanes x 8 elements
+  static constexpr int kTileBytes = kOffP + 4 * kPBytes;  // two pairs, two slabs in flight
+  static constexpr int ES = D + 8;
+  static constexpr int kEpiBytes = 4 * 32 * ES * 2;
+  static constexpr int kLdsBytes = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
+};
+
+template <typename T, bool kCausal, bool kRot>
+__global__ void __launch_bounds__(256, 3) fa_bwd_dkdv_pair_kernel(const BwdParams p) {
+  using Cfg = PairCfg;
+  using E = Elem<T>;
+  using vec8 = typename E::vec8;
+  using vec4 = typename E::vec4;
+  constexpr int D = Cfg::D, BM = Cfg::BM, BN = Cfg::BN, CH = Cfg::CH;
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes];
+
+  int bh, kt;
+  if (!map_tile<kCausal>(blockIdx.x, p.nk_tiles, p.B * p.H, &bh, &kt, p.tile_group)) return;
+  const int b = bh / p.H, h = bh % p.H;
+  int q_begin = 0, Lq = 0, k_begin, Lk;
+  if (!seq_extent(p.cu_k, b, p.total_k, p.max_sk, &k_begin, &Lk)) return;
+  if (!seq_extent(p.cu_q, b, p.total_q, p.max_sq, &q_begin, &Lq)) Lq = 0;  // no queries: dK = dV = 0
+  const int n0 = kt * BN;
+  if (n0 >= Lk) return;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int pr = wave >> 1;        // the pair, i.e. which 32 of the workgroup's 64 keys
+  const bool second = wave & 1;    // false: S, P, dV;  true: dP, dS', dK
+  const int c = lane & 31, hf = lane >> 5;
+  const int key = n0 + pr * 32 + c;  // this lane's key (sequence-local)
+
+  // ---- this wave's B operand: the K (first wave) or V (second wave) fragments of the pair's 32 keys; keys past the end
+  // are zero.  Issued here, looked at after the first tile has been asked for.
+  vec8 breg[D / 16];
+  u32x4 braw[D / 16];
+  {
+    const int kr = key < Lk ? key : Lk - 1;
+    const T* bp = second ? reinterpret_cast<const T*>(p.v) + (int64_t)(k_begin + kr) * p.v_rs + (int64_t)h * p.v_hs
+                         : reinterpret_cast<const T*>(p.k) + (int64_t)(k_begin + kr) * p.k_rs + (int64_t)h * p.k_hs;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ks++) braw[ks] = ld_global16(bp + hf * 8 + ks * 16);
+  }
+  const int mt_begin = kCausal ? n0 / BM : 0;  // query rows above the tile's first key see none of its keys
+  const int mt_end = (Lq + BM - 1) / BM;
+  const int n_slabs = mt_end > mt_begin ? mt_end - mt_begin : 0;
+  const float* lsebase = p.lse + ((int64_t)b * p.H + h) * p.lse_stride;
+  const float* dsbase = p.dsoftmax + ((int64_t)b * p.H + h) * p.sq_r;
+
+  typename Cfg::Stager stager;
+  stager.init(wave, lane, reinterpret_cast<const T*>(p.q) + (int64_t)q_begin * p.q_rs + (int64_t)h * p.q_hs, p.q_rs,
+              reinterpret_cast<const T*>(p.dout) + (int64_t)q_begin * p.do_rs + (int64_t)h * p.do_hs, p.do_rs);
+  float statpre = 0.f;  // a slab's lse (threads 0 .. BM-1) and Dk (BM .. 2 BM-1), converted when the slab is consumed
+  // q3 / d2: which of the three Q and of the two dO buffers the slab goes to (the stager adds one tile's size for the waves
+  // that fetch the second tensor)
+  auto stage = [&](int m0, int q3, int d2) {
+    if (tid < BM) {
+      statpre = INFINITY;  // rows past the end are switched off (P = 0)
+      if (m0 + tid < Lq) statpre = lsebase[m0 + tid];
+    } else if (tid < 2 * BM) {
+      statpre = 0.f;
+      if (m0 + tid - BM < Lq) statpre = dsbase[m0 + tid - BM];
+    }
+    stager.issue(lds_raw + (stager.second ? Cfg::kOffdO + (d2 - 1) * Cfg::kTile : Cfg::kOffQ + q3 * Cfg::kTile), m0, Lq);
+  };
+  auto stat_value = [&]() -> float {
+    if (tid < BM) return (statpre == -INFINITY) ? INFINITY : statpre * kLog2e;
+    return -statpre;
+  };
+
+  f32x16 acc[D / 32];
+#pragma unroll
+  for (int i = 0; i < D / 32; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
+  const float cs = p.scale_log2;
+  int foff[D / 16], tlo[D / 32], thi[D / 32];
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ks++) foff[ks] = frag_off<D, kSwzDual>(c, ks * 2 + hf);
+#pragma unroll
+  for (int db = 0; db < D / 32; db++) {
+    tlo[db] = tr_off<D, kSwzDual>(0, db * 4, lane);
+    thi[db] = tr_off<D, kSwzDual>(8, db * 4, lane);
+  }
+  // P of a slab: [slab parity][pair][half t][lane] x 16 bytes
+  u32x4* const Pl = reinterpret_cast<u32x4*>(lds_raw + Cfg::kOffP + pr * Cfg::kPBytes) + lane;
+
+  if (n_slabs > 0) stage(mt_begin * BM, 0, 0);
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ks++) breg[ks] = bitcast<vec8>(key < Lk ? braw[ks] : u32x4{0, 0, 0, 0});
+
+  f32x16 x;  // first wave: S, then P of the slab;  second wave: dP - Dk of the slab it has started
+  auto accumulate = [&](const T* cols, vec8 x0, vec8 x1) {  // acc += cols^T (x0 | x1)
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+      u32x4 at[D / 32];
+#pragma unroll
+      for (int db = 0; db < D / 32; db++) {
+        const u32x2 lo = lds_read_tr16(cols + 16 * t * D + tlo[db]), hi = lds_read_tr16(cols + 16 * t * D + thi[db]);
+        at[db] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+      }
+#pragma unroll
+      for (int db = 0; db < D / 32; db++) acc[db] = E::mfma32(bitcast<vec8>(at[db]), t == 0 ? x0 : x1, acc[db]);
+    }
+  };
+  int q3 = 0, d2 = 0;  // buffers of slab i
+  for (int i = 0; i <= n_slabs; i++) {  // (the last round only lets the second waves finish the last slab)
+    if (n_slabs == 0) break;
+    const bool cur = i < n_slabs;
+    const int m0 = (mt_begin + i) * BM;
+    wait_vmem();
+    float* const lse_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffStat + d2 * Cfg::kStatBytes);
+    float* const dk_l = lse_l + BM;
+    if (cur && tid < 2 * BM) lse_l[tid] = stat_value();
+    __syncthreads();  // slab i is complete, P of slab i - 1 is there, nobody still reads what slab i + 1 will overwrite
+    const int q3n = q3 == 2 ? 0 : q3 + 1, q3p = q3 == 0 ? 2 : q3 - 1;
+    if (i + 1 < n_slabs) stage(m0 + BM, q3n, d2 ^ 1);
+    const T* const Ql = reinterpret_cast<const T*>(lds_raw + Cfg::kOffQ + q3 * Cfg::kTile);
+    const T* const dOl = reinterpret_cast<const T*>(lds_raw + Cfg::kOffdO + d2 * Cfg::kTile);
+
+    if (second && i > 0) {  // ---- finish slab i - 1: dS' = P o (dP - Dk), dK^T += Q^T dS'
+      const vec8 p0 = bitcast<vec8>(Pl[(d2 ^ 1) * (2 * Cfg::kPBytes / 16)]);
+      const vec8 p1 = bitcast<vec8>(Pl[(d2 ^ 1) * (2 * Cfg::kPBytes / 16) + 64]);
+      f32x8 d0, d1;
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        d0[e] = (float)p0[e] * x[e];
+        d1[e] = (float)p1[e] * x[8 + e];
+      }
+      accumulate(reinterpret_cast<const T*>(lds_raw + Cfg::kOffQ + q3p * Cfg::kTile), cvt8<T>(d0), cvt8<T>(d1));
+    }
+    if (cur) {
+      // ---- S = Q K^T (first wave) or dP - Dk = dO V^T - Dk (second wave: the accumulator starts from -Dk of its rows)
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        f32x4 nd4 = {0.f, 0.f, 0.f, 0.f};
+        if (second) nd4 = *reinterpret_cast<const f32x4*>(dk_l + 8 * j + 4 * hf);
+#pragma unroll
+        for (int e = 0; e < 4; e++) x[4 * j + e] = nd4[e];
+      }
+      {
+        const T* const rows = second ? dOl : Ql;
+        vec8 a[D / 16];
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ks++) a[ks] = *reinterpret_cast<const vec8*>(rows + foff[ks]);
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ks++) x = E::mfma32(a[ks], breg[ks], x);
+      }
+      if (!second) {  // ---- P, left for the partner; dV^T += dO^T P
+        if (kCausal && m0 < n0 + pr * 32 + 32) {  // the slab straddles the diagonal: scores above it become -inf (P = 0)
+#pragma unroll
+          for (int r = 0; r < 16; r++)
+            if (key > m0 + 8 * (r >> 2) + 4 * hf + (r & 3)) x[r] = -INFINITY;
+        }
+        f32x8 pf0, pf1;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_l + 8 * j + 4 * hf);
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float pe = fast_exp2(__builtin_fmaf(x[4 * j + e], cs, -lse4[e]));
+            if (j < 2) pf0[4 * j + e] = pe;
+            else pf1[4 * (j - 2) + e] = pe;
+          }
+        }
+        const vec8 p0 = cvt8<T>(pf0), p1 = cvt8<T>(pf1);
+        Pl[d2 * (2 * Cfg::kPBytes / 16)] = bitcast<u32x4>(p0);
+        Pl[d2 * (2 * Cfg::kPBytes / 16) + 64] = bitcast<u32x4>(p1);
+        accumulate(dOl, p0, p1);
+      }
+    }
+    q3 = q3n;
+    d2 ^= 1;
+  }
+
+  // ---- rotary: k came in rotated; dk goes out turned back by the angles of this lane's key, in fp32 before its rounding
+  if constexpr (kRot) {
+    if (second) {
+      const int t = key < p.rot_rows ? key : p.rot_rows - 1;
+#pragma unroll
+      for (int db = 0; db < D / 32; db++)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          f32x4 xr;
+#pragma unroll
+          for (int i = 0; i < 4; i++) xr[i] = acc[db][g4 * 4 + i];
+          xr = unrotate4<T>(xr, p.rot_cos, p.rot_sin, t, D / 2, db * 32 + g4 * 8 + hf * 4);
+#pragma unroll
+          for (int i = 0; i < 4; i++) acc[db][g4 * 4 + i] = xr[i];
+        }
+    }
+  }
+
+  // ---- epilogue: scale, transpose this wave's dV^T or dK^T through LDS, coalesced stores
+  __syncthreads();
+  constexpr int ES = Cfg::ES;
+  T* Stg = reinterpret_cast<T*>(lds_raw) + wave * 32 * ES;  // 32 keys x D per wave
+  const float f = second ? p.scale * p.rp_keep : p.rp_keep;
+#pragma unroll
+  for (int db = 0; db < D / 32; db++)
+#pragma unroll
+    for (int g4 = 0; g4 < 4; g4++) {
+      f32x4 xo;
+#pragma unroll
+      for (int i = 0; i < 4; i++) xo[i] = acc[db][g4 * 4 + i] * f;
+      *reinterpret_cast<vec4*>(Stg + c * ES + db * 32 + g4 * 8 + hf * 4) = cvt4<T>(xo);
+    }
+  __builtin_amdgcn_wave_barrier();
+  T* const gbase = second ? reinterpret_cast<T*>(p.dk) + (int64_t)k_begin * p.dk_rs + (int64_t)h * p.dk_hs
+                          : reinterpret_cast<T*>(p.dv) + (int64_t)k_begin * p.dv_rs + (int64_t)h * p.dv_hs;
+  const int64_t grs = second ? p.dk_rs : p.dv_rs;
+#pragma unroll
+  for (int i = 0; i < 32 * CH / 64; i++) {
+    const int ch = lane + i * 64;
+    const int row = ch / CH, col = (ch % CH) * 8;
+    const int krow = n0 + pr * 32 + row;
+    if (krow < Lk) st_global16(gbase + (int64_t)krow * grs + col, *reinterpret_cast<const u32x4*>(Stg + row * ES + col));
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 // dQ
 // ---------------------------------------------------------------------------------------------------------------
 // KS: key split as in the forward kernel (FwdCfg): 1 = four waves with 32 of the workgroup's 128 query rows each;

@@ -186,7 +186,7 @@ def load_library():
 def set_launch_policy(policy):
     """Tile shape: 0 chosen per launch (default), 1 always the full-size tiles, 2 the half-size tiles wherever they exist;
     plus the backward plan: 0x10 the dQ + dK/dV kernel pair (also the default), 0x20 the one-kernel backward where it
-    exists (fa_set_launch_policy)."""
+    exists; plus 0x40: the head-dim-128 dK/dV kernel as wave pairs where it exists (fa_set_launch_policy)."""
     lib = load_library()
     rc = lib.fa_set_launch_policy(int(policy))
     if rc != 0:

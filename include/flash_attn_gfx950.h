@@ -285,6 +285,9 @@ int fa_rotary(const fa_rotary_args* args);
  * Backward plan (bits 4-5): 0 (default) and 0x10: two kernels (dQ with softmax_d, then dK/dV), no scratch; 0x20: one kernel
  * that also passes dQ from key tile to key tile through fp32 scratch, where it exists (head_dim 64, no blockmask, mask,
  * dropout or bias, max_seqlen_k <= 4096) and only if the caller brings the scratch fa_bwd_workspace_bytes() then asks for.
+ * Bit 6 (0x40): at head_dim 128 without dropout, blockmask or bias the dK/dV kernel runs as wave pairs (one wave holds K and
+ * owns dV, its partner holds V and owns dK; 64 keys per workgroup) instead of four waves with 32 keys each and V in LDS.
+ * The defaults are the faster choices on the shapes measured; the others are kept for parts and shapes where the balance differs.
  * Results agree within rounding between the choices (the order of fp32 summation differs), not bit for bit; each choice is
  * reproducible bit for bit from run to run. */
 int fa_set_launch_policy(int policy);

@@ -406,9 +406,9 @@ def test_launch_policy_values_and_one_kernel_backward_scratch(lib):
     """fa_set_launch_policy: tile shape in the low bits, backward plan in 0x30; the one-kernel backward asks for scratch only
     where it exists (head dim 64, dense, no mask, dropout or bias, at most 32 key tiles)"""
     from flash_attn import flash_attn_gfx950 as be
-    for ok in (0, 1, 2, 0x10, 0x11, 0x12, 0x20, 0x21, 0x22):
+    for ok in (0, 1, 2, 0x10, 0x11, 0x12, 0x20, 0x21, 0x22, 0x40, 0x52):
         assert lib.fa_set_launch_policy(ok) == 0
-    for bad in (3, 0x30, 0x40, -1, 0x100):
+    for bad in (3, 0x30, 0x80, 0x43, -1, 0x100):
         assert lib.fa_set_launch_policy(bad) == -1 and b"launch policy" in lib.fa_last_error()
     a = be.BwdArgs()
     a.struct_bytes = ctypes.sizeof(a)

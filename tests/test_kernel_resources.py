@@ -115,3 +115,7 @@ def test_d128_backward_keeps_two_waves_per_simd():
             assert k["Occupancy"] >= 2 and k["VGPRs Spill"] == 0 and k["LDS Size"] <= 80 * 1024, (dt, flags, k)
             k = _pick(bwd, "fa_bwd_dq_kernel%sLi128E" % dt, flags + "Li1EEEv")
             assert k["Occupancy"] >= 2 and k["VGPRs Spill"] <= (1 if "Lb1ELi0E" in flags[8:] else 0), ("dq", dt, flags, k)
+        # the dK/dV kernel of wave pairs (launch policy 0x40) is built for three waves per SIMD and three workgroups' LDS
+        for flags in ("Lb0ELb0E", "Lb1ELb0E", "Lb0ELb1E", "Lb1ELb1E"):
+            k = _pick(bwd, "fa_bwd_dkdv_pair_kernel%s" % dt, flags + "EEv")
+            assert k["Occupancy"] >= 3 and k["VGPRs Spill"] <= 2 and k["LDS Size"] <= 160 * 1024 // 3, (dt, flags, k)

@@ -1552,6 +1552,55 @@ def test_blocksparse_modules_layout_sources_and_padding():
 
 
 # ------------------------------------------------------------------------------------------------
+# head dim 128: the dK/dV kernel of wave pairs (launch policy 0x40)
+# ------------------------------------------------------------------------------------------------
+@pytest.fixture
+def d128_wave_pairs():
+    from flash_attn import flash_attn_gfx950 as be
+    be.set_launch_policy(0x40)
+    yield
+    be.set_launch_policy(0)
+
+
+@pytest.mark.parametrize("lens_q,lens_k,dtype,causal,packing", [
+    ([256, 256], [256, 256], torch.float16, False, "qkv"),
+    ([300, 77, 1], [300, 77, 1], torch.bfloat16, True, "qkv"),
+    ([1024, 130], [1024, 130], torch.float16, True, "qkv"),
+    ([200, 31, 512], [640, 129, 96], torch.float16, False, "kv"),
+    ([33], [1500], torch.bfloat16, False, "sep"),
+    ([700, 5], [1, 260], torch.float16, False, "sep"),
+])
+def test_d128_wave_pair_dkdv_parity(lens_q, lens_k, dtype, causal, packing, d128_wave_pairs):
+    """the parity bar of the default kernels, on shapes with ragged ends, single rows, more keys than queries and the reverse"""
+    _parity_case(lens_q, lens_k, 3, 128, dtype, causal, packing=packing, seed=7)
+
+
+def test_d128_wave_pair_dkdv_full_size_and_rotary(d128_wave_pairs):
+    """B=16 H=12 N=2048 against the default kernels (same arithmetic, P handed to the partner wave rounded: dK within a
+    rounding of the default's, dV bit for bit), twice (reproducible), and with the rotation inside the kernels"""
+    from flash_attn import flash_attn_gfx950 as be
+    from flash_attn.rotary import RotaryEmbedding
+    torch.manual_seed(1)
+    B, H, D, N = 16, 12, 128, 2048
+    qkv = torch.randn(B * N, 3, H, D, device="cuda").half()
+    do = torch.randn(B * N, H, D, device="cuda").half()
+    cu = _cu([N] * B)
+    q, k, v = qkv[:, 0], qkv[:, 1], qkv[:, 2]
+    cos_h, sin_h = RotaryEmbedding(D).half_tables(torch.empty(1, N, 3, H, D, device="cuda", dtype=torch.float16))
+    for causal, rotary in ((False, None), (True, None), (False, (cos_h, sin_h))):
+        o, lse = be.fwd(q, k, v, cu, cu, N, N, 0.0, D ** -0.5, False, causal, False)
+        grads = []
+        for policy in (0, 0x40, 0x40):
+            be.set_launch_policy(policy)
+            g = torch.empty_like(qkv)
+            be.bwd(do, q, k, v, o, lse, g[:, 0], g[:, 1], g[:, 2], cu, cu, N, N, 0.0, D ** -0.5, False, causal, rotary=rotary)
+            grads.append(g)
+        assert torch.equal(grads[1], grads[2])
+        assert torch.equal(grads[0][:, 0], grads[1][:, 0]) and torch.equal(grads[0][:, 2], grads[1][:, 2])
+        assert _maxerr(grads[0][:, 1], grads[1][:, 1]) <= 2.0 ** -9 * float(grads[0][:, 1].abs().max())
+
+
+# ------------------------------------------------------------------------------------------------
 # rotary embedding kernel (fa_rotary) against the oracle; tolerance: one rounding of the result (the reference's
 # elementwise fp16 ops round three times, rotary.py:32-42)
 # ------------------------------------------------------------------------------------------------
