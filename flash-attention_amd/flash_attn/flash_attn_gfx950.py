@@ -120,7 +120,7 @@ EXPORTED_SYMBOLS = (
     "fa_fwd", "fa_bwd", "fa_fwd_block", "fa_bwd_block", "fa_fwd_block_noalloc", "fa_fwd_workspace_bytes", "fa_bwd_workspace_bytes",
     "fa_round_seqlens", "fa_philox_offset_increment", "fa_last_error", "fa_abi_version",
     "fa_gather_rows", "fa_scatter_rows", "fa_scatter_rows_workspace_bytes", "fa_rotary", "fa_set_launch_policy",
-    "fa_keep_words_bytes",
+    "fa_keep_words_bytes", "fa_blocksparse_row_order",
 )
 # declared in include/flash_attn_gfx950_bench.h: instrumentation for bench.py, not part of the drop-in boundary
 BENCH_SYMBOLS = ("fa_bwd_profiled",)
@@ -175,6 +175,8 @@ def load_library():
         lib.fa_scatter_rows_workspace_bytes.restype = ctypes.c_size_t
         lib.fa_rotary.argtypes = [ctypes.POINTER(RotaryArgs)]
         lib.fa_rotary.restype = ctypes.c_int
+        lib.fa_blocksparse_row_order.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
+        lib.fa_blocksparse_row_order.restype = ctypes.c_int
         lib.fa_set_launch_policy.argtypes = [ctypes.c_int]
         lib.fa_set_launch_policy.restype = ctypes.c_int
         if lib.fa_abi_version() != FA_ABI_VERSION:
@@ -248,8 +250,8 @@ def _philox_state(device, p_dropout, gen):
 
 
 def _stream_handle(device):
-    idx = device.index if device.index is not None else torch.cuda.current_device()
-    return torch._C._cuda_getCurrentRawStream(idx)
+    """hipStream_t of torch's current stream on `device`, as an integer."""
+    return torch.cuda.current_stream(device).cuda_stream
 
 
 class _OnDevice:
@@ -350,46 +352,18 @@ def blockmask_row_order(layout):
     """An order of the 16-row blocks of a block-sparse layout ((rows / 16, keys / 256) of 0 / 1) for the `row_order` argument
     of fwd_block / bwd_block.  A workgroup of the forward and of the dQ kernel owns eight consecutive entries and stages every
     key tile that any of the eight lists; each of its waves owns two consecutive entries and computes on every tile that
-    either of the two lists.  Greedy: a group starts with the fullest row block left and takes, seven times, the row block
-    that adds the fewest key blocks to the group's set (most shared ones on a tie); inside a group the two row blocks with
-    the smallest union are paired, then the next two.  If that saves less than 5 % of the staged tiles against the plain
-    order 0, 1, 2, ... (layouts made of whole 128-row tiles), the plain order is returned.  int32 tensor on the layout's
-    device; computed on the host."""
+    either of the two lists.  fa_blocksparse_row_order (host code of the library) groups row blocks with similar lists: a
+    greedy grouping, then exchanges that lower the staged and computed tiles; the plain order 0, 1, 2, ... if that saves
+    less than 5 % of the staged tiles (layouts made of whole 128-row tiles).  int32 tensor on the layout's device."""
     import numpy as np
-    m = (layout != 0).cpu().numpy()
-    nr, nc = m.shape
-    left = np.ones(nr, dtype=bool)
-    counts = m.sum(1)
-    order, staged = [], 0
-    while left.any():
-        seed = int(np.argmax(np.where(left, counts, -1)))
-        left[seed] = False
-        group, union = [seed], m[seed].copy()
-        while len(group) < 8 and left.any():
-            added = (m & ~union).sum(1)
-            shared = (m & union).sum(1)
-            score = np.where(left, added * (nc + 1) - shared, np.iinfo(np.int64).max)
-            best = int(np.argmin(score))
-            left[best] = False
-            group.append(best)
-            union |= m[best]
-        staged += int(union.sum())
-        rest = sorted(group)
-        while len(rest) >= 2:  # pair the two with the smallest union (the wave's work), ties: the lowest row blocks
-            best = None
-            for i in range(len(rest)):
-                for j in range(i + 1, len(rest)):
-                    u = int((m[rest[i]] | m[rest[j]]).sum())
-                    if best is None or u < best[0]:
-                        best = (u, i, j)
-            _, i, j = best
-            order += [rest[i], rest[j]]
-            rest = [r for n, r in enumerate(rest) if n not in (i, j)]
-        order += rest
-    plain = sum(int(m[i:i + 8].any(0).sum()) for i in range(0, nr, 8))
-    if staged > 0.95 * plain:
-        order = list(range(nr))
-    return torch.tensor(order, dtype=torch.int32, device=layout.device)
+    m = np.ascontiguousarray((layout != 0).cpu().numpy().astype(np.uint8))
+    _check(m.ndim == 2, "layout must be (rows / 16, keys / 256)")
+    order = np.empty(m.shape[0], dtype=np.int32)
+    lib = load_library()
+    rc = lib.fa_blocksparse_row_order(m.ctypes.data, m.shape[0], m.shape[1], order.ctypes.data)
+    if rc != 0:
+        _raise(rc, lib)
+    return torch.from_numpy(order).to(layout.device)
 
 
 def _rotary_arg(a, rotary, q, rows_needed):

@@ -277,6 +277,14 @@ typedef struct fa_rotary_args {
 } fa_rotary_args;
 int fa_rotary(const fa_rotary_args* args);
 
+/* Host-side helper of the block-sparse entry points (no GPU work, no counterpart in the reference): an order of the 16-row
+ * blocks for fa_fwd_args.row_order / fa_bwd_args.row_order that puts row blocks with similar key-block lists into the same
+ * workgroup (eight consecutive entries) and wave (two).  layout: HOST array [n_row_blocks][n_col_blocks] of bytes, non-zero
+ * = the 16 x 256 block is listed (the layout before convert_blockmask); order: HOST array of n_row_blocks int32, written:
+ * a permutation of 0 .. n_row_blocks - 1, the identity if reordering would save less than 5 % of the staged key blocks.
+ * Deterministic; a greedy grouping followed by 2000 * n_row_blocks exchange attempts (tens of milliseconds for 4096 tokens). */
+int fa_blocksparse_row_order(const uint8_t* layout, int32_t n_row_blocks, int32_t n_col_blocks, int32_t* order);
+
 /* Launch policy (process-wide state; no counterpart in the reference, whose launchers pick their tile by head size
  * and sequence length alone, fmha_api.cpp:232-241).  policy = tile shape | backward plan.
  * Tile shape (bits 0-1): 0 (default): short-sequence launches that would leave compute units idle with the full-size

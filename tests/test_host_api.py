@@ -201,23 +201,32 @@ def test_public_signatures_match_the_reference():
 
 
 def test_blockmask_row_order_is_a_permutation_that_groups_similar_rows():
-    """the greedy grouping lists every row block once, never stages more tiles than the plain order, saves a third of them
-    on independently drawn 16 x 256 blocks and leaves layouts made of whole 128-row tiles alone"""
+    """fa_blocksparse_row_order (host code of the library) lists every row block once, is deterministic, never stages more
+    key blocks than the plain order, saves a third of the staged blocks and a fifth of the waves' work on independently drawn
+    16 x 256 blocks, handles more than 64 key blocks and ragged ends, and leaves layouts made of whole 128-row tiles alone"""
     from flash_attn import flash_attn_gfx950 as be
     g = torch.Generator().manual_seed(0)
 
-    def staged(m, order):
+    def staged(m, order):  # key blocks a workgroup (eight consecutive entries) has to stage, summed
         return sum(int(m[order[i:i + 8]].any(0).sum()) for i in range(0, len(order), 8))
 
-    for nrow, ncol, dens in ((256, 16, 0.25), (19, 2, 0.5), (64, 4, 0.1), (8, 1, 1.0), (1, 1, 0.0)):
+    def computed(m, order):  # key blocks a wave (two consecutive entries) has to compute on, summed
+        return sum(int(m[order[i:i + 2]].any(0).sum()) for i in range(0, len(order), 2))
+
+    for nrow, ncol, dens in ((256, 16, 0.25), (19, 2, 0.5), (64, 4, 0.1), (8, 1, 1.0), (1, 1, 0.0), (100, 70, 0.2)):
         m = torch.rand(nrow, ncol, generator=g) < dens
         order = be.blockmask_row_order(m)
         assert order.dtype == torch.int32 and sorted(order.tolist()) == list(range(nrow))
-        assert staged(m, order.long()) <= staged(m, torch.arange(nrow))
+        assert torch.equal(order, be.blockmask_row_order(m))
+        ident = torch.arange(nrow)
+        assert staged(m, order.long()) <= staged(m, ident)
         if nrow == 256:
-            assert staged(m, order.long()) < 0.7 * staged(m, torch.arange(nrow))
+            assert staged(m, order.long()) < 0.7 * staged(m, ident)
+            assert computed(m, order.long()) < 0.82 * computed(m, ident)
     tiles = (torch.rand(16, 16, generator=g) < 0.3).repeat_interleave(16, 0)  # 256 x 256 blocks
     assert be.blockmask_row_order(tiles).tolist() == list(range(256))
+    lib = be.load_library()
+    assert lib.fa_blocksparse_row_order(None, 4, 4, None) == -1
 
 
 # ---------------------------------------------------------------- host helpers
