@@ -89,7 +89,10 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasT
   // XCD-aware id map (see map_tile): the key tiles of one (batch, head) share one XCD's L2 copy of Q and dO.
   int bh, kt;  // under a causal mask the first key tiles see the most query rows: rank order is already heavy-first
   if (!map_tile<kCausal>(blockIdx.x, p.nk_tiles, p.B * p.H, &bh, &kt, p.tile_group)) return;
-  const int b = bh / p.H, h = bh % p.H;
+  const int h = bh % p.H;
+  // (dense, no mask: the batch entries are taken longest first - here by their queries, which a key tile walks; longest_first)
+  const int b = (!kCausal && !kSparse && p.tile_group < 0) ? longest_first(p.cu_q, p.B, bh / p.H) : bh / p.H;
+  bh = b * p.H + h;  // (what the dropout counters and the keep words are indexed by)
 
   int q_begin = 0, Lq = 0, k_begin, Lk;
   if (!seq_extent(p.cu_k, b, p.total_k, p.max_sk, &k_begin, &Lk)) return;
@@ -799,7 +802,10 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
   const int split = rank % n_splits;
   rank /= n_splits;
   const int qt = kCausal ? p.nq_tiles - 1 - rank : rank;
-  const int b = bh / p.H, h = bh % p.H;
+  const int h = bh % p.H;
+  // (dense, no mask: the batch entries are taken longest keys first, see longest_first)
+  const int b = (!kCausal && !kSparse && p.tile_group < 0) ? longest_first(p.cu_k, p.B, bh / p.H) : bh / p.H;
+  bh = b * p.H + h;  // (what the dropout counters and the keep words are indexed by)
 
   int q_begin, Lq, k_begin = 0, Lk = 0;
   if (!seq_extent(p.cu_q, b, p.total_q, p.max_sq, &q_begin, &Lq)) return;

@@ -51,7 +51,7 @@ struct FwdCfg {
 // kWords (dropout, dense): the keep decisions are also left in p.keep_words for the backward (fa_common.h)
 template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, int kBias = 0, int KS = 1,
           bool kWords = false>
-__global__ void __launch_bounds__(256, (!kDropout && kBias == 0 && D <= 64) ? 4 : ((!kDropout && kBias == kBiasTensor && D <= 64) ? 3 : 2)) fa_fwd_kernel(const FwdParams p) {
+__global__ void __launch_bounds__(256, ((!kDropout || KS == 2) && kBias == 0 && D <= 64) ? 4 : ((!kDropout && kBias == kBiasTensor && D <= 64) ? 3 : 2)) fa_fwd_kernel(const FwdParams p) {
   constexpr bool kAlibi = kBias == kBiasAlibi, kTensorBias = kBias == kBiasTensor;
   static_assert(!kWords || (kDropout && !kSparse), "keep words: dense dropout variants only");
   static_assert(kBias == 0 || !kSparse, "score bias: dense variants only");
@@ -73,7 +73,10 @@ __global__ void __launch_bounds__(256, (!kDropout && kBias == 0 && D <= 64) ? 4 
   const int split = rank % n_splits;
   rank /= n_splits;
   const int qt = kCausal ? p.nq_tiles - 1 - rank : rank;  // under a causal mask the last query tiles cost most
-  const int b = bh / p.H, h = bh % p.H;
+  const int h = bh % p.H;
+  // (dense, no mask: the batch entries are taken longest keys first, see longest_first)
+  const int b = (!kCausal && !kSparse && p.tile_group < 0) ? longest_first(p.cu_k, p.B, bh / p.H) : bh / p.H;
+  bh = b * p.H + h;  // (what the dropout counters and the keep words are indexed by)
 
   int q_begin, Lq, k_begin = 0, Lk = 0;
   if (!seq_extent(p.cu_q, b, p.total_q, p.max_sq, &q_begin, &Lq)) return;

@@ -183,6 +183,29 @@ FA_DEVICE bool seq_extent(const int32_t* cu, int b, int total, int max_len, int*
   return true;
 }
 
+// Ragged batches: workgroup ids enumerate the batch entries longest first.  A launch deals its workgroups out in id order;
+// the entries with the longest walks should be under way first and - in a grid that is resident all at once - spread over
+// the compute units instead of arriving together as some units' third workgroup.  Slot `slot` of the launch's batch
+// dimension therefore goes to the entry with the slot-th largest length in cu (ties: lower index first, so a batch of
+// equal lengths keeps its order).  Every wave finds the entry itself: lane i holds entry i's length, counts the entries
+// that precede it (one readlane and compare per entry), and the lane whose count is `slot` is the answer.  Batches of
+// more than 64 entries keep their order.  The search costs every workgroup's prologue a few instructions per batch entry,
+// so the launchers ask for it (tile_group < 0 in a launch without a mask) only for grids that are resident all at once
+// (longest_first_launch), where the spreading is what it buys.
+FA_DEVICE int longest_first(const int32_t* cu, int B, int slot) {
+  if (B > 64 || B < 2) return slot;
+  const int lane = threadIdx.x & 63;
+  const int i = lane < B ? lane : B - 1;
+  const int len = cu[i + 1] - cu[i];
+  int before = 0;
+  for (int j = 0; j < B; j++) {
+    const int lj = __builtin_amdgcn_readlane(len, j);
+    before += (lj > len || (lj == len && j < lane)) ? 1 : 0;
+  }
+  const uint64_t hit = __builtin_amdgcn_ballot_w64(lane < B && before == slot);
+  return __builtin_amdgcn_readfirstlane(hit != 0 ? (int)__builtin_ctzll(hit) : slot);
+}
+
 // Workgroup id -> (batch*head, tile rank).  The hardware deals consecutive workgroup ids to the 8 XCDs in turn
 // (id % 8), and each XCD has its own L2.
 //   kTileMajor = false (tiles of equal cost): the tiles of one (batch, head) are consecutive in one XCD's share of the
@@ -235,6 +258,11 @@ FA_DEVICE bool map_tile(int block, int tiles_per_bh, int BH, int* bh, int* rank,
 }
 inline int tile_grid(bool tile_major, int tiles_per_bh, int BH) {
   return ((BH + 7) & ~7) * tiles_per_bh;
+}
+// see longest_first: dense launches without a mask whose grid is resident all at once (at most 4 workgroups on each of the
+// 256 compute units), 2 to 64 batch entries
+inline bool longest_first_launch(bool causal, bool sparse, int grid, int B) {
+  return !causal && !sparse && grid <= 1024 && B >= 2 && B <= 64;
 }
 
 // Launch shape: with 128-row tiles a short-sequence batch gives the compute units one or two workgroups each, and one
