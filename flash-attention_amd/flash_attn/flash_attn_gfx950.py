@@ -189,10 +189,12 @@ def set_launch_policy(policy):
     """Tile shape: 0 chosen per launch (default), 1 always the full-size tiles, 2 the half-size tiles wherever they exist;
     plus the backward plan: 0x10 the dQ + dK/dV kernel pair (also the default), 0x20 the one-kernel backward where it
     exists; plus 0x40: the head-dim-128 dK/dV kernel as wave pairs where it exists (fa_set_launch_policy)."""
+    global _policy_epoch
     lib = load_library()
     rc = lib.fa_set_launch_policy(int(policy))
     if rc != 0:
         _raise(rc, lib)
+    _policy_epoch += 1
 
 
 @functools.lru_cache(maxsize=256)
@@ -249,9 +251,39 @@ def _philox_state(device, p_dropout, gen):
     return seed & 0xFFFFFFFFFFFFFFFF, offset & 0xFFFFFFFFFFFFFFFF
 
 
+# torch's current stream as a raw hipStream_t: the public route (torch.cuda.current_stream(device).cuda_stream) builds a
+# Stream object per call and costs 4 us, a fifth of a whole call here; the accessor below is what it wraps
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_handle(device):
     """hipStream_t of torch's current stream on `device`, as an integer."""
+    if _raw_stream is not None:
+        return _raw_stream(device.index if device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
+
+
+# Argument structs are kept per thread and per call signature (shapes, strides, flags): a call then only writes what changes
+# from call to call - pointers, dropout state, stream - instead of allocating and filling forty fields, and does not ask the
+# library for the workspace size again.  set_launch_policy() empties the cache (the workspace size depends on the policy).
+_args_tls = threading.local()
+_policy_epoch = 0
+
+
+def _cached_args(key, cls, fill):
+    """(struct, workspace bytes) for a call signature; fill(struct) -> workspace bytes runs on a miss."""
+    cache = getattr(_args_tls, "cache", None)
+    if cache is None or getattr(_args_tls, "epoch", -1) != _policy_epoch:
+        cache = _args_tls.cache = {}
+        _args_tls.epoch = _policy_epoch
+    ent = cache.get(key)
+    if ent is None:
+        if len(cache) >= 512:
+            cache.clear()
+        a = cls()
+        a.struct_bytes = ctypes.sizeof(cls)
+        ent = cache[key] = (a, fill(a))
+    return ent
 
 
 class _OnDevice:
@@ -408,28 +440,43 @@ def _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_
         lse = torch.empty((batch, nheads, sq_r), dtype=torch.float32, device=dev)
         s = torch.empty((batch, nheads, sq_r, sk_r), dtype=q.dtype, device=dev) if return_softmax else None
         seed, offset = _philox_state(dev, p_dropout, gen)
-        a = FwdArgs()
-        a.struct_bytes = ctypes.sizeof(FwdArgs)
-        a.dtype = code
+        qs, ks, vs = q.stride(), k.stride(), v.stride()
+        mq, mk = int(max_seqlen_q), int(max_seqlen_k)
+        dropout = p_dropout > 0
+
+        def fill(a):  # everything a call signature fixes; returns the workspace size of such calls
+            a.dtype = code
+            a.q_row_stride, a.q_head_stride = qs[0], qs[1]
+            a.k_row_stride, a.k_head_stride = ks[0], ks[1]
+            a.v_row_stride, a.v_head_stride = vs[0], vs[1]
+            a.o_row_stride, a.o_head_stride = nheads * head_dim, head_dim
+            a.batch, a.nheads, a.head_dim = batch, nheads, head_dim
+            a.total_q, a.total_k = total_q, total_k
+            a.max_seqlen_q, a.max_seqlen_k = mq, mk
+            a.zero_tensors, a.is_causal = int(bool(zero_tensors)), int(bool(is_causal))
+            # (the size query reads shapes, is_causal, p_dropout > 0 and which optional pointers are set)
+            a.p_dropout = float(p_dropout)
+            a.blockmask = 16 if sparse else None
+            a.alibi_slopes = 16 if alibi_slopes is not None else None
+            a.attn_bias = 16 if attn_bias is not None else None
+            return lib.fa_fwd_workspace_bytes(ctypes.byref(a))
+
+        a, ws_bytes = _cached_args(("fwd", code, qs, ks, vs, batch, nheads, head_dim, total_q, total_k, mq, mk,
+                                    bool(zero_tensors), bool(is_causal), dropout, sparse, alibi_slopes is not None,
+                                    attn_bias is not None), FwdArgs, fill)
         a.q, a.k, a.v, a.o = q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr()
         a.softmax_lse = lse.data_ptr()
         a.s_dmask = s.data_ptr() if s is not None else None
         a.cu_seqlens_q, a.cu_seqlens_k = cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr()
         a.blockmask = blockmask.data_ptr() if sparse else None
-        a.q_row_stride, a.q_head_stride = q.stride(0), q.stride(1)
-        a.k_row_stride, a.k_head_stride = k.stride(0), k.stride(1)
-        a.v_row_stride, a.v_head_stride = v.stride(0), v.stride(1)
-        a.o_row_stride, a.o_head_stride = o.stride(0), o.stride(1)
-        a.batch, a.nheads, a.head_dim = batch, nheads, head_dim
-        a.total_q, a.total_k = total_q, total_k
-        a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
         a.p_dropout, a.softmax_scale = float(p_dropout), float(softmax_scale)
-        a.zero_tensors, a.is_causal = int(bool(zero_tensors)), int(bool(is_causal))
         a.philox_seed, a.philox_offset = seed, offset
-        ws_bytes = lib.fa_fwd_workspace_bytes(ctypes.byref(a))
         ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev) if ws_bytes else None
         a.workspace = ws.data_ptr() if ws is not None else None
         a.workspace_bytes = ws_bytes
+        # (the struct is reused: the optional fields are cleared before the helpers below set the ones that are given)
+        a.keep_words, a.keep_words_bytes, a.attn_bias, a.row_order = None, 0, None, None
+        a.rotary_cos, a.rotary_sin, a.q_rot = None, None, None
         a.stream = _stream_handle(dev)
         a.alibi_slopes = _check_alibi(alibi_slopes, nheads, dev, sparse)
         _keep_words_arg(a, keep_words, dev, sparse)
@@ -479,34 +526,45 @@ def _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seql
     with _OnDevice(dev):
         softmax_d = torch.empty((batch, nheads, sq_r), dtype=torch.float32, device=dev)
         seed, offset = _philox_state(dev, p_dropout, gen)
-        a = BwdArgs()
-        a.struct_bytes = ctypes.sizeof(BwdArgs)
-        a.dtype = code
+        strides = (dout.stride(), q.stride(), k.stride(), v.stride(), out.stride(), dq.stride(), dk.stride(), dv.stride())
+        mq, mk = int(max_seqlen_q), int(max_seqlen_k)
+        lse_stride = softmax_lse.shape[2]
+
+        def fill(a):  # everything a call signature fixes; returns the workspace size of such calls
+            a.dtype = code
+            for name, st in zip(("do", "q", "k", "v", "o", "dq", "dk", "dv"), strides):
+                setattr(a, name + "_row_stride", st[0])
+                setattr(a, name + "_head_stride", st[1])
+            a.lse_seq_stride = lse_stride
+            a.batch, a.nheads, a.head_dim = batch, nheads, head_dim
+            a.total_q, a.total_k = total_q, total_k
+            a.max_seqlen_q, a.max_seqlen_k = mq, mk
+            a.zero_tensors, a.is_causal = int(bool(zero_tensors)), int(bool(is_causal))
+            # (the size query reads shapes, is_causal, p_dropout > 0 and which optional pointers are set)
+            a.p_dropout = float(p_dropout)
+            a.blockmask = 16 if sparse else None
+            a.alibi_slopes = 16 if alibi_slopes is not None else None
+            a.attn_bias = 16 if attn_bias is not None else None
+            a.rotary_cos = 16 if rotary is not None else None
+            return lib.fa_bwd_workspace_bytes(ctypes.byref(a))
+
+        a, ws_bytes = _cached_args(("bwd", code, strides, lse_stride, batch, nheads, head_dim, total_q, total_k, mq, mk,
+                                    bool(zero_tensors), bool(is_causal), p_dropout > 0, sparse, alibi_slopes is not None,
+                                    attn_bias is not None, rotary is not None), BwdArgs, fill)
         a.dout, a.q, a.k, a.v, a.out = dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
         a.softmax_lse = softmax_lse.data_ptr()
         a.dq, a.dk, a.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
         a.softmax_d = softmax_d.data_ptr()
         a.cu_seqlens_q, a.cu_seqlens_k = cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr()
         a.blockmask = blockmask.data_ptr() if sparse else None
-        a.do_row_stride, a.do_head_stride = dout.stride(0), dout.stride(1)
-        a.q_row_stride, a.q_head_stride = q.stride(0), q.stride(1)
-        a.k_row_stride, a.k_head_stride = k.stride(0), k.stride(1)
-        a.v_row_stride, a.v_head_stride = v.stride(0), v.stride(1)
-        a.o_row_stride, a.o_head_stride = out.stride(0), out.stride(1)
-        a.dq_row_stride, a.dq_head_stride = dq.stride(0), dq.stride(1)
-        a.dk_row_stride, a.dk_head_stride = dk.stride(0), dk.stride(1)
-        a.dv_row_stride, a.dv_head_stride = dv.stride(0), dv.stride(1)
-        a.lse_seq_stride = softmax_lse.shape[2]
-        a.batch, a.nheads, a.head_dim = batch, nheads, head_dim
-        a.total_q, a.total_k = total_q, total_k
-        a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
         a.p_dropout, a.softmax_scale = float(p_dropout), float(softmax_scale)
-        a.zero_tensors, a.is_causal = int(bool(zero_tensors)), int(bool(is_causal))
         a.philox_seed, a.philox_offset = seed, offset
-        ws_bytes = lib.fa_bwd_workspace_bytes(ctypes.byref(a))
         ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev) if ws_bytes else None
         a.workspace = ws.data_ptr() if ws is not None else None
         a.workspace_bytes = ws_bytes
+        # (the struct is reused: the optional fields are cleared before the helpers below set the ones that are given)
+        a.keep_words, a.keep_words_bytes, a.attn_bias, a.dbias, a.row_order = None, 0, None, None, None
+        a.rotary_cos, a.rotary_sin = None, None
         a.stream = _stream_handle(dev)
         a.alibi_slopes = _check_alibi(alibi_slopes, nheads, dev, sparse)
         _keep_words_arg(a, keep_words, dev, sparse)
