@@ -502,6 +502,12 @@ def main():
         "what": "standard attention with PyTorch fp16 ops, fwd+bwd, same inputs, same GPU: the comparison point of the "
                 "reference's published speed-ups (about 2x on A100 for this shape without mask or dropout) and memory "
                 "savings (about 10x at N=2048); step memory = peak device memory of one fwd+bwd beyond its inputs"}
+    # with dropout the autograd function also holds the keep words (one bit per score) from forward to backward, when they
+    # are no larger than q, k and v together
+    wd = Workload(torch, B, H, D, N, torch.float16, p=0.1)
+    res["pytorch_attention_same_gpu"]["fused_step_memory_mb_dropout"] = round(fused_step_memory(torch, wd) / 2 ** 20, 1)
+    res["pytorch_attention_same_gpu"]["keep_words_mb"] = round(wd.keep_words.numel() / 2 ** 20, 1) if wd.keep_words is not None else 0.0
+    del wd
     if not a.no_cpu:
         res["cpu_baseline"] = cpu_baseline(torch, B, H, D, N, a.cpu_budget)
     else:

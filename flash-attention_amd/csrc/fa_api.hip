@@ -457,6 +457,14 @@ int bwd_impl(const fa_bwd_args* a, bool want_block, void* ev_main_start = nullpt
     p.n_splits = sp.n_splits;
     p.dq_part = reinterpret_cast<float*>(a->workspace);
   }
+  if (!split && fa::merged_backward_launch(a->head_dim, a->batch * a->nheads, a->max_seqlen_q, a->is_causal != 0, dropout,
+                                           p.keep_words != nullptr, sparse, p.alibi != nullptr || p.bias != nullptr,
+                                           p.rot_cos != nullptr, sp.n_splits)) {
+    if (ev_main_start) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(ev_main_start), stream));
+    FA_LAUNCH(fa::launch_bwd(p, 2, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));  // both in one launch
+    if (ev_main_stop) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(ev_main_stop), stream));
+    return FA_OK;
+  }
   FA_LAUNCH(fa::launch_bwd(p, 0, a->dtype, a->head_dim, a->is_causal != 0, dropout, sparse, stream));  // dQ, softmax_d
   if (split) FA_LAUNCH(fa::launch_dq_combine(p, a->dtype, a->head_dim, stream));
   if (ev_main_start) FA_LAUNCH(hipEventRecord(reinterpret_cast<hipEvent_t>(ev_main_start), stream));

@@ -60,6 +60,7 @@ struct BwdCfg {
   static constexpr int kLdsBytes = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
   static constexpr int CH = D / 8;
   static constexpr int kMinBlocks = (D == 128 && kDropout) ? 1 : 2;
+  static constexpr int kBiasTileBytes = BM * 32 * 2;  // per wave, behind everything else: the bias-tensor variants' tile
 };
 
 // kDrop: 0 = no dropout; 1 = the keep decisions are drawn here (Philox); 2 = they are read from the keep words the
@@ -67,9 +68,14 @@ struct BwdCfg {
 // kBias: as in fa_fwd_kernel; with a bias tensor the kernel also leaves d(loss)/d(bias) in p.dbias if that is not null
 // kRot: the keys came in rotated (rotary position embedding) and dK goes out turned back (dense variants without score bias
 // only; a variant of its own because the plain kernels sit at their register limit)
-template <typename T, int D, bool kCausal, int kDrop, bool kSparse, int kBias = 0, bool kRot = false>
-__global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasTensor) ? 3 : ((D == 128 && kBias == kBiasTensor) ? 1 : BwdCfg<T, D, kDrop == 1>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
+// (the kernel proper is fa_bwd_dkdv_kernel below: `block` is its workgroup id, `lds_raw` its LDS)
+// kOwnD: the kernel forms Dk = keep * rowsum(dO o O) of every tile's rows itself instead of reading what the dQ kernel left in
+// p.dsoftmax (four threads per row, 16 elements each, fetched with the tile): it then depends on nothing the dQ kernel writes,
+// and the two can share one launch (fa_bwd_merged_kernel).  64-row tiles, head dim 64.
+template <typename T, int D, bool kCausal, int kDrop, bool kSparse, int kBias = 0, bool kRot = false, bool kOwnD = false>
+FA_DEVICE void fa_bwd_dkdv_body(const BwdParams& p, const int block, unsigned char* const lds_raw) {
   static_assert(!kRot || (!kSparse && kBias == 0), "rotary: dense variants without score bias");
+  static_assert(!kOwnD || (D == 64 && !kSparse && kBias == 0 && BwdCfg<T, D, kDrop == 1>::BM == 64), "own Dk: d = 64, dense");
   constexpr bool kDropout = kDrop == 1, kStored = kDrop == 2;
   constexpr bool kAlibi = kBias == kBiasAlibi, kTensorBias = kBias == kBiasTensor;
   static_assert(!(kStored && kSparse), "keep words: dense only");
@@ -84,11 +90,11 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasT
 
   // kTensorBias: behind everything else, per wave BM rows x its 32 keys of bias (see load_bias below)
   constexpr int kBiasTileBytes = BM * 32 * 2;
-  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes + (kBias == kBiasTensor ? 4 * kBiasTileBytes : 0)];
+  static_assert(kBiasTileBytes == BwdCfg<T, D, kDrop == 1>::kBiasTileBytes, "LDS size of the kernel");
 
   // XCD-aware id map (see map_tile): the key tiles of one (batch, head) share one XCD's L2 copy of Q and dO.
   int bh, kt;  // under a causal mask the first key tiles see the most query rows: rank order is already heavy-first
-  if (!map_tile<kCausal>(blockIdx.x, p.nk_tiles, p.B * p.H, &bh, &kt, p.tile_group)) return;
+  if (!map_tile<kCausal>(block, p.nk_tiles, p.B * p.H, &bh, &kt, p.tile_group)) return;
   const int h = bh % p.H;
   // (dense, no mask: the batch entries are taken longest first - here by their queries, which a key tile walks; longest_first)
   const int b = (!kCausal && !kSparse && p.tile_group < 0) ? longest_first(p.cu_q, p.B, bh / p.H) : bh / p.H;
@@ -169,16 +175,28 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasT
   uint32_t kwpre = 0;
   const uint32_t* const kw_wave =
       kStored ? p.keep_words + ((int64_t)bh * p.kw_kb + (n0 >> 5) + wave) * p.kw_q : nullptr;
+  // kOwnD: this thread's quarter (16 elements) of row tid / 4 of the tile's dO and O
+  u32x4 dopre[kOwnD ? 2 : 1], opre[kOwnD ? 2 : 1];
+  const T* const do_quarter = reinterpret_cast<const T*>(p.dout) + (int64_t)q_begin * p.do_rs + (int64_t)h * p.do_hs + (tid & 3) * 16;
+  const T* const o_quarter = reinterpret_cast<const T*>(p.out) + (int64_t)q_begin * p.o_rs + (int64_t)h * p.o_hs + (tid & 3) * 16;
   auto stage = [&](int mt, int buf) {
     const int m0 = mt * BM;
     if (tid < BM) {
       const int row = m0 + tid;
       statpre = INFINITY;  // rows past the end are switched off (P = 0)
       if (row < Lq) statpre = lsebase[row];
-    } else if (tid < 2 * BM) {
+    } else if (!kOwnD && tid < 2 * BM) {
       const int row = m0 + tid - BM;
       statpre = 0.f;
       if (row < Lq) statpre = dsbase[row];
+    }
+    if constexpr (kOwnD) {  // (rows past the end read the last row: their P is 0, any finite Dk will do)
+      const int row = m0 + (tid >> 2) < Lq ? m0 + (tid >> 2) : Lq - 1;
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        dopre[i] = ld_global16(do_quarter + (int64_t)row * p.do_rs + 8 * i);
+        opre[i] = ld_global16(o_quarter + (int64_t)row * p.o_rs + 8 * i);
+      }
     }
     if (kStored && (BM == 64 || lane < BM)) kwpre = kw_wave[m0 + lane];
     stager.issue(lds_raw + buf * kBufBytes, m0, Lq);
@@ -187,6 +205,19 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasT
   auto stat_value = [&]() -> float {
     if (tid < BM) return (statpre == -INFINITY) ? INFINITY : statpre * kLog2e;
     return -statpre;
+  };
+  auto own_dk = [&]() -> float {  // -Dk of row tid / 4, in every thread of its quad; the dQ kernel's order of summation
+    float part[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+      const vec8 dv = bitcast<vec8>(dopre[i]), ov = bitcast<vec8>(opre[i]);
+      part[i] = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) part[i] = __builtin_fmaf((float)dv[e], (float)ov[e], part[i]);
+      part[i] += __uint_as_float(quad_perm<kQuadXor1>(__float_as_uint(part[i])));
+      part[i] += __uint_as_float(quad_perm<kQuadXor2>(__float_as_uint(part[i])));
+    }
+    return -((part[0] + part[1]) * p.p_keep);
   };
 
   // Sparse: the tiles are not slices of the query side but packed lists of the 16-row blocks that attend this key block
@@ -298,7 +329,13 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasT
     wait_vmem();  // this thread's share of the tile has arrived (LDS) / is in statpre
     float* const lse_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffStat + buf * Cfg::kStatBytes);
     float* const dk_l = lse_l + BM;
-    if (tid < 2 * BM) lse_l[tid] = stat_value();
+    if constexpr (kOwnD) {
+      if (tid < BM) lse_l[tid] = stat_value();
+      const float nd = own_dk();
+      if ((tid & 3) == 0) dk_l[tid >> 2] = nd;
+    } else {
+      if (tid < 2 * BM) lse_l[tid] = stat_value();
+    }
     const uint32_t kwcur = kwpre;
     __syncthreads();  // the tile is complete, and nobody still reads the other buffer
     if (kSparse) {
@@ -509,6 +546,13 @@ __global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasT
     }
     __builtin_amdgcn_wave_barrier();
   }
+}
+
+template <typename T, int D, bool kCausal, int kDrop, bool kSparse, int kBias = 0, bool kRot = false>
+__global__ void __launch_bounds__(256, (kDrop == 0 && D <= 64 && kBias != kBiasTensor) ? 3 : ((D == 128 && kBias == kBiasTensor) ? 1 : BwdCfg<T, D, kDrop == 1>::kMinBlocks)) fa_bwd_dkdv_kernel(const BwdParams p) {
+  using Cfg = BwdCfg<T, D, kDrop == 1>;
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes + (kBias == kBiasTensor ? 4 * Cfg::kBiasTileBytes : 0)];
+  fa_bwd_dkdv_body<T, D, kCausal, kDrop, kSparse, kBias, kRot>(p, blockIdx.x, lds_raw);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -776,11 +820,13 @@ struct DqCfg {
   static constexpr int kLdsBytes0 = kTileBytes > kEpiBytes ? kTileBytes : kEpiBytes;
   static constexpr int kLdsBytes = kLdsBytes0 > kMergeBytes ? kLdsBytes0 : kMergeBytes;
   static constexpr int CH = D / 8;
+  static constexpr int kBiasWaveBytes = 32 * (BN * 2 + 8);  // per wave, behind the tiles: the bias-tensor variants' rows
 };
 
 // kDrop: as in fa_bwd_dkdv_kernel
+// (the kernel proper is fa_bwd_dq_kernel below: `block` is its workgroup id, `lds_raw` its LDS)
 template <typename T, int D, int BN, bool kCausal, int kDrop, bool kSparse, int kBias = 0, int KS = 1>
-__global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasTensor) ? 3 : 2) fa_bwd_dq_kernel(const BwdParams p) {
+FA_DEVICE void fa_bwd_dq_body(const BwdParams& p, const int block, unsigned char* const lds_raw) {
   constexpr bool kDropout = kDrop == 1, kStored = kDrop == 2;
   constexpr bool kAlibi = kBias == kBiasAlibi, kTensorBias = kBias == kBiasTensor;
   static_assert(kBias == 0 || !kSparse, "score bias: dense variants only");
@@ -794,11 +840,11 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
 
   // kTensorBias: behind the tiles, per wave 32 rows x BN keys of bias, rows padded by 8 bytes (as in fa_fwd_kernel)
   constexpr int kBiasRowBytes = BN * 2 + 8, kBiasWaveBytes = 32 * kBiasRowBytes;
-  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes + (kBias == kBiasTensor ? 4 * kBiasWaveBytes : 0)];
+  static_assert(kBiasWaveBytes == Cfg::kBiasWaveBytes, "LDS size of the kernel");
 
   int bh, rank;
   const int n_splits = p.n_splits > 1 ? p.n_splits : 1;  // key splits per query tile (see BwdParams)
-  if (!map_tile<kCausal>(blockIdx.x, p.nq_tiles * n_splits, p.B * p.H, &bh, &rank, p.tile_group)) return;
+  if (!map_tile<kCausal>(block, p.nq_tiles * n_splits, p.B * p.H, &bh, &rank, p.tile_group)) return;
   const int split = rank % n_splits;
   rank /= n_splits;
   const int qt = kCausal ? p.nq_tiles - 1 - rank : rank;
@@ -965,16 +1011,22 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
   }
   // ---- now the fragments: rows past the end are zero; Dk and -Dk, lse in base-2 units (+inf switches a row off)
   {
-    float dsum = 0.f;
+    // (summed as the dK/dV kernel's own_dk sums it - eight elements in a chain, the chains pairwise - so that both give the same bits)
+    float dpart[D / 16];
 #pragma unroll
     for (int ks = 0; ks < D / 16; ks++) {
       const vec8 ov = bitcast<vec8>(oraw[ks]);
       qreg[ks] = bitcast<vec8>(qrow < Lq ? qraw[ks] : u32x4{0, 0, 0, 0});
       doreg[ks] = bitcast<vec8>(qrow < Lq ? doraw[ks] : u32x4{0, 0, 0, 0});
+      dpart[ks] = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; i++) dsum = __builtin_fmaf((float)doreg[ks][i], (float)ov[i], dsum);
+      for (int i = 0; i < 8; i++) dpart[ks] = __builtin_fmaf((float)doreg[ks][i], (float)ov[i], dpart[ks]);
     }
-    dsum = half_sum(dsum) * p.p_keep;  // lanes l and l^32 hold the two halves of each 16-element group of the row
+#pragma unroll
+    for (int step = 1; step < D / 16; step *= 2)
+#pragma unroll
+      for (int ks = 0; ks + step < D / 16; ks += 2 * step) dpart[ks] += dpart[ks + step];
+    float dsum = half_sum(dpart[0]) * p.p_keep;  // lanes l and l^32 hold the two halves of each 16-element group of the row
     if (qrow < Lq) {
       lse2 = (lse_raw == -INFINITY) ? INFINITY : lse_raw * kLog2e;
       dkv = dsum;
@@ -1165,6 +1217,37 @@ __global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasT
       u32x4 val = *reinterpret_cast<const u32x4*>(Os + row * OS + col);
       st_global16(gbase + (int64_t)orow * p.dq_rs + col, val);
     }
+  }
+}
+
+template <typename T, int D, int BN, bool kCausal, int kDrop, bool kSparse, int kBias = 0, int KS = 1>
+__global__ void __launch_bounds__(256, (D <= 64 && kDrop == 0 && kBias != kBiasTensor) ? 3 : 2) fa_bwd_dq_kernel(const BwdParams p) {
+  using Cfg = DqCfg<T, D, BN, KS>;
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[Cfg::kLdsBytes + (kBias == kBiasTensor ? 4 * Cfg::kBiasWaveBytes : 0)];
+  fa_bwd_dq_body<T, D, BN, kCausal, kDrop, kSparse, kBias, KS>(p, blockIdx.x, lds_raw);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Short launches: dQ and dK/dV in one launch
+// ---------------------------------------------------------------------------------------------------------------
+// A launch of a few hundred short workgroups spends a third of its time filling and draining the chip, and the backward
+// pays that twice.  Here the workgroups of the dK/dV kernel (ids below p.merged_dkdv_blocks; they form their own Dk, kOwnD) and
+// the half-size workgroups of the dQ kernel (the ids after them) make one grid: one fill, one drain, and the two kinds run
+// side by side.  Head dim 64, dense, no score bias; kDrop 0 or 2.
+template <typename T, bool kCausal, int kDrop>
+__global__ void __launch_bounds__(256, 2) fa_bwd_merged_kernel(const BwdParams p) {
+  constexpr int D = 64;
+  using CfgK = BwdCfg<T, D, kDrop == 1>;
+  using CfgQ = DqCfg<T, D, 64, 2>;
+  constexpr int kLds = CfgK::kLdsBytes > CfgQ::kLdsBytes ? CfgK::kLdsBytes : CfgQ::kLdsBytes;
+  __shared__ __attribute__((aligned(16))) unsigned char lds_raw[kLds];
+  const int block = blockIdx.x;
+  if (block < p.merged_dkdv_blocks) {
+    fa_bwd_dkdv_body<T, D, kCausal, kDrop, false, 0, false, true>(p, block, lds_raw);
+  } else {
+    BwdParams pq = p;
+    pq.nq_tiles = p.merged_nq_tiles;
+    fa_bwd_dq_body<T, D, 64, kCausal, kDrop, false, 0, 2>(pq, block - p.merged_dkdv_blocks, lds_raw);
   }
 }
 

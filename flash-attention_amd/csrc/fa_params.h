@@ -137,6 +137,7 @@ struct BwdParams {
   int sq_r;        // innermost extent of dsoftmax
   int lse_stride;  // innermost extent of lse
   int nk_tiles;      // key tiles of the dK/dV kernel
+  int merged_dkdv_blocks, merged_nq_tiles;  // fa_bwd_merged_kernel: its dK/dV workgroups come first; query tiles of the dQ part
   int nq_tiles;      // query tiles of the dQ kernel
   int tile_group;    // causal launches: (batch, head) pairs of an XCD in flight together (map_tile); 0 = all
   float scale;
@@ -283,6 +284,15 @@ inline bool small_launch(int kernel, int BH, int max_s, bool causal, bool dropou
   const int64_t wgs = (int64_t)BH * ((max_s + 127) / 128);  // x = wgs / 256 compute units
   if (kernel == kSmallLaunchFwd) return max_s > 128 && (wgs < 2 * 256 || (dropout && wgs < 3 * 256));
   return wgs >= 256 && wgs < 2 * 256 && (causal || dropout);
+}
+
+// Short backward launches run dQ and dK/dV as one grid (fa_bwd_merged_kernel): where the dQ kernel takes its half-size tiles
+// (small_launch), at head dim 64, dense, no score bias, no rotation, no key split, dropout off or read from the keep words.
+inline bool merged_backward_launch(int head_dim, int BH, int max_sq, bool causal, bool dropout, bool keep_words, bool sparse,
+                                   bool bias, bool rotary, int n_splits) {
+  if ((launch_policy() & 0x30) == 0x10) return false;  // (the two-kernel plan was asked for)
+  return head_dim == 64 && !sparse && !bias && !rotary && n_splits <= 1 && (!dropout || keep_words) &&
+         small_launch(kSmallLaunchDq, BH, max_sq, causal, dropout);
 }
 
 // Launchers (defined in fa_fwd.hip / fa_bwd.hip / fa_aux.hip).  Return hipError_t of the launch.

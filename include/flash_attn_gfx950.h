@@ -290,7 +290,9 @@ int fa_blocksparse_row_order(const uint8_t* layout, int32_t n_row_blocks, int32_
  * Tile shape (bits 0-1): 0 (default): short-sequence launches that would leave compute units idle with the full-size
  * tiles (128 query rows / 128 keys per workgroup) use the half-size variants where they exist (head_dim <= 64, no
  * blockmask, no alibi_slopes); 1: always full-size; 2: always half-size where they exist.
- * Backward plan (bits 4-5): 0 (default) and 0x10: two kernels (dQ with softmax_d, then dK/dV), no scratch; 0x20: one kernel
+ * Backward plan (bits 4-5): 0 (default): two kernels (dQ with softmax_d, then dK/dV), no scratch - as two launches, or, for
+ * short launches at head_dim 64 (where the dQ kernel takes its half-size tiles), as one launch that holds both kinds of
+ * workgroup, with bit-identical results; 0x10: always two launches; 0x20: one kernel
  * that also passes dQ from key tile to key tile through fp32 scratch, where it exists (head_dim 64, no blockmask, mask,
  * dropout or bias, max_seqlen_k <= 4096) and only if the caller brings the scratch fa_bwd_workspace_bytes() then asks for.
  * Bit 6 (0x40): at head_dim 128 without dropout, blockmask or bias the dK/dV kernel runs as wave pairs (one wave holds K and

@@ -92,11 +92,16 @@ def test_d64_bias_tensor_and_one_kernel_backward_variants():
         for drop, words in (("Lb1E", "Lb0E"), ("Lb1E", "Lb1E")):
             k = _pick(fwd, "fa_fwd_kernelIDF16_Li64E", causal + drop + "Lb0ELi2ELi1E" + words + "EEv")
             assert k["Occupancy"] >= 2 and k["VGPRs Spill"] == 0, ("forward, bias tensor, dropout", causal, words, k)
-        for drop, spill in (("Li0E", 0), ("Li2E", 4), ("Li1E", 12)):
+        for drop, spill in (("Li0E", 0), ("Li2E", 4), ("Li1E", 16)):
             k = _pick(bwd, "fa_bwd_dq_kernelIDF16_Li64E", causal + drop + "Lb0ELi2ELi1EEEv")
             assert k["Occupancy"] >= 2 and k["VGPRs Spill"] == 0, ("dq, bias tensor", causal, drop, k)
             k = _pick(bwd, "fa_bwd_dkdv_kernelIDF16_Li64E", causal + drop + "Lb0ELi2ELb0EEEv")
             assert k["Occupancy"] >= 2 and k["VGPRs Spill"] <= spill, ("dkdv, bias tensor", causal, drop, k)
+    # dQ and dK/dV in one launch (short launches): the register count of the dK/dV part, two waves per SIMD, nothing spilled
+    for dt in ("IDF16_", "IDF16b"):
+        for flags in ("Lb0ELi0E", "Lb0ELi2E", "Lb1ELi0E", "Lb1ELi2E"):
+            k = _pick(bwd, "fa_bwd_merged_kernel" + dt, flags + "EEv")
+            assert k["Occupancy"] >= 2 and k["VGPRs Spill"] == 0 and k["LDS Size"] <= 80 * 1024, ("merged backward", dt, flags, k)
     fused = _resources("fa_bwd_fused.hip")
     for dt in ("IDF16_", "IDF16b"):
         k = _pick(fused, "fa_bwd_fused_kernel%sLi64ELi0E" % dt)

@@ -1552,6 +1552,52 @@ def test_blocksparse_modules_layout_sources_and_padding():
 
 
 # ------------------------------------------------------------------------------------------------
+# short launches: dQ and dK/dV in one launch (fa_bwd_merged_kernel; the default where the dQ kernel takes half-size tiles)
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("lens,dtype,causal,p", [
+    ([405, 435, 303, 318, 325, 368, 319, 504], torch.float16, False, 0.1),   # the BERT batch
+    ([405, 435, 303, 318, 325, 368, 319, 504], torch.bfloat16, True, 0.0),
+    ([512] * 8, torch.float16, True, 0.1),
+    ([300, 1, 77, 512, 129], torch.bfloat16, False, 0.2),
+])
+def test_merged_backward_equals_the_two_kernel_backward(lens, dtype, causal, p):
+    """Shapes whose backward runs as one launch by default (12 heads: 256 to 511 full-size dQ workgroups, dropout or a causal
+    mask): dq, dk, dv and softmax_d are bit for bit those of the two-kernel plan (launch policy 0x10; the dK/dV part sums its
+    own Dk in the dQ kernel's order), with the forward's keep words and without dropout; parity with the oracle is what
+    test_config_bert_varlen_dropout and the sweeps check."""
+    from flash_attn import flash_attn_gfx950 as be
+    torch.manual_seed(len(lens))
+    H, D = 12, 64
+    total, max_s = sum(lens), max(lens)
+    cu = _cu(lens)
+    qkv = torch.randn(total, 3, H, D, device="cuda").to(dtype)
+    do = torch.randn(total, H, D, device="cuda").to(dtype)
+    q, k, v = qkv[:, 0], qkv[:, 1], qkv[:, 2]
+    g = torch.Generator(device="cuda")
+    g.manual_seed(3)
+    st = g.get_state()
+    kw = be.new_keep_words(q, cu, max_s, max_s, p)
+    o, lse = be.fwd(q, k, v, cu, cu, max_s, max_s, p, D ** -0.5, False, causal, False, g, keep_words=kw)
+    res = []
+    try:
+        for policy in (0, 0x10, 0):
+            be.set_launch_policy(policy)
+            g.set_state(st)
+            grads = torch.full_like(qkv, float("nan"))
+            out = be.bwd(do, q, k, v, o, lse, grads[:, 0], grads[:, 1], grads[:, 2], cu, cu, max_s, max_s, p, D ** -0.5, False,
+                         causal, g, keep_words=kw)
+            res.append((grads, out[3]))
+    finally:
+        be.set_launch_policy(0)
+    torch.cuda.synchronize()
+    assert torch.isfinite(res[0][0].float()).all()
+    for a, b in ((res[0], res[1]), (res[0], res[2])):
+        assert torch.equal(a[0], b[0])
+        for bi, L in enumerate(lens):
+            assert torch.equal(a[1][bi, :, :L], b[1][bi, :, :L])
+
+
+# ------------------------------------------------------------------------------------------------
 # head dim 128: the dK/dV kernel of wave pairs (launch policy 0x40)
 # ------------------------------------------------------------------------------------------------
 @pytest.fixture
