@@ -1559,6 +1559,8 @@ def test_blocksparse_modules_layout_sources_and_padding():
     ([405, 435, 303, 318, 325, 368, 319, 504], torch.bfloat16, True, 0.0),
     ([512] * 8, torch.float16, True, 0.1),
     ([300, 1, 77, 512, 129], torch.bfloat16, False, 0.2),
+    ([300, 0, 77, 512, 129, 200], torch.float16, False, 0.1),                # a batch entry without tokens
+    ([300, 0, 77, 512, 129, 200], torch.bfloat16, True, 0.0),
 ])
 def test_merged_backward_equals_the_two_kernel_backward(lens, dtype, causal, p):
     """Shapes whose backward runs as one launch by default (12 heads: 256 to 511 full-size dQ workgroups, dropout or a causal
