@@ -5,7 +5,7 @@
 //     sum over groups of eight of |union of the eight lists|  +  sum over pairs of |union of the two lists|,
 // and this file looks for an order that makes it small: a greedy grouping (a group starts with the fullest row block left
 // and takes, seven times, the row block that adds the fewest key blocks to the group's set), then a fixed number of
-// pairwise exchanges between random positions, each kept if the cost does not rise (2000 attempts per row block).  Deterministic (own generator, fixed seed).
+// pairwise exchanges between random positions, each kept if the cost does not rise (2000 attempts per row block, four million at most).  Deterministic (own generator, fixed seed).
 #include <cstdint>
 #include <cstring>
 #include <vector>
@@ -105,7 +105,7 @@ extern "C" int fa_blocksparse_row_order(const uint8_t* layout, int32_t n_row_blo
     s ^= s >> 12; s ^= s << 25; s ^= s >> 27;
     return (uint32_t)((s * 0x2545F4914F6CDD1Dull) >> 32);
   };
-  const int64_t rounds = (int64_t)2000 * nr;
+  const int64_t rounds = (int64_t)2000 * nr < 4000000 ? (int64_t)2000 * nr : 4000000;  // (a second or so at most)
   for (int64_t it = 0; it < rounds; it++) {
     const int i = (int)(((uint64_t)next() * (uint64_t)nr) >> 32), j = (int)(((uint64_t)next() * (uint64_t)nr) >> 32);
     if (i == j) continue;

@@ -282,7 +282,8 @@ int fa_rotary(const fa_rotary_args* args);
  * workgroup (eight consecutive entries) and wave (two).  layout: HOST array [n_row_blocks][n_col_blocks] of bytes, non-zero
  * = the 16 x 256 block is listed (the layout before convert_blockmask); order: HOST array of n_row_blocks int32, written:
  * a permutation of 0 .. n_row_blocks - 1, the identity if reordering would save less than 5 % of the staged key blocks.
- * Deterministic; a greedy grouping followed by 2000 * n_row_blocks exchange attempts (tens of milliseconds for 4096 tokens). */
+ * Deterministic; a greedy grouping followed by 2000 * n_row_blocks exchange attempts, four million at most (tens of
+ * milliseconds for 4096 tokens, about a second for 65536). */
 int fa_blocksparse_row_order(const uint8_t* layout, int32_t n_row_blocks, int32_t n_col_blocks, int32_t* order);
 
 /* Launch policy (process-wide state; no counterpart in the reference, whose launchers pick their tile by head size
