@@ -456,8 +456,9 @@ def main():
             fb = 3.5 * wl.fwd_flops / ((tt["fwd_ms"] + tt["bwd_ms"]) * 1e-3) / 1e12
             gbs = (wl.bytes_fwd + wl.bytes_bwd) / ((tt["fwd_ms"] + tt["bwd_ms"]) * 1e-3) / 1e9
             print("%-31s fwd %.4f ms  bwd %.4f ms  fwd+bwd %.1f TFLOP/s (%.2f %% of MFMA peak)  %.1f GB/s of algorithmic bytes "
-                  "(fwd %.1f MB, bwd %.1f MB)" % (name.strip(), tt["fwd_ms"], tt["bwd_ms"], fb, 100 * fb / MFMA_PEAK_TFLOPS, gbs,
-                                                   wl.bytes_fwd / 1e6, wl.bytes_bwd / 1e6), file=sys.stderr)
+                  "(fwd %.1f MB, bwd %.1f MB)  [step %.4f ms by the host clock over %d steps]"
+                  % (name.strip(), tt["fwd_ms"], tt["bwd_ms"], fb, 100 * fb / MFMA_PEAK_TFLOPS, gbs,
+                     wl.bytes_fwd / 1e6, wl.bytes_bwd / 1e6, tt["ms_per_step"], a.steps), file=sys.stderr)
             del wl
             torch.cuda.empty_cache()
         return
