@@ -594,6 +594,19 @@ def main():
         ms_sep, ms_in = graph_replay_ms(torch, step_separate), graph_replay_ms(torch, step_in_kernel)
         print("%-28s %9.4f ms with separate passes, %.4f ms inside the kernels (%.1f %% less)  [same shape, fwd + bwd, no "
               "dropout]" % ("rotary + attention step", ms_sep, ms_in, 100 * (1 - ms_in / ms_sep)), file=sys.stderr)
+        # gradient of a bias shared over the batch: the per-(batch, head) slices the dK/dV kernel wrote, summed in one pass
+        # (fp32 sums, one rounding) against the same sum with torch ops (a float copy, a sum, a cast)
+        del qkv_r, packed, do_r, dqkv_r, rot_r
+        torch.cuda.empty_cache()
+        Bb, Hb, Nb = 8, 12, 2048
+        db = torch.randn(Bb, Hb, Nb, Nb, device="cuda", dtype=torch.float16)
+        red = torch.empty(1, Hb, Nb, Nb, device="cuda", dtype=torch.float16)
+        ms_lib = graph_replay_ms(torch, lambda: be.reduce_bias_grad(db, red, True, False), calls=5)
+        ms_torch = graph_replay_ms(torch, lambda: db.float().sum(0, keepdim=True).to(torch.float16), calls=5)
+        nbytes = (Bb + 1) * Hb * Nb * Nb * 2
+        print("%-28s %9.4f ms  %8.1f GB/s of %d (%.1f %% of HBM peak); with torch ops %.4f ms  [B=%d H=%d N=%d fp16 -> (1, H, "
+              "N, N)]" % ("bias gradient over batch", ms_lib, nbytes / ms_lib / 1e6, HBM_PEAK_GBS,
+                          100 * nbytes / ms_lib / 1e6 / HBM_PEAK_GBS, ms_torch, Bb, Hb, Nb), file=sys.stderr)
     print(json.dumps(res))
 
 

@@ -600,6 +600,29 @@ int fa_scatter_rows(const void* src, void* dst, const int64_t* indices, int64_t 
   return FA_OK;
 }
 
+int fa_bias_grad_reduce(const void* dbias, void* out, int32_t dtype, int32_t batch, int32_t heads, int32_t rows,
+                        int32_t cols, int64_t dbias_batch_stride, int64_t dbias_head_stride, int64_t dbias_row_stride,
+                        int32_t sum_batch, int32_t sum_heads, int64_t out_batch_stride, int64_t out_head_stride,
+                        int64_t out_row_stride, void* stream) {
+  FA_REQUIRE(dtype == 0 || dtype == 1, "fa_bias_grad_reduce: dtype must be 0 (fp16) or 1 (bf16)");
+  FA_REQUIRE(batch >= 0 && heads >= 0 && rows >= 0 && cols >= 0, "fa_bias_grad_reduce: negative size");
+  FA_REQUIRE(batch <= 65535 && heads <= 65535, "fa_bias_grad_reduce: more than 65535 batch entries or heads");
+  if (batch == 0 || heads == 0 || rows == 0 || cols == 0) return FA_OK;
+  FA_REQUIRE(dbias && out, "fa_bias_grad_reduce: null pointer");
+  const int64_t cols8 = ((int64_t)cols + 7) / 8 * 8;
+  FA_REQUIRE((reinterpret_cast<uintptr_t>(dbias) & 15) == 0 && dbias_batch_stride % 8 == 0 && dbias_head_stride % 8 == 0 &&
+                 dbias_row_stride % 8 == 0 && dbias_row_stride >= cols8,
+             "fa_bias_grad_reduce: dbias must be 16-byte aligned, its strides multiples of 8 and its rows padded to a "
+             "multiple of 8 columns");
+  FA_REQUIRE(out_row_stride >= cols, "fa_bias_grad_reduce: out row stride smaller than a row");
+  const bool vec_store = (reinterpret_cast<uintptr_t>(out) & 15) == 0 && out_batch_stride % 8 == 0 &&
+                         out_head_stride % 8 == 0 && out_row_stride % 8 == 0;
+  FA_LAUNCH(fa::launch_bias_grad_reduce(dbias, out, dtype, batch, heads, rows, cols, dbias_batch_stride, dbias_head_stride,
+                                        dbias_row_stride, sum_batch != 0, sum_heads != 0, out_batch_stride, out_head_stride,
+                                        out_row_stride, vec_store, reinterpret_cast<hipStream_t>(stream)));
+  return FA_OK;
+}
+
 int fa_rotary(const fa_rotary_args* a) {
   FA_REQUIRE(a && a->struct_bytes == sizeof(fa_rotary_args), "fa_rotary: struct size mismatch");
   FA_REQUIRE(a->dtype == FA_FP16 || a->dtype == FA_BF16, "fa_rotary: dtype must be fp16 or bf16");

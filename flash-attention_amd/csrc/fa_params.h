@@ -323,6 +323,9 @@ hipError_t launch_gather_rows(const void* src, void* dst, const int64_t* idx, in
 hipError_t launch_scatter_rows(const void* src, void* dst, const int64_t* idx, int64_t n_idx, int64_t n_dst,
                                int64_t row_bytes, int64_t src_stride, int64_t dst_stride, int vec, int32_t* inv,
                                hipStream_t stream);
+hipError_t launch_bias_grad_reduce(const void* in, void* out, int dtype, int nb, int nh, int rows, int cols, int64_t in_bs,
+                                   int64_t in_hs, int64_t in_rs, int sum_batch, int sum_heads, int64_t out_bs, int64_t out_hs,
+                                   int64_t out_rs, bool vec_store, hipStream_t stream);
 hipError_t launch_dump_probs(const DumpParams& p, int dtype, hipStream_t stream);
 // which: 0 = dQ kernel, 1 = dK/dV kernel
 hipError_t launch_bwd(const BwdParams& p, int which, int dtype, int head_dim, bool causal, bool dropout, bool sparse,

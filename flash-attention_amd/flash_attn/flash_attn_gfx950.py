@@ -120,7 +120,7 @@ EXPORTED_SYMBOLS = (
     "fa_fwd", "fa_bwd", "fa_fwd_block", "fa_bwd_block", "fa_fwd_block_noalloc", "fa_fwd_workspace_bytes", "fa_bwd_workspace_bytes",
     "fa_round_seqlens", "fa_philox_offset_increment", "fa_last_error", "fa_abi_version",
     "fa_gather_rows", "fa_scatter_rows", "fa_scatter_rows_workspace_bytes", "fa_rotary", "fa_set_launch_policy",
-    "fa_keep_words_bytes", "fa_blocksparse_row_order",
+    "fa_keep_words_bytes", "fa_blocksparse_row_order", "fa_bias_grad_reduce",
 )
 # declared in include/flash_attn_gfx950_bench.h: instrumentation for bench.py, not part of the drop-in boundary
 BENCH_SYMBOLS = ("fa_bwd_profiled",)
@@ -171,6 +171,9 @@ def load_library():
         lib.fa_scatter_rows.argtypes = ([ctypes.c_void_p] * 3 + [ctypes.c_int64] * 5 +
                                         [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p])
         lib.fa_scatter_rows.restype = ctypes.c_int
+        lib.fa_bias_grad_reduce.argtypes = ([ctypes.c_void_p] * 2 + [ctypes.c_int32] * 5 + [ctypes.c_int64] * 3 +
+                                            [ctypes.c_int32] * 2 + [ctypes.c_int64] * 3 + [ctypes.c_void_p])
+        lib.fa_bias_grad_reduce.restype = ctypes.c_int
         lib.fa_scatter_rows_workspace_bytes.argtypes = [ctypes.c_int64]
         lib.fa_scatter_rows_workspace_bytes.restype = ctypes.c_size_t
         lib.fa_rotary.argtypes = [ctypes.POINTER(RotaryArgs)]
@@ -664,6 +667,27 @@ def gather_rows(input, indices):
         rc = lib.fa_gather_rows(input.data_ptr(), out.data_ptr(), idx.data_ptr(), idx.numel(), input.shape[0],
                                 input.shape[1] * es, input.stride(0) * es, out.stride(0) * es,
                                 _stream_handle(input.device))
+    if rc != 0:
+        _raise(rc, lib)
+    return out
+
+
+def reduce_bias_grad(dbias, out, sum_batch, sum_heads):
+    """out[...] = sum of the per-(batch, head) bias gradient `dbias` (batch, nheads, rows, cols padded to 8) over the
+    batch entries (sum_batch) and / or heads (sum_heads), added in fp32 and rounded once, by fa_bias_grad_reduce.
+    out: a (1 or batch, 1 or nheads, rows, cols) view in dbias's dtype, cols <= dbias.shape[3], innermost stride 1."""
+    _check(dbias.dim() == 4 and out.dim() == 4 and dbias.is_cuda and out.device == dbias.device and out.dtype == dbias.dtype,
+           "dbias and out must be 4-D tensors of one dtype on one GPU")
+    batch, nheads, rows, _ = dbias.shape
+    _check(tuple(out.shape[:3]) == (1 if sum_batch else batch, 1 if sum_heads else nheads, rows) and
+           out.shape[3] <= dbias.shape[3] and dbias.stride(3) == 1 and (out.stride(3) == 1 or out.shape[3] <= 1),
+           "out must be (1 or batch, 1 or nheads, rows, cols <= dbias's) with contiguous keys")
+    lib = load_library()
+    with _OnDevice(dbias.device):
+        rc = lib.fa_bias_grad_reduce(dbias.data_ptr(), out.data_ptr(), _dtype_code(dbias), batch, nheads, rows, out.shape[3],
+                                     dbias.stride(0), dbias.stride(1), dbias.stride(2), int(bool(sum_batch)),
+                                     int(bool(sum_heads)), out.stride(0), out.stride(1), out.stride(2),
+                                     _stream_handle(dbias.device))
     if rc != 0:
         _raise(rc, lib)
     return out

@@ -129,14 +129,14 @@ def _backward(ctx, dout):
         torch.cuda.set_rng_state(cur_rng_state, dev)
     ctx.dbias = None
     if dbias is not None:  # back to the shape the caller's bias has: summed over the batch entries / heads that shared it
-        g = dbias[:, :, :, :ctx.max_seqlen_k]
         shp = ctx.bias_shape
-        if shp[0] == 1 and g.shape[0] > 1:
-            g = g.float().sum(0, keepdim=True)
-        if shp[1] == 1 and g.shape[1] > 1:
-            g = g.float().sum(1, keepdim=True)
         full = torch.zeros(shp, dtype=q.dtype, device=dev)  # rows / keys beyond max_seqlen get no gradient
-        full[:, :, :ctx.max_seqlen_q, :ctx.max_seqlen_k] = g.to(q.dtype)
+        view = full[:, :, :ctx.max_seqlen_q, :ctx.max_seqlen_k]
+        sum_batch, sum_heads = shp[0] == 1 and dbias.shape[0] > 1, shp[1] == 1 and dbias.shape[1] > 1
+        if sum_batch or sum_heads:  # one pass, fp32 sums, one rounding
+            _backend.reduce_bias_grad(dbias, view, sum_batch, sum_heads)
+        else:
+            view.copy_(dbias[:, :, :, :ctx.max_seqlen_k])
         ctx.dbias = full
     return grads
 

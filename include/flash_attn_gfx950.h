@@ -249,6 +249,18 @@ int fa_scatter_rows(const void* src, void* dst, const int64_t* indices, int64_t 
                     size_t workspace_bytes, void* stream);
 size_t fa_scatter_rows_workspace_bytes(int64_t n_dst_rows);
 
+/* Sum of the bias gradient over the batch entries and / or heads that shared one bias (no counterpart in the
+ * reference, which takes no bias).  fa_bwd writes `dbias` per (batch, head); a bias of batch or head extent 1 that
+ * was broadcast wants the sum.  dbias: [batch, heads, rows, >= cols rounded up to 8] in `dtype` (strides in elements,
+ * multiples of 8, base 16-byte aligned: the rows are read as whole 16-byte chunks).  out: [sum_batch ? 1 : batch,
+ * sum_heads ? 1 : heads, rows, cols] in the same dtype, any strides with innermost stride 1.  One pass; the slices are
+ * added in fp32 in a fixed order (batch outer, head inner) and rounded once, so the result is reproducible bit for
+ * bit. */
+int fa_bias_grad_reduce(const void* dbias, void* out, int32_t dtype, int32_t batch, int32_t heads, int32_t rows,
+                        int32_t cols, int64_t dbias_batch_stride, int64_t dbias_head_stride, int64_t dbias_row_stride,
+                        int32_t sum_batch, int32_t sum_heads, int64_t out_batch_stride, int64_t out_head_stride,
+                        int64_t out_row_stride, void* stream);
+
 /* Rotary position embedding of the query and key parts of a packed tensor in one pass: what
  * RotaryEmbedding.forward / apply_rotary_pos_emb compute with elementwise torch ops (flash_attn/rotary.py:22-42,
  * 89-100; FlashMHA applies it to q and k before attention, flash_attention.py:109-113).

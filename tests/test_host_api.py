@@ -494,6 +494,21 @@ def test_rows_and_rotary_argument_checks(lib):
     assert lib.fa_rotary(ctypes.byref(r)) == 0
 
 
+def test_bias_grad_reduce_argument_checks(lib):
+    """fa_bias_grad_reduce rejects bad arguments before any launch (CPU only: nothing valid is executed)"""
+    ok_in = (2, 3, 16, 20, 3 * 16 * 24, 16 * 24, 24)   # batch, heads, rows, cols, dbias strides (rows padded to 24 columns)
+    ok_out = (1, 0, 3 * 16 * 20, 16 * 20, 20)          # sum_batch, sum_heads, out strides
+    call = lambda dbias, out, dtype, i, o: lib.fa_bias_grad_reduce(dbias, out, dtype, *i, *o, None)
+    assert call(0x1000, 0x2000, 2, ok_in, ok_out) == -1 and b"dtype" in lib.fa_last_error()
+    assert call(None, 0x2000, 0, ok_in, ok_out) == -1 and b"null" in lib.fa_last_error()
+    assert call(0x1008, 0x2000, 0, ok_in, ok_out) == -1 and b"aligned" in lib.fa_last_error()            # 8-byte aligned only
+    assert call(0x1000, 0x2000, 0, (2, 3, 16, 20, 3 * 16 * 20, 16 * 20, 20), ok_out) == -1               # rows not padded to 8
+    assert call(0x1000, 0x2000, 0, ok_in, (1, 0, 3 * 16 * 20, 16 * 20, 19)) == -1 and b"out row" in lib.fa_last_error()
+    assert call(0x1000, 0x2000, 0, (70000, 3, 16, 20, 3 * 16 * 24, 16 * 24, 24), ok_out) == -1
+    assert call(None, None, 1, (0, 3, 16, 20, 0, 0, 24), ok_out) == 0                                    # nothing to do
+    assert call(None, None, 1, (2, 3, 16, 0, 0, 0, 0), ok_out) == 0
+
+
 def test_header_is_plain_c(tmp_path):
     """include/flash_attn_gfx950.h must be usable from C (the boundary a cgo / JNI / ctypes binding sees): it compiles as
     C99 with warnings as errors, and every declared entry point can be named."""

@@ -850,6 +850,39 @@ def test_attn_bias_random_shapes_sweep():
             assert (S[b, :, :Lq, :Lk] - ref["probs"][b]).abs().max() < (2e-3 if dtype == torch.float16 else 1.6e-2)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_bias_grad_reduce_sums_in_fp32_and_rounds_once(dtype):
+    """fa_bias_grad_reduce against float64 sums of the same slices: over the batch, over the heads, over both; key extents
+    that are and are not multiples of 8, an output whose rows are not 16-byte aligned (scalar stores), a view into a larger
+    tensor whose surroundings must stay untouched.  The fp32 running sum and the one rounding bound the error; two calls
+    give the same bits."""
+    from flash_attn import flash_attn_gfx950 as be
+    g = torch.Generator(device="cuda").manual_seed(5)
+    eps = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
+    for B, H, rows, cols, out_cols in ((5, 3, 37, 64, 64), (2, 4, 16, 45, 53), (9, 1, 130, 200, 200), (1, 6, 8, 7, 7)):
+        cols8 = (cols + 7) // 8 * 8
+        dbias = (torch.randn(B, H, rows, cols8, device="cuda", generator=g) * 3).to(dtype)
+        for sum_batch, sum_heads in ((True, False), (False, True), (True, True)):
+            ob, oh = (1 if sum_batch else B), (1 if sum_heads else H)
+            full = torch.full((ob, oh, rows + 3, out_cols + 2), 7.0, device="cuda", dtype=dtype)
+            view = full[:, :, :rows, :cols]
+            be.reduce_bias_grad(dbias, view, sum_batch, sum_heads)
+            ref = dbias[..., :cols].double()
+            mag = dbias[..., :cols].double().abs()
+            if sum_batch:
+                ref, mag = ref.sum(0, keepdim=True), mag.sum(0, keepdim=True)
+            if sum_heads:
+                ref, mag = ref.sum(1, keepdim=True), mag.sum(1, keepdim=True)
+            err = (view.double() - ref).abs()
+            assert bool((err <= eps * ref.abs() * 1.001 + 2.0 ** -22 * mag).all()), (B, H, rows, cols, sum_batch, sum_heads)
+            assert bool((full[:, :, rows:] == 7).all()) and bool((full[:, :, :, cols:] == 7).all())
+            again = torch.empty_like(full)[:, :, :rows, :cols]
+            be.reduce_bias_grad(dbias, again, sum_batch, sum_heads)
+            assert torch.equal(again, view)
+    with pytest.raises(RuntimeError):
+        be.reduce_bias_grad(dbias, torch.empty(2, 6, 8, 7, device="cuda", dtype=dtype), True, False)  # wrong batch extent
+
+
 @pytest.mark.parametrize("D,dtype,causal", [(64, torch.float16, False), (128, torch.bfloat16, True), (32, torch.float16, True)])
 def test_attn_bias_with_dropout(D, dtype, causal, dropout_path):
     """bias and dropout together (the backward reading the forward's keep words, or drawing again): the mask is the defined
