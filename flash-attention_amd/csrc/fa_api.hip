@@ -191,8 +191,6 @@ int fwd_impl(const fa_fwd_args* a, bool want_block) {
   FA_REQUIRE(out_stride_ok(a->o_row_stride, a->head_dim) && out_stride_ok(a->o_head_stride, a->head_dim),
              "row and head strides of o must be at least head_dim (the output's rows and heads may not overlap)");
 
-  if (sparse && (a->alibi_slopes || a->attn_bias))
-    return fail(FA_ERR_UNSUPPORTED, "alibi_slopes and attn_bias are not supported together with a blockmask");
   if (a->alibi_slopes && a->attn_bias) return fail(FA_ERR_UNSUPPORTED, "alibi_slopes and attn_bias are not supported together");
 
   const Rounded r = round_seqlens(a->head_dim, a->max_seqlen_q, a->max_seqlen_k, sparse);
@@ -327,8 +325,6 @@ int bwd_impl(const fa_bwd_args* a, bool want_block, void* ev_main_start = nullpt
   if (rc) return rc;
   const bool sparse = a->blockmask != nullptr;
   FA_REQUIRE(sparse == want_block, want_block ? "fa_bwd_block needs a blockmask" : "fa_bwd takes no blockmask; call fa_bwd_block");
-  if (sparse && (a->alibi_slopes || a->attn_bias))
-    return fail(FA_ERR_UNSUPPORTED, "alibi_slopes and attn_bias are not supported together with a blockmask");
   if (a->alibi_slopes && a->attn_bias) return fail(FA_ERR_UNSUPPORTED, "alibi_slopes and attn_bias are not supported together");
   FA_REQUIRE(a->dout && a->q && a->k && a->v && a->out && a->softmax_lse && a->dq && a->dk && a->dv && a->softmax_d &&
                  a->cu_seqlens_q && a->cu_seqlens_k, "NULL tensor pointer");

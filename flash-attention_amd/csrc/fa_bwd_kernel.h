@@ -79,7 +79,6 @@ FA_DEVICE void fa_bwd_dkdv_body(const BwdParams& p, const int block, unsigned ch
   constexpr bool kDropout = kDrop == 1, kStored = kDrop == 2;
   constexpr bool kAlibi = kBias == kBiasAlibi, kTensorBias = kBias == kBiasTensor;
   static_assert(!(kStored && kSparse), "keep words: dense only");
-  static_assert(kBias == 0 || !kSparse, "score bias: dense variants only");
   using Cfg = BwdCfg<T, D, kDropout>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
@@ -290,10 +289,13 @@ FA_DEVICE void fa_bwd_dkdv_body(const BwdParams& p, const int block, unsigned ch
   T* const bias_lds = reinterpret_cast<T*>(lds_raw + Cfg::kLdsBytes + wave * kBiasTileBytes);
   constexpr int kBiasNLD = BM * 4 / 64;  // 16-byte loads per lane and tile
   u32x4 bpre[kTensorBias ? kBiasNLD : 1];
-  auto load_bias = [&](int q_first) {
+  // (q_first: the tile's first query row; sparse: the packed tile's list of 16-row blocks instead, -1 = no block)
+  auto load_bias = [&](int q_first, const int* rb) {
 #pragma unroll
     for (int i = 0; i < kBiasNLD; i++) {
-      const int qr = q_first + i * 16 + (lane >> 2), k0 = n0 + wave * 32 + (lane & 3) * 8;
+      const int k0 = n0 + wave * 32 + (lane & 3) * 8;
+      int qr = q_first + i * 16 + (lane >> 2);
+      if (kSparse) qr = rb[i] >= 0 ? rb[i] * 16 + (lane >> 2) : Lq;
       bpre[i] = u32x4{0, 0, 0, 0};  // chunks that begin past the last key are not read; rows past the end read the last row
       if (k0 < Lk) bpre[i] = ld_global16(bias_bh + (uint32_t)(qr < Lq ? qr : Lq - 1) * bias_rs + (uint32_t)k0);
     }
@@ -323,7 +325,7 @@ FA_DEVICE void fa_bwd_dkdv_body(const BwdParams& p, const int block, unsigned ch
     else stage(mt, 0);
   }
   finish_kv();
-  if (kTensorBias && more) load_bias(mt * BM);
+  if (kTensorBias && more) load_bias(mt * BM, tc.rb);
   while (more) {
     const int m0 = mt * BM;
     wait_vmem();  // this thread's share of the tile has arrived (LDS) / is in statpre
@@ -347,7 +349,7 @@ FA_DEVICE void fa_bwd_dkdv_body(const BwdParams& p, const int block, unsigned ch
     }
     if (kTensorBias) {  // (the wave's own reads of the last tile's values are behind it: LDS operations of a wave stay in order)
       bias_to_lds();
-      if (more) load_bias((mt + 1) * BM);
+      if (more) load_bias((mt + 1) * BM, tn.rb);
     }
     const T* const Ql = reinterpret_cast<const T*>(lds_raw + buf * kBufBytes);
     const T* const dOl = Ql + BM * D;
@@ -438,7 +440,9 @@ FA_DEVICE void fa_bwd_dkdv_body(const BwdParams& p, const int block, unsigned ch
           km[r] = ((uint64_t)hi << 32) | lo;
         }
       }
-      const float dbase = (float)(key - m0 - qb * 32 - 4 * hf);  // key - query of register 0 (kAlibi; dense only)
+      // kAlibi: key - query of register 0, and (sparse: the slab's second row block is any later one) of register 8 plus 16
+      const float dbase = kSparse ? (float)(key - q_lo - 4 * hf) : (float)(key - m0 - qb * 32 - 4 * hf);
+      const float dbase_hi = kSparse ? (float)(key - q_hi + 16 - 4 * hf) : dbase;
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const f32x4 lse4 = *reinterpret_cast<const f32x4*>(lse_l + qb * 32 + 8 * j + 4 * hf);
@@ -448,7 +452,7 @@ FA_DEVICE void fa_bwd_dkdv_body(const BwdParams& p, const int block, unsigned ch
         for (int i = 0; i < 4; i++) {
           const int r = 4 * j + i;
           float e = -lse4[i];
-          if (kAlibi) e = __builtin_fmaf(__builtin_fabsf(dbase - (float)(8 * j + i)), -sl2, -lse4[i]);
+          if (kAlibi) e = __builtin_fmaf(__builtin_fabsf((j < 2 ? dbase : dbase_hi) - (float)(8 * j + i)), -sl2, -lse4[i]);
           if (kTensorBias) e = __builtin_fmaf((float)braw[r], kLog2e, -lse4[i]);
           const float pe = fast_exp2(__builtin_fmaf(s[r], cs, e));
           float dpe = dp[r];  // dP - Dk
@@ -460,10 +464,10 @@ FA_DEVICE void fa_bwd_dkdv_body(const BwdParams& p, const int block, unsigned ch
         }
       }
       if (kTensorBias && dbias_bh != nullptr && key < Lk) {  // d(loss)/d(bias) = dS = dS' / keep
-        const uint32_t q0 = (uint32_t)(q_lo + 4 * hf);
+        const uint32_t q0 = (uint32_t)(q_lo + 4 * hf), q8 = (uint32_t)(q_hi - 16 + 4 * hf);  // (dense: q8 == q0)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          const uint32_t qr = q0 + 8 * (r >> 2) + (r & 3);
+          const uint32_t qr = (kSparse && r >= 8 ? q8 : q0) + 8 * (r >> 2) + (r & 3);
           if (qr < (uint32_t)Lq) dbias_bh[qr * dbias_rs + (uint32_t)key] = (T)(dp[r] * p.rp_keep);
         }
       }
@@ -829,7 +833,6 @@ template <typename T, int D, int BN, bool kCausal, int kDrop, bool kSparse, int 
 FA_DEVICE void fa_bwd_dq_body(const BwdParams& p, const int block, unsigned char* const lds_raw) {
   constexpr bool kDropout = kDrop == 1, kStored = kDrop == 2;
   constexpr bool kAlibi = kBias == kBiasAlibi, kTensorBias = kBias == kBiasTensor;
-  static_assert(kBias == 0 || !kSparse, "score bias: dense variants only");
   static_assert(!(kStored && kSparse), "keep words: dense only");
   constexpr bool kRotCapable = !kSparse && kBias == 0;  // rotary (p.rot_cos): dense variants without score bias
   using Cfg = DqCfg<T, D, BN, KS>;
@@ -979,7 +982,12 @@ FA_DEVICE void fa_bwd_dq_body(const BwdParams& p, const int block, unsigned char
   auto load_bias = [&](int tile) {
 #pragma unroll
     for (int i = 0; i < kBiasNLD; i++) {
-      const int row = mw + i * kBiasRPI + lane / kBiasCPR, k0 = tile * BN + (lane % kBiasCPR) * 8;
+      const int lr = i * kBiasRPI + lane / kBiasCPR, k0 = tile * BN + (lane % kBiasCPR) * 8;
+      int row = mw + lr;
+      if (kSparse) {  // the slab's two row blocks (rows of no block read the last row: their results are never stored)
+        const int rbl = lr < 16 ? rb_a : rb_b;
+        row = rbl >= 0 ? rbl * 16 + (lr & 15) : Lq;
+      }
       braw[i] = u32x4{0, 0, 0, 0};
       if (k0 < Lk) braw[i] = ld_global16(bias_bh + (uint32_t)(row < Lq ? row : Lq - 1) * (uint32_t)p.bias_rs + (uint32_t)k0);
     }

@@ -54,7 +54,6 @@ template <typename T, int D, int BN, bool kCausal, bool kDropout, bool kSparse, 
 __global__ void __launch_bounds__(256, ((!kDropout || KS == 2) && kBias == 0 && D <= 64) ? 4 : ((!kDropout && kBias == kBiasTensor && D <= 64) ? 3 : 2)) fa_fwd_kernel(const FwdParams p) {
   constexpr bool kAlibi = kBias == kBiasAlibi, kTensorBias = kBias == kBiasTensor;
   static_assert(!kWords || (kDropout && !kSparse), "keep words: dense dropout variants only");
-  static_assert(kBias == 0 || !kSparse, "score bias: dense variants only");
   using Cfg = FwdCfg<T, D, BN, KS>;
   using E = Elem<T>;
   using vec8 = typename E::vec8;
@@ -186,7 +185,12 @@ __global__ void __launch_bounds__(256, ((!kDropout || KS == 2) && kBias == 0 && 
   auto load_bias = [&](int tile) {
 #pragma unroll
     for (int i = 0; i < kBiasNLD; i++) {
-      const int row = mw + i * kBiasRPI + lane / kBiasCPR, k0 = tile * BN + (lane % kBiasCPR) * 8;
+      const int lr = i * kBiasRPI + lane / kBiasCPR, k0 = tile * BN + (lane % kBiasCPR) * 8;
+      int row = mw + lr;
+      if (kSparse) {  // the slab's two row blocks (rows of no block read the last row: their results are never stored)
+        const int rbl = lr < 16 ? rb_a : rb_b;
+        row = rbl >= 0 ? rbl * 16 + (lr & 15) : Lq;
+      }
       braw[i] = u32x4{0, 0, 0, 0};
       if (k0 < Lk) braw[i] = ld_global16(bias_bh + (uint32_t)(row < Lq ? row : Lq - 1) * (uint32_t)p.bias_rs + (uint32_t)k0);
     }

@@ -316,7 +316,6 @@ def _check_alibi(alibi_slopes, nheads, device, sparse):
     """alibi_slopes: None or nheads fp32 slopes on the tensors' device (an extension: the reference has no attention bias)."""
     if alibi_slopes is None:
         return None
-    _check(not sparse, "alibi_slopes are not supported together with a blockmask")
     _check(alibi_slopes.device == device and alibi_slopes.dtype == torch.float32 and alibi_slopes.is_contiguous() and
            tuple(alibi_slopes.shape) == (nheads,), "alibi_slopes must be a contiguous fp32 tensor of nheads slopes on the GPU")
     return alibi_slopes.data_ptr()
@@ -344,7 +343,6 @@ def _bias_arg(a, attn_bias, q, batch, nheads, max_seqlen_q, max_seqlen_k, sparse
     """Fills the attn_bias fields of a FwdArgs / BwdArgs; returns the tensor they point into (to be kept alive)."""
     if attn_bias is None:
         return None
-    _check(not sparse, "attn_bias is not supported together with a blockmask")
     t = prepare_attn_bias(attn_bias, q, batch, nheads, int(max_seqlen_q), int(max_seqlen_k))
     a.attn_bias = t.data_ptr()
     a.bias_batch_stride = 0 if t.shape[0] == 1 else t.stride(0)
@@ -626,20 +624,24 @@ def bwd(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
 
 
 def fwd_block(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout, softmax_scale,
-              is_causal, return_softmax, gen=None, row_order=None):
+              is_causal, return_softmax, gen=None, row_order=None, alibi_slopes=None, attn_bias=None):
     """mha_fwd_block (fmha_api.cpp:451-573).  row_order (extension): None, or the int32 order of the 16-row blocks from
-    blockmask_row_order() of the layout: the kernels' workgroups then own row blocks with similar key-block lists."""
+    blockmask_row_order() of the layout: the kernels' workgroups then own row blocks with similar key-block lists.
+    alibi_slopes, attn_bias (extensions): as in fwd."""
     _check(blockmask is not None, "blockmask is required")
     return _fwd_impl(q, k, v, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q, max_seqlen_k, p_dropout,
-                     softmax_scale, False, is_causal, return_softmax, gen, row_order=row_order)
+                     softmax_scale, False, is_causal, return_softmax, gen, alibi_slopes=alibi_slopes, attn_bias=attn_bias,
+                     row_order=row_order)
 
 
 def bwd_block(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q,
-              max_seqlen_k, p_dropout, softmax_scale, is_causal, gen=None, row_order=None):
-    """mha_bwd_block (fmha_api.cpp:575-718).  row_order: as in fwd_block."""
+              max_seqlen_k, p_dropout, softmax_scale, is_causal, gen=None, row_order=None, alibi_slopes=None,
+              attn_bias=None, dbias=None):
+    """mha_bwd_block (fmha_api.cpp:575-718).  row_order: as in fwd_block; alibi_slopes, attn_bias, dbias: as in bwd."""
     _check(blockmask is not None, "blockmask is required")
     return _bwd_impl(dout, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k, blockmask, max_seqlen_q,
-                     max_seqlen_k, p_dropout, softmax_scale, False, is_causal, gen, row_order=row_order)
+                     max_seqlen_k, p_dropout, softmax_scale, False, is_causal, gen, alibi_slopes=alibi_slopes,
+                     attn_bias=attn_bias, dbias=dbias, row_order=row_order)
 
 
 def _check_rows(name, t):

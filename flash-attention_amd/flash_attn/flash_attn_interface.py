@@ -115,10 +115,7 @@ def _backward(ctx, dout):
     grads = tuple(torch.empty_like(t) for t in tensors)
     dq, dk, dv = _split(ctx.packing, grads)
     dev = q.device
-    dbias = None
-    if ctx.bias_needs_grad:  # per (batch, head); only the tiles the kernels visit are written
-        dbias = torch.zeros((cu_seqlens_q.numel() - 1, q.shape[1], ctx.max_seqlen_q, (ctx.max_seqlen_k + 7) // 8 * 8),
-                            dtype=q.dtype, device=dev)
+    dbias = new_bias_grad(q, cu_seqlens_q.numel() - 1, ctx.max_seqlen_q, ctx.max_seqlen_k) if ctx.bias_needs_grad else None
     if rng_state is not None:
         cur_rng_state = torch.cuda.get_rng_state(dev)
         torch.cuda.set_rng_state(rng_state, dev)
@@ -127,18 +124,27 @@ def _backward(ctx, dout):
                          ctx.alibi_slopes, ctx.keep_words, bias_t, dbias, ctx.rotary)
     if rng_state is not None:
         torch.cuda.set_rng_state(cur_rng_state, dev)
-    ctx.dbias = None
-    if dbias is not None:  # back to the shape the caller's bias has: summed over the batch entries / heads that shared it
-        shp = ctx.bias_shape
-        full = torch.zeros(shp, dtype=q.dtype, device=dev)  # rows / keys beyond max_seqlen get no gradient
-        view = full[:, :, :ctx.max_seqlen_q, :ctx.max_seqlen_k]
-        sum_batch, sum_heads = shp[0] == 1 and dbias.shape[0] > 1, shp[1] == 1 and dbias.shape[1] > 1
-        if sum_batch or sum_heads:  # one pass, fp32 sums, one rounding
-            _backend.reduce_bias_grad(dbias, view, sum_batch, sum_heads)
-        else:
-            view.copy_(dbias[:, :, :, :ctx.max_seqlen_k])
-        ctx.dbias = full
+    ctx.dbias = bias_grad_in_shape(dbias, ctx.bias_shape, ctx.max_seqlen_q, ctx.max_seqlen_k) if dbias is not None else None
     return grads
+
+
+def new_bias_grad(q, batch, max_seqlen_q, max_seqlen_k):
+    """The tensor the backward kernels leave the bias gradient in: per (batch, head), rows padded to 8 keys, cleared (only
+    the tiles the kernels visit are written)."""
+    return torch.zeros((batch, q.shape[1], max_seqlen_q, (max_seqlen_k + 7) // 8 * 8), dtype=q.dtype, device=q.device)
+
+
+def bias_grad_in_shape(dbias, shape, max_seqlen_q, max_seqlen_k):
+    """The gradient of an attn_bias of `shape` from the per-(batch, head) tensor of new_bias_grad(): summed over the batch
+    entries / heads that shared the bias (one pass, fp32 sums, one rounding); rows / keys beyond max_seqlen get none."""
+    full = torch.zeros(shape, dtype=dbias.dtype, device=dbias.device)
+    view = full[:, :, :max_seqlen_q, :max_seqlen_k]
+    sum_batch, sum_heads = shape[0] == 1 and dbias.shape[0] > 1, shape[1] == 1 and dbias.shape[1] > 1
+    if sum_batch or sum_heads:
+        _backend.reduce_bias_grad(dbias, view, sum_batch, sum_heads)
+    else:
+        view.copy_(dbias[:, :, :, :max_seqlen_k])
+    return full
 
 
 def _extra_grads(ctx, grads):

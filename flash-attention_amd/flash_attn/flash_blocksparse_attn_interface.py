@@ -9,6 +9,7 @@ C++ argument order.
 import torch
 
 from . import flash_attn_gfx950 as _backend
+from .flash_attn_interface import bias_grad_in_shape, new_bias_grad
 
 
 def convert_blockmask(blockmask, causal):
@@ -62,82 +63,104 @@ def _row_order(blockmask, causal):
 
 
 def _flash_blocksparse_attn_forward(qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal,
-                                    return_softmax):
+                                    return_softmax, alibi_slopes=None, attn_bias=None):
     res = _backend.fwd_block(qkv[:, 0], qkv[:, 1], qkv[:, 2], cu_seqlens, cu_seqlens, blockmask, max_s, max_s,
-                             dropout_p, softmax_scale, causal, return_softmax, None, row_order=_row_order(blockmask, causal))
+                             dropout_p, softmax_scale, causal, return_softmax, None, row_order=_row_order(blockmask, causal),
+                             alibi_slopes=alibi_slopes, attn_bias=attn_bias)
     return res[0], res[1], (res[2] if return_softmax else None)
 
 
 def _flash_blocksparse_attn_backward(dout, qkv, out, S_dmask, softmax_lse, cu_seqlens, blockmask, dropout_p, max_s,
-                                     softmax_scale, causal):
+                                     softmax_scale, causal, alibi_slopes=None, attn_bias=None, dbias=None):
     dqkv = torch.empty_like(qkv)
     _backend.bwd_block(dout.contiguous(), qkv[:, 0], qkv[:, 1], qkv[:, 2], out, softmax_lse, dqkv[:, 0], dqkv[:, 1],
                        dqkv[:, 2], cu_seqlens, cu_seqlens, blockmask, max_s, max_s, dropout_p, softmax_scale, causal,
-                       None, row_order=_row_order(blockmask, causal))
+                       None, row_order=_row_order(blockmask, causal), alibi_slopes=alibi_slopes, attn_bias=attn_bias,
+                       dbias=dbias)
     return dqkv
 
 
-def _fwd_common(ctx, qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal, return_softmax):
+def _fwd_common(ctx, qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal, return_softmax, alibi_slopes,
+                attn_bias):
     rng_state = torch.cuda.get_rng_state(qkv.device) if dropout_p > 0 else None
     if softmax_scale is None:
         softmax_scale = qkv.shape[-1] ** (-0.5)
+    # the bias in the form the kernels read (the caller's tensor itself if its layout allows, else a padded copy)
+    bias_t = None
+    if attn_bias is not None:
+        bias_t = _backend.prepare_attn_bias(attn_bias.detach(), qkv[:, 0], cu_seqlens.numel() - 1, qkv.shape[2], int(max_s),
+                                            int(max_s))
     context, softmax_lse, S_dmask = _flash_blocksparse_attn_forward(
-        qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal, return_softmax)
-    ctx.save_for_backward(qkv, context, softmax_lse, cu_seqlens, blockmask, rng_state)
+        qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal, return_softmax, alibi_slopes, bias_t)
+    ctx.save_for_backward(qkv, context, softmax_lse, cu_seqlens, blockmask, rng_state, bias_t)
     ctx.dropout_p = dropout_p
     ctx.max_s = max_s
     ctx.softmax_scale = softmax_scale
     ctx.causal = causal
+    ctx.alibi_slopes = alibi_slopes  # fixed slopes, not differentiated
+    ctx.bias_shape = tuple(attn_bias.shape) if attn_bias is not None else None
+    ctx.bias_needs_grad = attn_bias is not None and attn_bias.requires_grad
     return context, S_dmask, softmax_lse
 
 
 def _bwd_common(ctx, dout):
-    qkv, context, softmax_lse, cu_seqlens, blockmask, rng_state = ctx.saved_tensors
+    """(dqkv, gradient of attn_bias or None)"""
+    qkv, context, softmax_lse, cu_seqlens, blockmask, rng_state, bias_t = ctx.saved_tensors
     dev = qkv.device
     if rng_state is not None:
         cur_rng_state = torch.cuda.get_rng_state(dev)
         torch.cuda.set_rng_state(rng_state, dev)
+    dbias = None
+    if ctx.bias_needs_grad:
+        dbias = new_bias_grad(qkv[:, 0], cu_seqlens.numel() - 1, ctx.max_s, ctx.max_s)
     dqkv = _flash_blocksparse_attn_backward(dout, qkv, context, None, softmax_lse, cu_seqlens, blockmask,
-                                            ctx.dropout_p, ctx.max_s, ctx.softmax_scale, ctx.causal)
+                                            ctx.dropout_p, ctx.max_s, ctx.softmax_scale, ctx.causal, ctx.alibi_slopes,
+                                            bias_t, dbias)
     if rng_state is not None:
         torch.cuda.set_rng_state(cur_rng_state, dev)
-    return dqkv
+    return dqkv, (bias_grad_in_shape(dbias, ctx.bias_shape, ctx.max_s, ctx.max_s) if dbias is not None else None)
 
 
 class FlashBlocksparseAttnFun(torch.autograd.Function):
-    """apply(qkv, cu_seqlens, blockmask_converted, dropout_p, max_s, softmax_scale, causal) -> context"""
+    """apply(qkv, cu_seqlens, blockmask_converted, dropout_p, max_s, softmax_scale, causal, alibi_slopes, attn_bias)
+    -> context"""
 
     @staticmethod
-    def forward(ctx, qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal):
-        return _fwd_common(ctx, qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal, False)[0]
+    def forward(ctx, qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal, alibi_slopes=None, attn_bias=None):
+        return _fwd_common(ctx, qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal, False, alibi_slopes,
+                           attn_bias)[0]
 
     @staticmethod
     def backward(ctx, dout):
-        return _bwd_common(ctx, dout), None, None, None, None, None, None
+        dqkv, dbias = _bwd_common(ctx, dout)
+        return dqkv, None, None, None, None, None, None, None, dbias
 
 
 class FlashBlocksparseAttnFunWithS(torch.autograd.Function):
     """Same, returning (context, S_dmask, softmax_lse) for tests."""
 
     @staticmethod
-    def forward(ctx, qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal):
+    def forward(ctx, qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal, alibi_slopes=None, attn_bias=None):
         context, S_dmask, softmax_lse = _fwd_common(ctx, qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale,
-                                                    causal, True)
+                                                    causal, True, alibi_slopes, attn_bias)
         ctx.mark_non_differentiable(S_dmask, softmax_lse)
         return context, S_dmask, softmax_lse
 
     @staticmethod
     def backward(ctx, dout, _dS_dmask_ignored, _dsoftmax_sum_ignored):
-        return _bwd_common(ctx, dout), None, None, None, None, None, None
+        dqkv, dbias = _bwd_common(ctx, dout)
+        return dqkv, None, None, None, None, None, None, None, dbias
 
 
 def flash_blocksparse_attn_func(qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale=None,
-                                causal=False, return_attn_probs=False, convert_mask=True):
+                                causal=False, return_attn_probs=False, convert_mask=True, alibi_slopes=None, attn_bias=None):
     """Self-attention on packed qkv (total, 3, nheads, headdim) restricted to the active blocks of `blockmask`
     ((seqlen rounded to 16) / 16 rows by (seqlen rounded to 256) / 256 columns of 0/1, or already converted when
     convert_mask=False).  Query rows whose blocks are all inactive produce zeros.  dropout_p must be 0.0 at
-    evaluation time.  With return_attn_probs=True returns (context, S_dmask, softmax_lse)."""
+    evaluation time.  With return_attn_probs=True returns (context, S_dmask, softmax_lse).
+    alibi_slopes, attn_bias (extensions, as in flash_attn_unpadded_qkvpacked_func): a score bias inside the active
+    blocks; attn_bias is differentiable."""
     func = FlashBlocksparseAttnFun if not return_attn_probs else FlashBlocksparseAttnFunWithS
     if convert_mask:
         blockmask = convert_blockmask(blockmask, causal=causal)
-    return func.apply(qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal)
+    return func.apply(qkv, cu_seqlens, blockmask, dropout_p, max_s, softmax_scale, causal, alibi_slopes, attn_bias)

@@ -72,7 +72,8 @@ typedef struct fa_fwd_args {
   void* stream; /* hipStream_t */
   /* Attention bias (no counterpart in the reference's entry points; its README lists "attention bias (e.g. ALiBi)" as
    * planned, README.md:49-50).  NULL, or a device array of nheads fp32 slopes: softmax_scale * q.k - slope[h] * |i - j|
-   * is what the softmax sees, i and j being the positions of query and key in their sequences.  Not with a blockmask. */
+   * is what the softmax sees, i and j being the positions of query and key in their sequences.  With a blockmask: inside
+   * the active blocks. */
   const float* alibi_slopes;
   /* Dropout keep words (no counterpart in the reference, whose backward kernels draw every keep decision again,
    * fmha_dgrad_kernel_1xN_loop.h:337).  NULL, or 16-byte aligned device memory of keep_words_bytes >=
@@ -86,7 +87,8 @@ typedef struct fa_fwd_args {
    * (keys contiguous; batch and head stride may be 0: one bias for all of them): softmax_scale * q.k + bias[b, h, i, j] is
    * what the softmax sees, i < max_seqlen_q and j < max_seqlen_k being positions inside the sequences.  -inf entries mask.
    * 16-byte aligned, bias_row_stride a multiple of 8 and >= max_seqlen_k; every row is read in 16-byte pieces, i.e. up to the
-   * next multiple of 8 keys past max_seqlen_k (inside the row stride).  Not with a blockmask, not with alibi_slopes. */
+   * next multiple of 8 keys past max_seqlen_k (inside the row stride).  Not with alibi_slopes.  With a blockmask: read inside
+   * the active blocks only. */
   const void* attn_bias;
   int64_t bias_batch_stride, bias_head_stride, bias_row_stride;
   /* Block-sparse only (no counterpart in the reference).  NULL, or a device array of max_seqlen_q_rounded / 16 int32: a

@@ -163,7 +163,7 @@ def test_public_signatures_match_the_reference():
         return [(n, p.default if p.default is not inspect.Parameter.empty else "<req>")
                 for n, p in inspect.signature(f).parameters.items()]
 
-    # the three functions that reach the kernels take the reference's parameters followed by two extensions,
+    # the functions that reach the kernels take the reference's parameters followed by two extensions,
     # alibi_slopes=None and attn_bias=None (attention bias: planned in the reference's README, absent from its API)
     ext = [("alibi_slopes", None), ("attn_bias", None)]
     assert sig(fi.flash_attn_unpadded_qkvpacked_func) == [
@@ -182,7 +182,7 @@ def test_public_signatures_match_the_reference():
         ("softmax_scale", None), ("causal", False), ("return_attn_probs", False)]
     assert sig(bi.flash_blocksparse_attn_func) == [
         ("qkv", "<req>"), ("cu_seqlens", "<req>"), ("blockmask", "<req>"), ("dropout_p", "<req>"), ("max_s", "<req>"),
-        ("softmax_scale", None), ("causal", False), ("return_attn_probs", False), ("convert_mask", True)]
+        ("softmax_scale", None), ("causal", False), ("return_attn_probs", False), ("convert_mask", True)] + ext
     assert [n for n, _ in sig(bp.unpad_input)] == ["hidden_states", "attention_mask"]
     assert [n for n, _ in sig(bp.pad_input)] == ["hidden_states", "indices", "batch", "seqlen"]
     for cls in ("FlashAttnQKVPackedFunc", "FlashAttnKVPackedFunc", "FlashAttnFunc"):
@@ -197,7 +197,8 @@ def test_public_signatures_match_the_reference():
         ("dropout_p", "<req>"), ("softmax_scale", None), ("causal", False)]  # extension: rotary embedding inside the kernels
     assert list(inspect.signature(be.bwd_block).parameters) == [
         "dout", "q", "k", "v", "out", "softmax_lse", "dq", "dk", "dv", "cu_seqlens_q", "cu_seqlens_k", "blockmask",
-        "max_seqlen_q", "max_seqlen_k", "p_dropout", "softmax_scale", "is_causal", "gen", "row_order"]  # fmha_api.cpp:575-594 + extension
+        "max_seqlen_q", "max_seqlen_k", "p_dropout", "softmax_scale", "is_causal", "gen", "row_order", "alibi_slopes",
+        "attn_bias", "dbias"]  # fmha_api.cpp:575-594 + extensions
 
 
 def test_blockmask_row_order_is_a_permutation_that_groups_similar_rows():

@@ -760,8 +760,8 @@ def test_alibi_decode_shape_with_key_split():
 
 def test_alibi_headline_shape_and_errors():
     """ALiBi at the headline shape (all tiles full, no masking code in the way) against the fp32 closed form on the GPU
-    for one (batch, head) pair, slope 0 == no bias bit for bit, and the refusals: slopes of the wrong shape / dtype /
-    device, slopes together with a block layout."""
+    for one (batch, head) pair, slope 0 == no bias bit for bit, the refusals (slopes of the wrong shape / dtype / device),
+    and the same slopes under a block layout that lists every block."""
     from flash_attn import flash_attn_interface as fi
     from flash_attn.flash_blocksparse_attn_interface import convert_blockmask
     from flash_attn import flash_attn_gfx950 as be
@@ -788,11 +788,12 @@ def test_alibi_headline_shape_and_errors():
     for bad in (slopes[:3], slopes.double(), slopes.cpu(), slopes[None]):
         with pytest.raises(RuntimeError):
             fi.flash_attn_unpadded_qkvpacked_func(qkv.detach(), cu, N, 0.0, alibi_slopes=bad)
+    # with a block layout that lists every block the slopes give what the dense kernels give (other tile shapes: within rounding)
     sq_r, sk_r = be.round_seqlens(D, N, N, True)
-    bm = convert_blockmask(torch.ones(sq_r // 16, sk_r // 256, device="cuda"), causal=False)
+    bm = convert_blockmask(torch.ones(sq_r // 16, sk_r // 256, device="cuda"), causal=True)
     q3 = qkv.detach()
-    with pytest.raises(RuntimeError):
-        be._fwd_impl(q3[:, 0], q3[:, 1], q3[:, 2], cu, cu, bm, N, N, 0.0, D ** -0.5, False, False, False, None, slopes)
+    o_sparse = be.fwd_block(q3[:, 0], q3[:, 1], q3[:, 2], cu, cu, bm, N, N, 0.0, D ** -0.5, True, False, alibi_slopes=slopes)[0]
+    assert (o_sparse.float() - out.detach().float()).abs().max() < 1e-3
 
 
 # ------------------------------------------------------------------------------------------------
@@ -1084,6 +1085,63 @@ def test_blocksparse_random_layouts_sweep():
                               layout=layout.numpy(), dout=do.cuda())
         ours = {"out": ctx.detach(), "dq": qkv.grad[:, 0], "dk": qkv.grad[:, 1], "dv": qkv.grad[:, 2]}
         check_against_oracle(ours, ref, half, dtype, what=what)
+
+
+def test_blocksparse_with_score_bias_sweep():
+    """Twelve seeded random block-sparse cases with a score bias inside the active blocks: ALiBi slopes or a bias tensor
+    (per (batch, head), shared over the batch, over everything; with -inf entries), every head dim, both dtypes, causal or
+    not (causal: no row order, the packed tiles of the backward straddle the diagonal), ragged lengths, dropout - out, dq,
+    dk, dv and the bias gradient against the oracle's closed form with the layout, the bias and the drawn mask."""
+    from flash_attn.flash_blocksparse_attn_interface import flash_blocksparse_attn_func
+    from flash_attn import flash_attn_gfx950 as be
+    rng = np.random.default_rng(77)
+    for case in range(12):
+        D = int(rng.choice([16, 32, 64, 128]))
+        dtype = torch.float16 if rng.integers(2) else torch.bfloat16
+        B, H = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        N = int(rng.choice([100, 300, 520, 1100]))
+        lens = [N] + [int(x) for x in rng.integers(max(1, N // 3), N + 1, B - 1)]
+        dens = float(rng.choice([0.1, 0.3, 0.6]))
+        p = float(rng.choice([0.0, 0.0, 0.2]))
+        causal = bool(rng.integers(2))
+        kind = ("alibi", "tensor", "tensor")[int(rng.integers(3))]
+        sq_r, sk_r = be.round_seqlens(D, N, N, True)
+        layout = torch.rand(sq_r // 16, sk_r // 256, generator=torch.Generator().manual_seed(100 + case)) < dens
+        layout |= (torch.arange(sq_r // 16)[:, None] // 16) == torch.arange(sk_r // 256)[None, :]  # the diagonal band
+        slopes = bias = None
+        if kind == "alibi":
+            slopes = _alibi_slopes(H) * 0.5
+        else:
+            bshape = ((B, H), (1, H), (1, 1))[int(rng.integers(3))] + (N, N if rng.integers(2) else (N + 7) // 8 * 8)
+            bias = _random_bias(rng, bshape, dtype, minus_inf=float(rng.choice([0.0, 0.15])))
+        what = "case %d: D=%d %s B=%d H=%d lens=%s density %.1f p=%.1f causal=%s %s%s" % (
+            case, D, dtype, B, H, lens, dens, p, causal, kind, tuple(bias.shape) if bias is not None else "")
+        print(what, flush=True)
+        q, k, v, do = _inputs(lens, lens, H, D, dtype, 5000 + case)
+        cu = _cu(lens, "cpu")
+        qkv = torch.stack([q, k, v], 1).cuda().requires_grad_()
+        bias_g = bias.cuda().requires_grad_() if bias is not None else None
+        torch.manual_seed(case)
+        seed, offset = _gen_state()
+        ctx = flash_blocksparse_attn_func(qkv, cu.cuda(), layout.cuda(), p, N, causal=causal,
+                                          alibi_slopes=slopes.cuda() if slopes is not None else None, attn_bias=bias_g)
+        ctx.backward(do.cuda())
+        torch.cuda.synchronize()
+        masks = None
+        if p > 0:
+            masks = [torch.tensor(np.stack([orc.dropout_keep_mask(seed, offset, b * H + h, L, L, p) for h in range(H)]))
+                     for b, L in enumerate(lens)]
+        ref = orc.varlen_attention(q, k, v, cu, cu, None, causal, p_dropout=p, keep_mask=masks, layout=layout.numpy(), dout=do,
+                                   alibi_slopes=slopes, attn_bias=bias)
+        half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu.tolist(), cu.tolist(), D ** -0.5, causal, masks, p,
+                              layout=layout.numpy(), dout=do.cuda(), alibi_slopes=slopes,
+                              attn_bias=bias.cuda() if bias is not None else None)
+        ours = {"out": ctx.detach(), "dq": qkv.grad[:, 0], "dk": qkv.grad[:, 1], "dv": qkv.grad[:, 2]}
+        names = ("out", "dq", "dk", "dv")
+        if bias is not None:
+            ours["dbias"] = bias_g.grad
+            names += ("dbias",)
+        check_against_oracle(ours, ref, half, dtype, names=names, what=what)
 
 
 @pytest.mark.parametrize("D,N,dtype", [(64, 1280, torch.float16), (32, 300, torch.bfloat16), (128, 700, torch.float16)])
