@@ -1087,13 +1087,50 @@ def test_blocksparse_random_layouts_sweep():
         check_against_oracle(ours, ref, half, dtype, what=what)
 
 
+def _blocksparse_bias_case(case, D, dtype, H, lens, dens, p, causal, slopes, bias, what):
+    """one block-sparse case with ALiBi slopes or a bias tensor through flash_blocksparse_attn_func, against the oracle"""
+    from flash_attn.flash_blocksparse_attn_interface import flash_blocksparse_attn_func
+    from flash_attn import flash_attn_gfx950 as be
+    N = max(lens)
+    sq_r, sk_r = be.round_seqlens(D, N, N, True)
+    layout = torch.rand(sq_r // 16, sk_r // 256, generator=torch.Generator().manual_seed(100 + case)) < dens
+    layout |= (torch.arange(sq_r // 16)[:, None] // 16) == torch.arange(sk_r // 256)[None, :]  # the diagonal band
+    print(what, flush=True)
+    q, k, v, do = _inputs(lens, lens, H, D, dtype, 5000 + case)
+    cu = _cu(lens, "cpu")
+    qkv = torch.stack([q, k, v], 1).cuda().requires_grad_()
+    bias_g = bias.cuda().requires_grad_() if bias is not None else None
+    torch.manual_seed(case)
+    seed, offset = _gen_state()
+    ctx = flash_blocksparse_attn_func(qkv, cu.cuda(), layout.cuda(), p, N, causal=causal,
+                                      alibi_slopes=slopes.cuda() if slopes is not None else None, attn_bias=bias_g)
+    ctx.backward(do.cuda())
+    torch.cuda.synchronize()
+    masks = None
+    if p > 0:
+        masks = [torch.tensor(np.stack([orc.dropout_keep_mask(seed, offset, b * H + h, L, L, p) for h in range(H)]))
+                 for b, L in enumerate(lens)]
+    ref = orc.varlen_attention(q, k, v, cu, cu, None, causal, p_dropout=p, keep_mask=masks, layout=layout.numpy(), dout=do,
+                               alibi_slopes=slopes, attn_bias=bias)
+    half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu.tolist(), cu.tolist(), D ** -0.5, causal, masks, p,
+                          layout=layout.numpy(), dout=do.cuda(), alibi_slopes=slopes,
+                          attn_bias=bias.cuda() if bias is not None else None)
+    ours = {"out": ctx.detach(), "dq": qkv.grad[:, 0], "dk": qkv.grad[:, 1], "dv": qkv.grad[:, 2]}
+    names = ("out", "dq", "dk", "dv")
+    if bias is not None:
+        ours["dbias"] = bias_g.grad
+        names += ("dbias",)
+        # blocks the layout leaves out take no gradient
+        dead = ~orc.expand_block_layout(layout.numpy(), N, N)
+        assert bool((bias_g.grad[..., :N, :N].cpu()[..., dead] == 0).all()), what
+    check_against_oracle(ours, ref, half, dtype, names=names, what=what)
+
+
 def test_blocksparse_with_score_bias_sweep():
     """Twelve seeded random block-sparse cases with a score bias inside the active blocks: ALiBi slopes or a bias tensor
     (per (batch, head), shared over the batch, over everything; with -inf entries), every head dim, both dtypes, causal or
     not (causal: no row order, the packed tiles of the backward straddle the diagonal), ragged lengths, dropout - out, dq,
     dk, dv and the bias gradient against the oracle's closed form with the layout, the bias and the drawn mask."""
-    from flash_attn.flash_blocksparse_attn_interface import flash_blocksparse_attn_func
-    from flash_attn import flash_attn_gfx950 as be
     rng = np.random.default_rng(77)
     for case in range(12):
         D = int(rng.choice([16, 32, 64, 128]))
@@ -1105,9 +1142,6 @@ def test_blocksparse_with_score_bias_sweep():
         p = float(rng.choice([0.0, 0.0, 0.2]))
         causal = bool(rng.integers(2))
         kind = ("alibi", "tensor", "tensor")[int(rng.integers(3))]
-        sq_r, sk_r = be.round_seqlens(D, N, N, True)
-        layout = torch.rand(sq_r // 16, sk_r // 256, generator=torch.Generator().manual_seed(100 + case)) < dens
-        layout |= (torch.arange(sq_r // 16)[:, None] // 16) == torch.arange(sk_r // 256)[None, :]  # the diagonal band
         slopes = bias = None
         if kind == "alibi":
             slopes = _alibi_slopes(H) * 0.5
@@ -1116,32 +1150,24 @@ def test_blocksparse_with_score_bias_sweep():
             bias = _random_bias(rng, bshape, dtype, minus_inf=float(rng.choice([0.0, 0.15])))
         what = "case %d: D=%d %s B=%d H=%d lens=%s density %.1f p=%.1f causal=%s %s%s" % (
             case, D, dtype, B, H, lens, dens, p, causal, kind, tuple(bias.shape) if bias is not None else "")
-        print(what, flush=True)
-        q, k, v, do = _inputs(lens, lens, H, D, dtype, 5000 + case)
-        cu = _cu(lens, "cpu")
-        qkv = torch.stack([q, k, v], 1).cuda().requires_grad_()
-        bias_g = bias.cuda().requires_grad_() if bias is not None else None
-        torch.manual_seed(case)
-        seed, offset = _gen_state()
-        ctx = flash_blocksparse_attn_func(qkv, cu.cuda(), layout.cuda(), p, N, causal=causal,
-                                          alibi_slopes=slopes.cuda() if slopes is not None else None, attn_bias=bias_g)
-        ctx.backward(do.cuda())
-        torch.cuda.synchronize()
-        masks = None
-        if p > 0:
-            masks = [torch.tensor(np.stack([orc.dropout_keep_mask(seed, offset, b * H + h, L, L, p) for h in range(H)]))
-                     for b, L in enumerate(lens)]
-        ref = orc.varlen_attention(q, k, v, cu, cu, None, causal, p_dropout=p, keep_mask=masks, layout=layout.numpy(), dout=do,
-                                   alibi_slopes=slopes, attn_bias=bias)
-        half = half_attention(q.cuda(), k.cuda(), v.cuda(), cu.tolist(), cu.tolist(), D ** -0.5, causal, masks, p,
-                              layout=layout.numpy(), dout=do.cuda(), alibi_slopes=slopes,
-                              attn_bias=bias.cuda() if bias is not None else None)
-        ours = {"out": ctx.detach(), "dq": qkv.grad[:, 0], "dk": qkv.grad[:, 1], "dv": qkv.grad[:, 2]}
-        names = ("out", "dq", "dk", "dv")
-        if bias is not None:
-            ours["dbias"] = bias_g.grad
-            names += ("dbias",)
-        check_against_oracle(ours, ref, half, dtype, names=names, what=what)
+        _blocksparse_bias_case(case, D, dtype, H, lens, dens, p, causal, slopes, bias, what)
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("kind", ["alibi", "tensor"])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("p", [0.0, 0.2])
+def test_blocksparse_with_score_bias_variants(D, kind, causal, p):
+    """every block-sparse kernel variant with a score bias at the two large head dims: (ALiBi, tensor) x (causal or not) x
+    (dropout or not), ragged batch of two, a bias shared over the batch (its gradient is the sum of both entries')"""
+    H, lens, dtype = 2, [520, 300], torch.float16
+    slopes = bias = None
+    if kind == "alibi":
+        slopes = _alibi_slopes(H) * 0.5
+    else:
+        bias = _random_bias(np.random.default_rng(D + 3), (1, H, 520, 520), dtype)
+    what = "variant D=%d %s causal=%s p=%.1f" % (D, kind, causal, p)
+    _blocksparse_bias_case(D + 2 * causal + (p > 0), D, dtype, H, lens, 0.3, p, causal, slopes, bias, what)
 
 
 @pytest.mark.parametrize("D,N,dtype", [(64, 1280, torch.float16), (32, 300, torch.bfloat16), (128, 700, torch.float16)])
