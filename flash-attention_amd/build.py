@@ -26,7 +26,7 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
     "-Wno-inline-asm",  # fa_stage.h sets M0 inside an asm statement on purpose (direct-to-LDS loads need it)
-] + os.environ.get("FA_EXTRA_HIPCC_FLAGS", "").split()  # e.g. -DFA_FUSED_EXPERIMENTS (measurement variants of a kernel)
+] + os.environ.get("FA_EXTRA_HIPCC_FLAGS", "").split()  # measurement variants of a kernel: -DFA_FUSED_EXPERIMENTS, -DFA_ABLATE_FWD=<bits>, -DFA_ABLATE_DKDV=<bits>
 
 
 def sources():

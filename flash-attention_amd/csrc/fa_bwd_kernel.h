@@ -29,6 +29,13 @@
 #include "fa_params.h"
 #include "fa_stage.h"
 
+// Measurement variants of the dK/dV kernel (-DFA_ABLATE_DKDV=<bits>, as FA_ABLATE_FWD in fa_fwd_kernel.h; results are wrong,
+// never a product build).  1: no wait for the staged tile and no workgroup barrier; 2: a multiplication in place of every
+// exponential; 4: no dV and dK products; 8: no S and dP products.
+#ifndef FA_ABLATE_DKDV
+#define FA_ABLATE_DKDV 0
+#endif
+
 namespace fa {
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -328,7 +335,7 @@ FA_DEVICE void fa_bwd_dkdv_body(const BwdParams& p, const int block, unsigned ch
   if (kTensorBias && more) load_bias(mt * BM, tc.rb);
   while (more) {
     const int m0 = mt * BM;
-    wait_vmem();  // this thread's share of the tile has arrived (LDS) / is in statpre
+    if constexpr ((FA_ABLATE_DKDV & 1) == 0) wait_vmem();  // this thread's share of the tile has arrived (LDS) / is in statpre
     float* const lse_l = reinterpret_cast<float*>(lds_raw + Cfg::kOffStat + buf * Cfg::kStatBytes);
     float* const dk_l = lse_l + BM;
     if constexpr (kOwnD) {
@@ -339,7 +346,7 @@ FA_DEVICE void fa_bwd_dkdv_body(const BwdParams& p, const int block, unsigned ch
       if (tid < 2 * BM) lse_l[tid] = stat_value();
     }
     const uint32_t kwcur = kwpre;
-    __syncthreads();  // the tile is complete, and nobody still reads the other buffer
+    if constexpr ((FA_ABLATE_DKDV & 1) == 0) __syncthreads();  // the tile is complete, and nobody still reads the other buffer
     if (kSparse) {
       more = next_tile(tn);
       if (more) stage_blocks(tn, buf ^ 1);
@@ -408,11 +415,16 @@ FA_DEVICE void fa_bwd_dkdv_body(const BwdParams& p, const int block, unsigned ch
       }
       vec8 aq[D / 16], ad[D / 16];
       load_rows(qb, aq, ad);
+      if constexpr ((FA_ABLATE_DKDV & 8) == 0) {
 #pragma unroll
-      for (int ks = 0; ks < D / 16; ks++) s = E::mfma32(aq[ks], kreg[ks], s);
+        for (int ks = 0; ks < D / 16; ks++) s = E::mfma32(aq[ks], kreg[ks], s);
 #pragma unroll
-      for (int ks = 0; ks < D / 16; ks++)
-        dp = E::mfma32(ad[ks], kVLds ? *reinterpret_cast<const vec8*>(Vfrag + ks * 16) : vreg[ks], dp);
+        for (int ks = 0; ks < D / 16; ks++)
+          dp = E::mfma32(ad[ks], kVLds ? *reinterpret_cast<const vec8*>(Vfrag + ks * 16) : vreg[ks], dp);
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < D / 16; ks++) { s[ks] += (float)aq[ks][0] * (float)kreg[ks][0]; dp[ks] += (float)ad[ks][0]; }
+      }
       // ---- P and dS'
       KeepFields keep;
       if (kDropout) {  // this lane draws micro-block 2 (key % 4) + hf of the slab's eight (four query rows each)
@@ -454,7 +466,7 @@ FA_DEVICE void fa_bwd_dkdv_body(const BwdParams& p, const int block, unsigned ch
           float e = -lse4[i];
           if (kAlibi) e = __builtin_fmaf(__builtin_fabsf((j < 2 ? dbase : dbase_hi) - (float)(8 * j + i)), -sl2, -lse4[i]);
           if (kTensorBias) e = __builtin_fmaf((float)braw[r], kLog2e, -lse4[i]);
-          const float pe = fast_exp2(__builtin_fmaf(s[r], cs, e));
+          const float pe = (FA_ABLATE_DKDV & 2) ? __builtin_fmaf(s[r], cs, e) * 1e-3f : fast_exp2(__builtin_fmaf(s[r], cs, e));
           float dpe = dp[r];  // dP - Dk
           float pm = pe;
           if (kDropout && !keep.keep_col(r, p.keep_thr)) { dpe = nd4[i]; pm = 0.f; }  // dropped: M o dP = 0
@@ -483,8 +495,12 @@ FA_DEVICE void fa_bwd_dkdv_body(const BwdParams& p, const int block, unsigned ch
         load_tr(qb, t, avs, aqs);
 #pragma unroll
         for (int db = 0; db < DV / 32; db++) {
-          acc_dv[db] = E::mfma32(bitcast<vec8>(avs[db]), pb, acc_dv[db]);
-          acc_dk[db] = E::mfma32(bitcast<vec8>(aqs[db]), db8, acc_dk[db]);
+          if constexpr ((FA_ABLATE_DKDV & 4) == 0) {
+            acc_dv[db] = E::mfma32(bitcast<vec8>(avs[db]), pb, acc_dv[db]);
+            acc_dk[db] = E::mfma32(bitcast<vec8>(aqs[db]), db8, acc_dk[db]);
+          } else {
+            asm volatile("" ::"v"(avs[db]), "v"(aqs[db]), "v"(pb), "v"(db8));
+          }
         }
       }
     }

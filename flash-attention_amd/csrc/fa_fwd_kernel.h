@@ -18,6 +18,14 @@
 #include "fa_params.h"
 #include "fa_stage.h"
 
+// Measurement variants (-DFA_ABLATE_FWD=<bits> through FA_EXTRA_HIPCC_FLAGS; results are wrong, never a product build):
+// what one part of the main loop costs is read off the kernel's time without it.  1: no wait for the staged tile and no
+// workgroup barrier; 2: a multiplication in place of every exponential; 4: no P V products; 8: no Q K^T products; 16: the K
+// and V fragments not read from LDS (registers stand in); 32: no row sums of P and no test of them.
+#ifndef FA_ABLATE_FWD
+#define FA_ABLATE_FWD 0
+#endif
+
 namespace fa {
 
 // KS (key split) = 1: the workgroup's four waves own 32 of its 128 query rows each and every wave sees all keys of a tile.
@@ -254,9 +262,11 @@ __global__ void __launch_bounds__(256, ((!kDropout || KS == 2) && kBias == 0 && 
     // ties the last MFMA's result to the registers the epilogue reads and copies all of O back on every trip.
 #pragma unroll
     for (int i = 0; i < DV / 32; i++) asm volatile("" : "+v"(o_acc[i]));
-    wait_vmem();                         // this wave's share of tile `it` is in LDS
-    flush_keep_words();
-    __syncthreads();                     // so is everyone else's, and nobody still reads the other buffer
+    if constexpr ((FA_ABLATE_FWD & 1) == 0) {
+      wait_vmem();                       // this wave's share of tile `it` is in LDS
+      flush_keep_words();
+      __syncthreads();                   // so is everyone else's, and nobody still reads the other buffer
+    }
     const int it_next = next_active(it + 1);
     if (it_next < ntiles) stage(it_next, buf ^ 1);
     if (kTensorBias) {  // (the wave's own reads of the last tile's values are behind it: LDS operations of a wave stay in order)
@@ -299,8 +309,9 @@ __global__ void __launch_bounds__(256, ((!kDropout || KS == 2) && kBias == 0 && 
           for (int r = 0; r < 16; r++) s[kb][r] = 0.f;
 #pragma unroll
           for (int ks = 0; ks < D / 16; ks++) {
-            vec8 a = *reinterpret_cast<const vec8*>(Ks + (kb0 + kb) * 32 * D + koff[ks]);
-            s[kb] = E::mfma32(a, qreg[ks], s[kb]);
+            vec8 a = (FA_ABLATE_FWD & 16) ? qreg[(ks + 1) % (D / 16)] : *reinterpret_cast<const vec8*>(Ks + (kb0 + kb) * 32 * D + koff[ks]);
+            if constexpr ((FA_ABLATE_FWD & 8) == 0) s[kb] = E::mfma32(a, qreg[ks], s[kb]);
+            else s[kb][ks] = (float)a[ks] * (float)qreg[ks][0];
           }
         }
         // mask: only tiles that straddle the key length or the diagonal.  (An inactive row block inside an active tile is
@@ -356,7 +367,8 @@ __global__ void __launch_bounds__(256, ((!kDropout || KS == 2) && kBias == 0 && 
         for (int kb = 0; kb < KBW; kb++)
 #pragma unroll
           for (int r = 0; r < 16; r++) {
-            const float pe = fast_exp2(kBias != 0 ? s[kb][r] - mc : __builtin_fmaf(s[kb][r], cs, -mc));
+            const float pe_arg = kBias != 0 ? s[kb][r] - mc : __builtin_fmaf(s[kb][r], cs, -mc);
+            const float pe = (FA_ABLATE_FWD & 2) ? pe_arg * 1e-3f : fast_exp2(pe_arg);
             s[kb][r] = pe;
             if (kDropout) lt += pe;
           }
@@ -395,7 +407,7 @@ __global__ void __launch_bounds__(256, ((!kDropout || KS == 2) && kBias == 0 && 
 #pragma unroll
             for (int i = 0; i < 8; i++) pf[i] = s[kb][8 * t + i];
             pb[kb][t] = cvt8<T>(pf);
-            if (!kDropout) lt = sum8_acc(pb[kb][t], lt);
+            if (!kDropout && (FA_ABLATE_FWD & 32) == 0) lt = sum8_acc(pb[kb][t], lt);
           }
       };
       // ---- online softmax (fmha_fprop_kernel_1xN.h:408-454,560-611 restated for a register-resident row).
@@ -409,7 +421,7 @@ __global__ void __launch_bounds__(256, ((!kDropout || KS == 2) && kBias == 0 && 
       bool redo = __any(m_i == -INFINITY && (!kSparse || row_on));
       if (!redo) {
         probabilities();
-        redo = __any(!(lt <= kRescaleLimit));  // also catches inf and NaN
+        if constexpr ((FA_ABLATE_FWD & 32) == 0) redo = __any(!(lt <= kRescaleLimit));  // also catches inf and NaN
         if (__builtin_expect(redo, 0)) scores();
       }
       if (__builtin_expect(redo, 0)) {
@@ -439,10 +451,16 @@ __global__ void __launch_bounds__(256, ((!kDropout || KS == 2) && kBias == 0 && 
 #pragma unroll
           for (int db = 0; db < DV / 32; db++) {
             const T* vp = Vs + ((kb0 + kb) * 32 + 16 * t) * D + voff[db];
-            u32x2 lo = lds_read_tr16(vp);
-            u32x2 hi = lds_read_tr16(vp + 8 * D);
-            u32x4 av = {lo[0], lo[1], hi[0], hi[1]};
-            o_acc[db] = E::mfma32(bitcast<vec8>(av), pb[kb][t], o_acc[db]);
+            u32x4 av;
+            if constexpr ((FA_ABLATE_FWD & 16) == 0) {
+              u32x2 lo = lds_read_tr16(vp);
+              u32x2 hi = lds_read_tr16(vp + 8 * D);
+              av = u32x4{lo[0], lo[1], hi[0], hi[1]};
+            } else {
+              av = bitcast<u32x4>(qreg[db]);
+            }
+            if constexpr ((FA_ABLATE_FWD & 4) == 0) o_acc[db] = E::mfma32(bitcast<vec8>(av), pb[kb][t], o_acc[db]);
+            else asm volatile("" ::"v"(av), "v"(pb[kb][t]));
           }
         }
       }
